@@ -1,0 +1,183 @@
+"""Seeded synthetic lc0 networks (random-init weights of a given architecture).
+
+Produces nested dicts for `netproto.write_pb_gz`; the files are loadable by a
+real lc0 (FLOAT32 layers, legacy top-level head fields so that
+src/neural/loader.cc:146-153 does not switch the net to PE_DENSE).
+
+Tensor shapes follow src/neural/network_legacy.h and the consumers in
+src/neural/backends/blas/network_blas.cc: dense weights are [out][in]
+row-major, convolution filters [out][in][3][3].
+"""
+import os
+
+import numpy as np
+
+from . import netproto
+
+# pblczero.NetworkFormat enums (proto/net.proto:275-366)
+INPUT_CLASSICAL_112_PLANE = 1
+OUTPUT_WDL = 2
+NETWORK_SE_WITH_HEADFORMAT = 4
+NETWORK_ATTENTIONBODY_WITH_HEADFORMAT = 6
+POLICY_CLASSICAL, POLICY_CONVOLUTION, POLICY_ATTENTION = 1, 2, 3
+VALUE_WDL = 2
+MOVES_LEFT_NONE, MOVES_LEFT_V1 = 0, 1
+DEFAULT_ACTIVATION_RELU, DEFAULT_ACTIVATION_MISH = 0, 1
+ACTIVATION_DEFAULT, ACTIVATION_SWISH = 0, 7
+INPUT_EMBEDDING_PE_MAP = 1
+
+
+class _Gen:
+    def __init__(self, seed):
+        self.rng = np.random.default_rng(seed)
+
+    def normal(self, shape, std):
+        return (self.rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+
+
+def se_resnet(filters, blocks, se_channels, seed, policy_channels=32, value_channels=32,
+              value_fc=128, bias_std=0.02, moves_left=False, conv_policy=False):
+    """Classical SE-ResNet: weights N(0, 1/fan_in) (std = fan_in**-0.5)."""
+    g = _Gen(seed)
+
+    def conv(cout, cin, k):
+        fan_in = cin * k * k
+        return {"weights": g.normal((cout, cin, k, k), fan_in ** -0.5),
+                "biases": g.normal((cout,), bias_std)}
+
+    def fc(cout, cin):
+        return g.normal((cout, cin), cin ** -0.5), g.normal((cout,), bias_std)
+
+    w = {"input": conv(filters, 112, 3), "residual": []}
+    for _ in range(blocks):
+        blk = {"conv1": conv(filters, filters, 3), "conv2": conv(filters, filters, 3)}
+        if se_channels:
+            w1, b1 = fc(se_channels, filters)
+            w2, b2 = fc(2 * filters, se_channels)
+            blk["se"] = {"w1": w1, "b1": b1, "w2": w2, "b2": b2}
+        w["residual"].append(blk)
+    if conv_policy:
+        w["policy1"] = conv(filters, filters, 3)
+        w["policy"] = conv(80, filters, 3)
+    else:
+        w["policy"] = conv(policy_channels, filters, 1)
+        w["ip_pol_w"], w["ip_pol_b"] = fc(1858, policy_channels * 64)
+    w["value"] = conv(value_channels, filters, 1)
+    w["ip1_val_w"], w["ip1_val_b"] = fc(value_fc, value_channels * 64)
+    w["ip2_val_w"], w["ip2_val_b"] = fc(3, value_fc)
+    if moves_left:
+        w["moves_left"] = conv(8, filters, 1)
+        w["ip1_mov_w"], w["ip1_mov_b"] = fc(value_fc, 8 * 64)
+        w["ip2_mov_w"], w["ip2_mov_b"] = fc(1, value_fc)
+    nf = {"input": INPUT_CLASSICAL_112_PLANE, "output": OUTPUT_WDL,
+          "network": NETWORK_SE_WITH_HEADFORMAT,
+          "policy": POLICY_CONVOLUTION if conv_policy else POLICY_CLASSICAL,
+          "value": VALUE_WDL,
+          "moves_left": MOVES_LEFT_V1 if moves_left else MOVES_LEFT_NONE,
+          "default_activation": DEFAULT_ACTIVATION_RELU}
+    return {"format": {"weights_encoding": netproto.LINEAR16, "network_format": nf}, "weights": w}
+
+
+def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_std=0.02,
+                   policy_d=None, value_channels=32, value_fc=128, mlh_channels=32, mlh_fc=128,
+                   perturb_ln=False):
+    """Attention-body net (PE_MAP embedding, attention policy, WDL, MLH).
+
+    smolgen = (hidden_channels, hidden_sz, gen_sz) or None. Weights N(0, std),
+    LayerNorm gamma=1 / beta=0 unless perturb_ln (tests).
+    """
+    g = _Gen(seed)
+    d_model = emb
+    policy_d = policy_d or emb
+
+    def fc(cout, cin, bias=True):
+        w = g.normal((cout, cin), std)
+        return (w, g.normal((cout,), bias_std)) if bias else w
+
+    def ln(n):
+        if perturb_ln:
+            return 1.0 + g.normal((n,), 0.1), g.normal((n,), 0.1)
+        return np.ones(n, np.float32), np.zeros(n, np.float32)
+
+    w = {}
+    w["ip_emb_w"], w["ip_emb_b"] = fc(emb, 112 + 64)
+    w["encoder"] = []
+    for _ in range(layers):
+        mha = {}
+        mha["q_w"], mha["q_b"] = fc(d_model, emb)
+        mha["k_w"], mha["k_b"] = fc(d_model, emb)
+        mha["v_w"], mha["v_b"] = fc(d_model, emb)
+        mha["dense_w"], mha["dense_b"] = fc(emb, d_model)
+        if smolgen:
+            hc, hs, gsz = smolgen
+            sg = {"compress": fc(hc, emb, bias=False)}
+            sg["dense1_w"], sg["dense1_b"] = fc(hs, 64 * hc)
+            sg["ln1_gammas"], sg["ln1_betas"] = ln(hs)
+            sg["dense2_w"], sg["dense2_b"] = fc(heads * gsz, hs)
+            sg["ln2_gammas"], sg["ln2_betas"] = ln(heads * gsz)
+            mha["smolgen"] = sg
+        layer = {"mha": mha}
+        layer["ln1_gammas"], layer["ln1_betas"] = ln(emb)
+        ffn = {}
+        ffn["dense1_w"], ffn["dense1_b"] = fc(dff, emb)
+        ffn["dense2_w"], ffn["dense2_b"] = fc(emb, dff)
+        layer["ffn"] = ffn
+        layer["ln2_gammas"], layer["ln2_betas"] = ln(emb)
+        w["encoder"].append(layer)
+    w["headcount"] = heads
+    w["ip_pol_w"], w["ip_pol_b"] = fc(policy_d, emb)
+    w["ip2_pol_w"], w["ip2_pol_b"] = fc(policy_d, policy_d)
+    w["ip3_pol_w"], w["ip3_pol_b"] = fc(policy_d, policy_d)
+    w["ip4_pol_w"] = fc(4, policy_d, bias=False)
+    w["ip_val_w"], w["ip_val_b"] = fc(value_channels, emb)
+    w["ip1_val_w"], w["ip1_val_b"] = fc(value_fc, 64 * value_channels)
+    w["ip2_val_w"], w["ip2_val_b"] = fc(3, value_fc)
+    w["ip_mov_w"], w["ip_mov_b"] = fc(mlh_channels, emb)
+    w["ip1_mov_w"], w["ip1_mov_b"] = fc(mlh_fc, 64 * mlh_channels)
+    w["ip2_mov_w"], w["ip2_mov_b"] = fc(1, mlh_fc)
+    if smolgen:
+        w["smolgen_w"] = fc(64 * 64, smolgen[2], bias=False)
+    nf = {"input": INPUT_CLASSICAL_112_PLANE, "output": OUTPUT_WDL,
+          "network": NETWORK_ATTENTIONBODY_WITH_HEADFORMAT, "policy": POLICY_ATTENTION,
+          "value": VALUE_WDL, "moves_left": MOVES_LEFT_V1,
+          "default_activation": DEFAULT_ACTIVATION_MISH,
+          "smolgen_activation": ACTIVATION_SWISH if smolgen else ACTIVATION_DEFAULT,
+          "ffn_activation": ACTIVATION_DEFAULT,
+          "input_embedding": INPUT_EMBEDDING_PE_MAP}
+    return {"format": {"weights_encoding": netproto.LINEAR16, "network_format": nf}, "weights": w}
+
+
+# The benchmark configurations (name -> builder). Seeds are part of the spec.
+CONFIGS = {
+    # 6 blocks x 64 filters SE-ResNet, SE ratio 4, classical policy, WDL.
+    "c0_resnet_6x64": lambda: se_resnet(64, 6, 16, seed=1000),
+    # 10-layer d=256 attention body, 8 heads, dff 1024, no smolgen.
+    "c1_attn_10x256": lambda: attention_body(256, 10, 8, 1024, seed=1001),
+    # BT4 shape: 15 layers, d=1024, 32 heads, dff 1536, smolgen 32/256/256.
+    "c2_bt4_15x1024": lambda: attention_body(1024, 15, 32, 1536, seed=1002, smolgen=(32, 256, 256)),
+    # 20 blocks x 256 filters SE-ResNet, SE ratio 4.
+    "c3_resnet_20x256": lambda: se_resnet(256, 20, 64, seed=1003),
+    # tiny nets for fast parity tests
+    "tiny_resnet": lambda: se_resnet(32, 2, 8, seed=2000, moves_left=True),
+    "tiny_attn": lambda: attention_body(64, 2, 2, 96, seed=2001, smolgen=(8, 32, 32), perturb_ln=True),
+    "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 4, 128, seed=2002, perturb_ln=True),
+}
+
+
+def write_config(name, path):
+    """Generates config `name` into `path` (a .pb.gz); returns the path."""
+    net = CONFIGS[name]()
+    netproto.write_pb_gz(path, net)
+    return path
+
+
+def cached_config(name, cache_dir=None):
+    """Path of the generated file for `name`, generating it on first use."""
+    cache_dir = cache_dir or os.environ.get("LC0MI_NET_CACHE", "/tmp/lc0mi_nets")
+    os.makedirs(cache_dir, exist_ok=True)
+    path = os.path.join(cache_dir, name + ".pb.gz")
+    if not os.path.exists(path):
+        tmp = path + ".tmp%d" % os.getpid()
+        write_config(name, tmp)
+        os.replace(tmp, path)
+    return path
