@@ -1,0 +1,145 @@
+"""Benchmark of the NN-evaluation hot path on one MI355X.
+
+Metric (BASELINE.json): NN evals/sec at batch 256 on the BT4-shape fp16 net,
+with the dominant kernel's fraction of the MFMA roofline and the CPU oracle's
+evals/sec on the same host next to it. A "step" is one device pass over one
+batch of 256 seeded random-playout positions already resident in HBM.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--batch B]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
+
+WORKLOADS = {
+    "c2_bt4_15x1024": dict(batch=256, desc="BT4-shape attention body: 15 layers, d=1024, 32 heads, dff 1536, "
+                                           "smolgen 32/256/256, fp16 with fp32 accumulation"),
+    "c1_attn_10x256": dict(batch=64, desc="attention body: 10 layers, d=256, 8 heads, dff 1024, fp16"),
+    "tiny_attn": dict(batch=64, desc="tiny smolgen attention body (test net)"),
+}
+
+
+def cpu_baseline(path, masks, values, sample, seconds_budget=25.0):
+    """Oracle (numpy/BLAS restatement of the blas backend) timed on this host."""
+    from oracle import netread as nr
+    from oracle import nn as onn
+    bn = onn.BlasNetwork(nr.load(path))
+    m, v = masks[:sample], values[:sample]
+    bn.forward(m[:2], v[:2])  # warm-up
+    times = []
+    t_end = time.time() + seconds_budget
+    while len(times) < 3 or (time.time() < t_end and len(times) < 10):
+        t0 = time.perf_counter()
+        bn.forward(m, v)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": sample / med, "unit": "evals/s", "cores": cores, "kind": "port",
+            "sample": "%d positions per pass, %d timed passes, median; numpy float32 + its bundled BLAS sgemm"
+                      % (sample, len(times))}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c2_bt4_15x1024", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-sample", type=int, default=16)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend evaluates on one GPU (batch rows are independent; more GPUs means "
+                 "one backend instance per GPU fed by lc0's demux, nothing to measure here). Use --gpus 1.")
+
+    import numpy as np
+
+    from lc0_amd import Network, netgen
+    from oracle import chess as oc   # input generator only (seeded random playouts)
+
+    wl = WORKLOADS[args.config]
+    batch = args.batch or wl["batch"]
+    path = netgen.cached_config(args.config)
+    pos = oc.random_positions(max(batch, args.cpu_sample), seed=20240)
+    masks, values = pos["masks"], pos["values"]
+
+    net = Network(path, "gpu=0,max_batch=%d" % max(batch, 16))
+    comp = net.NewComputation()
+    comp.AddInputs(masks[:batch], values[:batch])
+    comp.ComputeBlocking()          # stages the batch into HBM and warms everything up
+    checksum = float(np.abs(comp.results()["policy"]).sum())
+
+    # Whole path including host staging (H2D of planes, D2H of 1858 logits): reported, never `value`.
+    t0 = time.perf_counter()
+    io_iters = max(3, min(10, args.steps))
+    for _ in range(io_iters):
+        comp.ComputeBlocking()
+    io_ms = (time.perf_counter() - t0) * 1e3 / io_iters
+
+    # Timed region: K device passes over the resident batch, bracketed by stream
+    # synchronisation on both sides (inside TimeResidentForward) and by the host clock.
+    if args.warmup > 0:
+        net.TimeResidentForward(batch, args.warmup)
+    t0 = time.perf_counter()
+    ev_ms = net.TimeResidentForward(batch, args.steps)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # Per-kernel HIP-event timing of one more pass (events on the compute stream).
+    net.SetProfiling(True)
+    prof_iters = 3
+    for _ in range(prof_iters):
+        comp.ComputeBlocking()
+    prof = net.TakeProfile()
+    net.SetProfiling(False)
+    total_kernel_ms = sum(k.ms for k in prof) / prof_iters
+    kernels = sorted(prof, key=lambda k: -k.ms)
+    dom = kernels[0]
+    gemm_ms = sum(k.ms for k in prof if k.name.startswith("gemm") or k.name == "attention") / prof_iters
+    gemm_flops = sum(k.flops for k in prof if k.name.startswith("gemm") or k.name == "attention") / prof_iters
+    if dom.flops > 0:
+        achieved = dom.flops / dom.launches / (dom.ms / dom.launches * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": dom.name, "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
+                    "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS, "traffic": None,
+                    "avg_launch_ms": dom.ms / dom.launches, "launches_per_step": dom.launches // prof_iters}
+    else:
+        achieved = dom.bytes / dom.launches / (dom.ms / dom.launches * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": dom.name, "achieved": achieved, "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                    "avg_launch_ms": dom.ms / dom.launches, "launches_per_step": dom.launches // prof_iters}
+
+    result = {
+        "metric": "NN evals/sec at batch 256, BT4-shape fp16",
+        "value": batch / (wall_ms * 1e-3),
+        "unit": "evals/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": args.config, "description": wl["desc"], "batch": batch,
+                   "inputs": "seeded random-playout positions, classical 112 planes"},
+        "roofline": roofline,
+        "event_ms_per_step": ev_ms,
+        "with_host_io_evals_per_s": batch / (io_ms * 1e-3),
+        "all_gemm_attention": {"ms_per_step": gemm_ms, "tflops": gemm_flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None,
+                               "frac_of_mfma_peak": gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS if gemm_ms else None},
+        "kernel_ms_per_step": {k.name: round(k.ms / prof_iters, 4) for k in kernels},
+        "sum_kernel_ms_per_step": total_kernel_ms,
+        "policy_checksum": checksum,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(path, masks, values, args.cpu_sample)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,50 @@
+/*
+ * Single-kernel entry points of liblc0mi.so, for parity tests and kernel
+ * micro-benchmarks. All pointers are HOST pointers; each call stages its
+ * operands into HBM, launches exactly one kernel of the forward pass and
+ * copies the result back. Halves are passed as raw IEEE binary16 bits.
+ * Return value: 0 on success, else lc0mi_last_error() has the message.
+ */
+#ifndef LC0MI_KERNELS_H_
+#define LC0MI_KERNELS_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* C[b][m][n] = act(scale * A[b][m][:] . W[b][n][:] + bias[n]); the kernel behind
+ * FullyConnectedLayer::Forward1D (src/neural/backends/blas/fully_connected_layer.cc:49-106).
+ * strides in elements between batch entries; out_f32 selects float output.
+ * If time_iters > 0, *ms receives the mean HIP-event time of that many extra launches. */
+int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* W, int ldw, long long strideW,
+                 const float* bias, int M, int N, int K, int batch, float scale, int act, int out_f32, void* C,
+                 int ldc, long long strideC, int time_iters, double* ms);
+/* float variant (fp32 configuration). */
+int lc0mi_k_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, int M, int N, int K,
+                     float scale, int act, float* C, int ldc);
+/* y = LN(x * alpha + skip) * gamma + beta, rows of C halves; skip may be NULL.
+ * (LayerNorm2DWithSkipConnection, src/neural/backends/blas/encoder.h:29-66) */
+int lc0mi_k_layer_norm(const uint16_t* x, const uint16_t* skip, const float* gamma, const float* beta, int rows,
+                       int C, float alpha, float eps, uint16_t* y, int time_iters, double* ms);
+/* Fused attention: qkv [B*64][3*heads*32] halves, bias [B][heads][64 q][64 k]
+ * halves in natural order (may be NULL), out [B*64][heads*32]
+ * (src/neural/backends/blas/network_blas.cc:352-439). */
+int lc0mi_k_attention(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, float scale, uint16_t* out,
+                      int time_iters, double* ms);
+/* Input planes -> [B*64][ld] halves with position encoding appended
+ * (src/neural/backends/blas/network_blas.cc:973-981, 630-652). */
+int lc0mi_k_expand_planes_attn(const uint64_t* masks, const float* values, int batch, int ld, uint16_t* out,
+                               int time_iters, double* ms);
+/* Input planes -> [B][112][64] floats (EncodePlanes, network_blas.cc:973-981). */
+int lc0mi_k_expand_planes_nchw(const uint64_t* masks, const float* values, int batch, float* out);
+/* Attention-policy tail: logits [B][4096] floats, keys [B*64][pd] halves,
+ * ppo [4][pd] floats -> policy [B][1858] (network_blas.cc:873-914). */
+int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const float* ppo, int pd, int batch,
+                               float* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LC0MI_KERNELS_H_ */

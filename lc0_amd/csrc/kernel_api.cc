@@ -1,0 +1,238 @@
+// Host-pointer wrappers around single kernels (see include/lc0mi_kernels.h).
+#include "../../include/lc0mi_kernels.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "kernels.h"
+#include "tables.h"
+#include "weights.h"
+
+extern "C" const char* lc0mi_last_error(void);
+namespace lc0mi {
+void SetLastError(const std::string& msg);
+}
+
+namespace {
+using lc0mi::Error;
+using lc0mi::half_t;
+
+#define K_CHECK(expr)                                                                              \
+  do {                                                                                             \
+    hipError_t e__ = (expr);                                                                       \
+    if (e__ != hipSuccess) throw Error(std::string("HIP error: ") + hipGetErrorString(e__) + " (" #expr ")"); \
+  } while (0)
+
+struct Dev {
+  std::vector<void*> ptrs;
+  ~Dev() {
+    for (void* p : ptrs) (void)hipFree(p);
+  }
+  void* Alloc(size_t bytes) {
+    void* p = nullptr;
+    K_CHECK(hipMalloc(&p, bytes < 256 ? 256 : bytes));
+    ptrs.push_back(p);
+    return p;
+  }
+  template <typename T>
+  T* Put(const T* host, size_t n) {
+    T* d = static_cast<T*>(Alloc(n * sizeof(T)));
+    if (n) K_CHECK(hipMemcpy(d, host, n * sizeof(T), hipMemcpyHostToDevice));
+    return d;
+  }
+};
+
+void RequireDevice() {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n == 0) throw Error("No HIP device is available.");
+}
+
+template <typename F>
+double TimeLaunches(int iters, F&& launch) {
+  hipEvent_t a, b;
+  K_CHECK(hipEventCreate(&a));
+  K_CHECK(hipEventCreate(&b));
+  launch();  // warm-up
+  K_CHECK(hipEventRecord(a, nullptr));
+  for (int i = 0; i < iters; i++) launch();
+  K_CHECK(hipEventRecord(b, nullptr));
+  K_CHECK(hipEventSynchronize(b));
+  float ms = 0;
+  K_CHECK(hipEventElapsedTime(&ms, a, b));
+  (void)hipEventDestroy(a);
+  (void)hipEventDestroy(b);
+  return ms / iters;
+}
+
+template <typename F>
+int Guard(F&& f) {
+  try {
+    f();
+    return 0;
+  } catch (const std::exception& e) {
+    lc0mi::SetLastError(e.what());
+    return 1;
+  }
+}
+}  // namespace
+
+extern "C" {
+
+int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* W, int ldw, long long strideW,
+                 const float* bias, int M, int N, int K, int batch, float scale, int act, int out_f32, void* C,
+                 int ldc, long long strideC, int time_iters, double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (K % 8 || lda % 8 || ldw % 8 || strideA % 8 || strideW % 8) throw Error("K, lda, ldw and strides must be multiples of 8");
+    if (M < 1 || N < 1 || batch < 1 || lda < K || ldw < K || ldc < N) throw Error("bad gemm shape");
+    Dev dev;
+    const size_t a_elems = (size_t)(batch - 1) * strideA + (size_t)(M - 1) * lda + K;
+    const size_t w_elems = (size_t)(batch - 1) * strideW + (size_t)(N - 1) * ldw + K;
+    const size_t c_elems = (size_t)(batch - 1) * strideC + (size_t)(M - 1) * ldc + N;
+    const size_t c_size = out_f32 ? 4 : 2;
+    lc0mi::GemmArgs g;
+    g.A = reinterpret_cast<const half_t*>(dev.Put(A, a_elems)); g.lda = lda; g.strideA = strideA;
+    g.W = reinterpret_cast<const half_t*>(dev.Put(W, w_elems)); g.ldw = ldw; g.strideW = strideW;
+    g.C = dev.Alloc(c_elems * c_size); g.ldc = ldc; g.strideC = strideC;
+    K_CHECK(hipMemcpy(g.C, C, c_elems * c_size, hipMemcpyHostToDevice));
+    g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
+    g.M = M; g.N = N; g.K = K; g.batch = batch; g.scale = scale; g.act = act; g.out_f32 = out_f32 != 0;
+    lc0mi::LaunchGemm(g, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(C, g.C, c_elems * c_size, hipMemcpyDeviceToHost));
+    if (time_iters > 0 && ms) *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchGemm(g, nullptr); });
+  });
+}
+
+int lc0mi_k_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, int M, int N, int K,
+                     float scale, int act, float* C, int ldc) {
+  return Guard([&] {
+    RequireDevice();
+    if (K % 4 || lda % 4 || ldw % 4) throw Error("K, lda and ldw must be multiples of 4");
+    if (M < 1 || N < 1 || lda < K || ldw < K || ldc < N) throw Error("bad gemm shape");
+    Dev dev;
+    lc0mi::GemmArgsF32 g;
+    g.A = dev.Put(A, (size_t)(M - 1) * lda + K); g.lda = lda;
+    g.W = dev.Put(W, (size_t)(N - 1) * ldw + K); g.ldw = ldw;
+    const size_t c_elems = (size_t)(M - 1) * ldc + N;
+    g.C = dev.Put(C, c_elems); g.ldc = ldc;
+    g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
+    g.M = M; g.N = N; g.K = K; g.scale = scale; g.act = act;
+    lc0mi::LaunchGemmF32(g, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(C, g.C, c_elems * sizeof(float), hipMemcpyDeviceToHost));
+  });
+}
+
+int lc0mi_k_layer_norm(const uint16_t* x, const uint16_t* skip, const float* gamma, const float* beta, int rows,
+                       int C, float alpha, float eps, uint16_t* y, int time_iters, double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (C % 8 || C < 8 || C > 8192 || rows < 1) throw Error("bad layer norm shape");
+    Dev dev;
+    const size_t n = (size_t)rows * C;
+    auto* dx = reinterpret_cast<half_t*>(dev.Put(x, n));
+    auto* ds = skip ? reinterpret_cast<half_t*>(dev.Put(skip, n)) : nullptr;
+    auto* dy = reinterpret_cast<half_t*>(dev.Alloc(n * 2));
+    float* dg = dev.Put(gamma, (size_t)C);
+    float* db = dev.Put(beta, (size_t)C);
+    lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(y, dy, n * 2, hipMemcpyDeviceToHost));
+    if (time_iters > 0 && ms) {
+      *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr); });
+    }
+  });
+}
+
+int lc0mi_k_attention(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, float scale, uint16_t* out,
+                      int time_iters, double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1 || heads < 1) throw Error("bad attention shape");
+    Dev dev;
+    const int d = heads * 32;
+    auto* dq = reinterpret_cast<half_t*>(dev.Put(qkv, (size_t)batch * 64 * 3 * d));
+    half_t* db = nullptr;
+    if (bias) {
+      std::vector<uint16_t> perm((size_t)batch * heads * 4096);
+      for (size_t bh = 0; bh < (size_t)batch * heads; bh++)
+        for (int q = 0; q < 64; q++)
+          for (int k = 0; k < 64; k++) perm[bh * 4096 + lc0mi::SmolgenBiasIndex(q, k)] = bias[bh * 4096 + q * 64 + k];
+      db = reinterpret_cast<half_t*>(dev.Put(perm.data(), perm.size()));
+    }
+    auto* dout = reinterpret_cast<half_t*>(dev.Alloc((size_t)batch * 64 * d * 2));
+    lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(out, dout, (size_t)batch * 64 * d * 2, hipMemcpyDeviceToHost));
+    if (time_iters > 0 && ms) {
+      *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr); });
+    }
+  });
+}
+
+int lc0mi_k_expand_planes_attn(const uint64_t* masks, const float* values, int batch, int ld, uint16_t* out,
+                               int time_iters, double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1 || ld < 176) throw Error("bad expand shape");
+    Dev dev;
+    uint64_t* dm = dev.Put(masks, (size_t)batch * 112);
+    float* dv = dev.Put(values, (size_t)batch * 112);
+    const std::vector<float>& pe = lc0mi::PosEncoding();
+    std::vector<half_t> peh(pe.size());
+    for (size_t i = 0; i < pe.size(); i++) peh[i] = (half_t)pe[i];
+    half_t* dpe = dev.Put(peh.data(), peh.size());
+    auto* dout = reinterpret_cast<half_t*>(dev.Alloc((size_t)batch * 64 * ld * 2));
+    lc0mi::LaunchExpandPlanesAttn<half_t>(dm, dv, dpe, dout, ld, batch, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(out, dout, (size_t)batch * 64 * ld * 2, hipMemcpyDeviceToHost));
+    if (time_iters > 0 && ms) {
+      *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchExpandPlanesAttn<half_t>(dm, dv, dpe, dout, ld, batch, nullptr); });
+    }
+  });
+}
+
+int lc0mi_k_expand_planes_nchw(const uint64_t* masks, const float* values, int batch, float* out) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1) throw Error("bad expand shape");
+    Dev dev;
+    uint64_t* dm = dev.Put(masks, (size_t)batch * 112);
+    float* dv = dev.Put(values, (size_t)batch * 112);
+    auto* dout = static_cast<float*>(dev.Alloc((size_t)batch * 112 * 64 * 4));
+    lc0mi::LaunchExpandPlanesNchw<float>(dm, dv, dout, batch, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(out, dout, (size_t)batch * 112 * 64 * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const float* ppo, int pd, int batch,
+                               float* out) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1 || pd < 1) throw Error("bad policy shape");
+    Dev dev;
+    float* dl = dev.Put(logits, (size_t)batch * 4096);
+    auto* dk = reinterpret_cast<half_t*>(dev.Put(keys, (size_t)batch * 64 * pd));
+    float* dp = dev.Put(ppo, (size_t)4 * pd);
+    const auto& inv = lc0mi::AttnPolicyInverseMap();
+    int16_t* di = dev.Put(inv.data(), inv.size());
+    auto* dout = static_cast<float*>(dev.Alloc((size_t)batch * 1858 * 4));
+    lc0mi::LaunchAttnPolicyGather(dl, dk, pd, 0, dp, pd, di, dout, batch, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(out, dout, (size_t)batch * 1858 * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+}  // extern "C"

@@ -1,0 +1,74 @@
+// Launchers of the gfx950 kernels. Host code sees only these plain functions;
+// all of them enqueue work on the given stream and return without waiting.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdint>
+
+namespace lc0mi {
+
+using half_t = _Float16;
+
+// C[b][m][n] = act(scale * sum_k A[b][m][k] * W[b][n][k] + bias[n]),  b < batch.
+// A and W are K-contiguous (row-major activations, lc0's [out][in] weights).
+// Requirements: K % 8 == 0, lda % 8 == 0, ldw % 8 == 0, 16-byte aligned bases
+// and batch strides; M, N arbitrary. bias may be null (then no bias; the
+// activation is still applied). out_f32 selects float output.
+struct GemmArgs {
+  const half_t* A = nullptr; int lda = 0; long long strideA = 0;
+  const half_t* W = nullptr; int ldw = 0; long long strideW = 0;
+  void* C = nullptr; int ldc = 0; long long strideC = 0;
+  const float* bias = nullptr;
+  int M = 0, N = 0, K = 0, batch = 1;
+  float scale = 1.0f;
+  int act = 3;  // Activation enum value (3 = none)
+  bool out_f32 = false;
+};
+void LaunchGemm(const GemmArgs& args, hipStream_t stream);
+
+// Same contract in float: C = act(scale * A.W^T + bias) with float A, W, C.
+// K % 4 == 0, lda % 4 == 0, ldw % 4 == 0.
+struct GemmArgsF32 {
+  const float* A = nullptr; int lda = 0; long long strideA = 0;
+  const float* W = nullptr; int ldw = 0; long long strideW = 0;
+  float* C = nullptr; int ldc = 0; long long strideC = 0;
+  const float* bias = nullptr;
+  int M = 0, N = 0, K = 0, batch = 1;
+  float scale = 1.0f;
+  int act = 3;
+};
+void LaunchGemmF32(const GemmArgsF32& args, hipStream_t stream);
+
+// Input planes -> token-major embedding input with the 64 position-encoding
+// channels appended: out[b*64+sq][c], c < 112 plane bits * value, 112..175 the
+// pos-enc row of sq, then zero padding up to ld. T = half_t or float.
+template <typename T>
+void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T* pos_enc /*[64][64]*/,
+                            T* out, int ld, int batch, hipStream_t stream);
+// Input planes -> NCHW dense planes out[b][c][sq] (T = half_t or float).
+template <typename T>
+void LaunchExpandPlanesNchw(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream);
+
+// rows x C layer norm: y = beta + gamma * (t - mean) / sqrt(var + eps) with
+// t = x * alpha + skip (skip may be null). x, skip, y may alias. C % 8 == 0, C <= 8192.
+void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
+                     int rows, int C, float alpha, float eps, hipStream_t stream);
+
+// Fused multi-head attention over 64 tokens, head depth 32.
+// qkv: [B*64][3*d_model] (q | k | v column blocks), bias: smolgen logits in the
+// tile-native layout produced by SmolgenBiasIndex (may be null), out: [B*64][d_model].
+void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int batch, int heads,
+                     float scale, hipStream_t stream);
+// Position inside one head's 4096-entry bias block of logit (query q, key k).
+int SmolgenBiasIndex(int q, int k);
+
+// Attention policy tail: promotion offsets + gather to 1858 moves.
+// logits: [B][64*64] float (already scaled), kq: [B*64][ld_kq] with keys at column
+// offset key_off, ppo: [4][pd] float, inv_map: [1858] source index into the
+// 4096+192 virtual buffer. out: [B][1858] float.
+void LaunchAttnPolicyGather(const float* logits, const half_t* kq, int ld_kq, int key_off, const float* ppo,
+                            int pd, const int16_t* inv_map, float* out, int batch, hipStream_t stream);
+
+}  // namespace lc0mi

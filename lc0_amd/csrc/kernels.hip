@@ -1,0 +1,597 @@
+// Hand-written gfx950 (CDNA4, wave64) kernels of the attention-body path.
+//
+// What each kernel replaces in the reference CPU backend (file:line):
+//   gemm_kernel           FullyConnectedLayer::Forward1D  blas/fully_connected_layer.cc:49-106
+//                         (+ bias/activation of shared/activation.cc:102-164) and the per-sample
+//                         Q.K^T sgemm of the attention policy (blas/network_blas.cc:850-872)
+//   expand_planes_*       BlasComputation::EncodePlanes + NCHW->NHWC + pos-enc concat
+//                         blas/network_blas.cc:973-981, 630-652
+//   layer_norm_kernel     LayerNorm2DWithSkipConnection   blas/encoder.h:29-66
+//   attention_kernel      per-head QK^T, +smolgen, softmax, .V   blas/network_blas.cc:352-439
+//   attn_policy_gather    promotion offsets + kAttnPolicyMap gather  blas/network_blas.cc:873-914
+#include "kernels.h"
+
+namespace lc0mi {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+// Activation functions with the reference's formulas (shared/activation.cc:51-100).
+__device__ __forceinline__ float ActMish(float v) {
+  float e = __expf(v);
+  float n = e * e + 2.0f * e;
+  float d = v / (n + 2.0f);
+  return v <= -0.125f ? n * d : v - 2.0f * d;
+}
+__device__ __forceinline__ float Activate(float v, int act) {
+  switch (act) {
+    case 1: return ActMish(v);
+    case 2: return v > 0.0f ? v : 0.0f;
+    case 4: return tanhf(v);
+    case 5: return 1.0f / (1.0f + __expf(-v));
+    case 6: return v > 0.0f ? 1.05070098f * v : 1.05070098f * 1.67326324f * (__expf(v) - 1.0f);
+    case 7: return v / (1.0f + __expf(-v));
+    case 8: return v > 0.0f ? v * v : 0.0f;
+    default: return v;
+  }
+}
+
+__device__ __forceinline__ float WaveSum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// ---------------------------------------------------------------------------
+// GEMM  C[m][n] = act(scale * sum_k A[m][k] W[n][k] + bias[n])
+//
+// 256 threads = 4 waves laid out WAVES_M x WAVES_N over a BM x BN block tile;
+// each wave owns (BM/WAVES_M) x (BN/WAVES_N) as 32x32 MFMA tiles
+// (v_mfma_f32_32x32x16_f16). The weight rows are the MFMA "A" operand and the
+// activation rows the "B" operand, so a lane ends up holding 4 consecutive n
+// for one m and stores 8 bytes at a time. Global tiles are fetched as 16-byte
+// vectors into registers one k-tile ahead and staged through padded LDS.
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, typename OutT>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
+  static_assert(WAVES_M * WAVES_N == 4, "four waves per block");
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int LDS_STRIDE = BK + 8;  // halves; 16-byte rows shifted by 4 banks per row
+  constexpr int VEC_PER_ROW = BK / 8;
+  constexpr int A_VECS = BM * VEC_PER_ROW / 256;
+  constexpr int W_VECS = BN * VEC_PER_ROW / 256;
+  static_assert(A_VECS >= 1 && W_VECS >= 1, "tile too small for 256 threads");
+
+  __shared__ __attribute__((aligned(16))) half_t As[BM * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) half_t Ws[BN * LDS_STRIDE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const half_t* A = p.A + (long long)blockIdx.z * p.strideA;
+  const half_t* W = p.W + (long long)blockIdx.z * p.strideW;
+  const int M = p.M, N = p.N, K = p.K;
+
+  uint4 ra[A_VECS], rw[W_VECS];
+  auto load_tile = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_VECS; i++) {
+      int v = tid + i * 256;
+      int row = v / VEC_PER_ROW, kv = v % VEC_PER_ROW;
+      int gm = min(m0 + row, M - 1), k = k0 + kv * 8;
+      ra[i] = k < K ? *reinterpret_cast<const uint4*>(A + (long long)gm * p.lda + k) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < W_VECS; i++) {
+      int v = tid + i * 256;
+      int row = v / VEC_PER_ROW, kv = v % VEC_PER_ROW;
+      int gn = min(n0 + row, N - 1), k = k0 + kv * 8;
+      rw[i] = k < K ? *reinterpret_cast<const uint4*>(W + (long long)gn * p.ldw + k) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < A_VECS; i++) {
+      int v = tid + i * 256;
+      int row = v / VEC_PER_ROW, kv = v % VEC_PER_ROW;
+      *reinterpret_cast<uint4*>(&As[row * LDS_STRIDE + kv * 8]) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W_VECS; i++) {
+      int v = tid + i * 256;
+      int row = v / VEC_PER_ROW, kv = v % VEC_PER_ROW;
+      *reinterpret_cast<uint4*>(&Ws[row * LDS_STRIDE + kv * 8]) = rw[i];
+    }
+  };
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+  const int nk = (K + BK - 1) / BK;
+  const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+  load_tile(0);
+  for (int kt = 0; kt < nk; kt++) {
+    store_tile();
+    __syncthreads();
+    if (kt + 1 < nk) load_tile((kt + 1) * BK);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      half8 af[TM], wf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+        af[i] = *reinterpret_cast<const half8*>(&As[(wm * WM + i * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+        wf[j] = *reinterpret_cast<const half8*>(&Ws[(wn * WN + j * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // Epilogue. Accumulator element e of a tile: n = 8*(e/4) + 4*(lane/32) + e%4, m = lane%32.
+  OutT* C = reinterpret_cast<OutT*>(p.C) + (long long)blockIdx.z * p.strideC;
+  const bool vec_ok = (p.ldc % 4 == 0);
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int m = m0 + wm * WM + i * 32 + frag_row;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+      for (int blk = 0; blk < 4; blk++) {
+        const int n = n0 + wn * WN + j * 32 + blk * 8 + (lane >> 5) * 4;
+        if (n >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          float x = acc[i][j][blk * 4 + r] * p.scale;
+          if (p.bias != nullptr && n + r < N) x += p.bias[n + r];
+          v[r] = Activate(x, p.act);
+        }
+        OutT* dst = C + (long long)m * p.ldc + n;
+        if (vec_ok && n + 3 < N) {
+          if constexpr (sizeof(OutT) == 2) {
+            half4 h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+            *reinterpret_cast<half4*>(dst) = h;
+          } else {
+            floatx4 f = {v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<floatx4*>(dst) = f;
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            if (n + r < N) dst[r] = (OutT)v[r];
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
+  dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch);
+  if (a.out_f32) {
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, float>), grid, dim3(256), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, half_t>), grid, dim3(256), 0, stream, a);
+  }
+}
+
+}  // namespace
+
+void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
+  const long long big_tiles = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
+  if (big_tiles >= 192) {
+    LaunchGemmTile<128, 128, 64, 2, 2>(a, stream);
+  } else {
+    LaunchGemmTile<64, 64, 64, 2, 2>(a, stream);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// float GEMM (fp32 configuration): same contract, LDS-tiled, 64x64 block tile,
+// each thread a 4x4 register tile, plain fp32 FMAs with fp32 accumulation.
+// ---------------------------------------------------------------------------
+namespace {
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgsF32 p) {
+  constexpr int BM = 64, BN = 64, BK = 16;
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Ws[BK][BN + 4];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const float* A = p.A + (long long)blockIdx.z * p.strideA;
+  const float* W = p.W + (long long)blockIdx.z * p.strideW;
+  float* C = p.C + (long long)blockIdx.z * p.strideC;
+  const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
+  float acc[4][4] = {};
+  const int lrow = tid / 4, lk = (tid % 4) * 4;  // 64 rows x 4 float4 per tile
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+    floatx4 va = {0, 0, 0, 0}, vw = {0, 0, 0, 0};
+    if (k0 + lk < p.K) {
+      va = *reinterpret_cast<const floatx4*>(A + (long long)min(m0 + lrow, p.M - 1) * p.lda + k0 + lk);
+      vw = *reinterpret_cast<const floatx4*>(W + (long long)min(n0 + lrow, p.N - 1) * p.ldw + k0 + lk);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) { As[lk + e][lrow] = va[e]; Ws[lk + e][lrow] = vw[e]; }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; k++) {
+      float a[4], w[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) { a[e] = As[k][tm + e]; w[e] = Ws[k][tn + e]; }
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int m = m0 + tm + i;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      int n = n0 + tn + j;
+      if (n >= p.N) continue;
+      float x = acc[i][j] * p.scale;
+      if (p.bias != nullptr) x += p.bias[n];
+      C[(long long)m * p.ldc + n] = Activate(x, p.act);
+    }
+  }
+}
+}  // namespace
+
+void LaunchGemmF32(const GemmArgsF32& a, hipStream_t stream) {
+  if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
+  dim3 grid((a.M + 63) / 64, (a.N + 63) / 64, a.batch);
+  hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, a);
+}
+
+// ---------------------------------------------------------------------------
+// Input plane expansion.
+// ---------------------------------------------------------------------------
+namespace {
+template <typename T>
+__global__ __launch_bounds__(256) void expand_planes_attn_kernel(const uint64_t* __restrict__ masks,
+                                                                 const float* __restrict__ values,
+                                                                 const T* __restrict__ pos_enc, T* __restrict__ out,
+                                                                 int ld) {
+  const int b = blockIdx.x;
+  __shared__ uint64_t smask[112];
+  __shared__ float sval[112];
+  if (threadIdx.x < 112) {
+    smask[threadIdx.x] = masks[(long long)b * 112 + threadIdx.x];
+    sval[threadIdx.x] = values[(long long)b * 112 + threadIdx.x];
+  }
+  __syncthreads();
+  T* o = out + (long long)b * 64 * ld;
+  for (int i = threadIdx.x; i < 64 * ld; i += 256) {
+    int sq = i / ld, c = i - sq * ld;
+    T v = (T)0.0f;
+    if (c < 112) {
+      if ((smask[c] >> sq) & 1ull) v = (T)sval[c];
+    } else if (c < 176) {
+      v = pos_enc[sq * 64 + (c - 112)];
+    }
+    o[i] = v;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void expand_planes_nchw_kernel(const uint64_t* __restrict__ masks,
+                                                                 const float* __restrict__ values,
+                                                                 T* __restrict__ out, long long total) {
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  long long plane = i >> 6;
+  int sq = (int)(i & 63);
+  out[i] = ((masks[plane] >> sq) & 1ull) ? (T)values[plane] : (T)0.0f;
+}
+}  // namespace
+
+template <typename T>
+void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T* pos_enc, T* out, int ld,
+                            int batch, hipStream_t stream) {
+  if (batch <= 0) return;
+  hipLaunchKernelGGL(expand_planes_attn_kernel<T>, dim3(batch), dim3(256), 0, stream, masks, values, pos_enc, out,
+                     ld);
+}
+template void LaunchExpandPlanesAttn<half_t>(const uint64_t*, const float*, const half_t*, half_t*, int, int,
+                                             hipStream_t);
+template void LaunchExpandPlanesAttn<float>(const uint64_t*, const float*, const float*, float*, int, int,
+                                            hipStream_t);
+
+template <typename T>
+void LaunchExpandPlanesNchw(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream) {
+  if (batch <= 0) return;
+  long long total = (long long)batch * 112 * 64;
+  hipLaunchKernelGGL(expand_planes_nchw_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                     masks, values, out, total);
+}
+template void LaunchExpandPlanesNchw<half_t>(const uint64_t*, const float*, half_t*, int, hipStream_t);
+template void LaunchExpandPlanesNchw<float>(const uint64_t*, const float*, float*, int, hipStream_t);
+
+// ---------------------------------------------------------------------------
+// Layer norm with optional skip: one wave per row, the row held in registers.
+// ---------------------------------------------------------------------------
+namespace {
+template <int NV>  // 16-byte vectors per lane; covers C <= 512 * NV
+__global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restrict__ x, const half_t* skip,
+                                                         half_t* y, const float* __restrict__ gamma,
+                                                         const float* __restrict__ beta, int rows, int C,
+                                                         float alpha, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int nvec = C / 8;
+  const half_t* xr = x + (long long)row * C;
+  const half_t* sr = skip ? skip + (long long)row * C : nullptr;
+  float t[NV][8];
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    int v = lane + i * 64;
+    if (v < nvec) {
+      half8 hx = *reinterpret_cast<const half8*>(xr + v * 8);
+      if (sr) {
+        half8 hs = *reinterpret_cast<const half8*>(sr + v * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++) t[i][e] = (float)hx[e] * alpha + (float)hs[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) t[i][e] = (float)hx[e] * alpha;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e++) sum += t[i][e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) t[i][e] = 0.0f;
+    }
+  }
+  const float mean = WaveSum(sum) / (float)C;
+  float var = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    if (lane + i * 64 < nvec) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) { float d = t[i][e] - mean; var += d * d; }
+    }
+  }
+  var = WaveSum(var) / (float)C;
+  const float den = 1.0f / sqrtf(var + eps);
+  half_t* yr = y + (long long)row * C;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    int v = lane + i * 64;
+    if (v < nvec) {
+      half8 o;
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = (half_t)(beta[v * 8 + e] + gamma[v * 8 + e] * (t[i][e] - mean) * den);
+      *reinterpret_cast<half8*>(yr + v * 8) = o;
+    }
+  }
+}
+}  // namespace
+
+void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
+                     int rows, int C, float alpha, float eps, hipStream_t stream) {
+  if (rows <= 0) return;
+  dim3 grid((rows + 3) / 4), block(256);
+  if (C <= 512) {
+    hipLaunchKernelGGL(layer_norm_kernel<1>, grid, block, 0, stream, x, skip, y, gamma, beta, rows, C, alpha, eps);
+  } else if (C <= 1024) {
+    hipLaunchKernelGGL(layer_norm_kernel<2>, grid, block, 0, stream, x, skip, y, gamma, beta, rows, C, alpha, eps);
+  } else if (C <= 2048) {
+    hipLaunchKernelGGL(layer_norm_kernel<4>, grid, block, 0, stream, x, skip, y, gamma, beta, rows, C, alpha, eps);
+  } else {  // callers guarantee C <= 8192
+    hipLaunchKernelGGL(layer_norm_kernel<16>, grid, block, 0, stream, x, skip, y, gamma, beta, rows, C, alpha,
+                       eps);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Fused attention for 64 tokens and head depth 32: one wave per (sample, head).
+//
+// S^T = K.Q^T is computed so that a lane holds, for its query column, 32 of the
+// 64 key logits in registers (the other 32 live in lane^32): the softmax over
+// keys is an in-register reduction plus one cross-lane exchange. The
+// probabilities are then already laid out as the "A" operand of P.V.
+// Key order inside one 16-key MFMA step s for lane half g and slot e:
+//   key = 16 s + 8 (e / 4) + 4 g + e % 4.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr int kVStride = 40;  // halves per key row of V in LDS
+
+__global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict__ qkv,
+                                                        const half_t* __restrict__ bias,
+                                                        half_t* __restrict__ out, int total_heads, int heads,
+                                                        float scale) {
+  __shared__ __attribute__((aligned(16))) half_t Vs[4][64 * kVStride];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int gh_raw = blockIdx.x * 4 + wave;
+  const bool live = gh_raw < total_heads;
+  const int gh = live ? gh_raw : total_heads - 1;
+  const int b = gh / heads, h = gh - b * heads;
+  const int d_model = heads * 32, ld = 3 * d_model;
+  const half_t* Q = qkv + (long long)b * 64 * ld + h * 32;
+  const half_t* Kp = Q + d_model;
+  const half_t* V = Q + 2 * d_model;
+  const int r = lane & 31, g = lane >> 5;
+
+  // Stage V (64 keys x 32 depth) into this wave's LDS region.
+  half_t* vs = Vs[wave];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int v = lane + 64 * i;
+    int row = v >> 2, cv = v & 3;
+    *reinterpret_cast<uint4*>(&vs[row * kVStride + cv * 8]) =
+        *reinterpret_cast<const uint4*>(V + (long long)row * ld + cv * 8);
+  }
+
+  floatx16 st[2][2];
+#pragma unroll
+  for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+    for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) st[mt][nt][e] = 0.0f;
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) {
+    half8 kf[2], qf[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      kf[t] = *reinterpret_cast<const half8*>(Kp + (long long)(32 * t + r) * ld + 16 * ks + 8 * g);
+      qf[t] = *reinterpret_cast<const half8*>(Q + (long long)(32 * t + r) * ld + 16 * ks + 8 * g);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++)
+        st[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[mt], qf[nt], st[mt][nt], 0, 0, 0);
+  }
+
+  // Scale, add the smolgen logits, softmax over keys per query column.
+  const half_t* bh = bias ? bias + (long long)gh * 4096 : nullptr;
+#pragma unroll
+  for (int nt = 0; nt < 2; nt++) {
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+      for (int bp = 0; bp < 2; bp++) {
+        half8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (bh) bv = *reinterpret_cast<const half8*>(bh + ((nt * 2 + mt) * 2 + bp) * 512 + lane * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          float s = st[mt][nt][bp * 8 + e] * scale + (float)bv[e];
+          st[mt][nt][bp * 8 + e] = s;
+          mx = fmaxf(mx, s);
+        }
+      }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float sum = 0.0f;
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        float ev = __expf(st[mt][nt][e] - mx);
+        st[mt][nt][e] = ev;
+        sum += ev;
+      }
+    sum += __shfl_xor(sum, 32, 64);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) st[mt][nt][e] *= inv;
+  }
+
+  __syncthreads();  // V tile visible (each wave reads only its own region)
+
+  floatx16 o[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) o[nt][e] = 0.0f;
+#pragma unroll
+  for (int s = 0; s < 4; s++) {
+    half8 vf;
+#pragma unroll
+    for (int e = 0; e < 8; e++) vf[e] = vs[(16 * s + 8 * (e / 4) + 4 * g + (e % 4)) * kVStride + r];
+#pragma unroll
+    for (int nt = 0; nt < 2; nt++) {
+      half8 pf;
+#pragma unroll
+      for (int e = 0; e < 8; e++) pf[e] = (half_t)st[s / 2][nt][8 * (s % 2) + e];
+      o[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(pf, vf, o[nt], 0, 0, 0);
+    }
+  }
+  if (!live) return;
+  half_t* O = out + (long long)b * 64 * d_model + h * 32;
+#pragma unroll
+  for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      int q = 32 * nt + 8 * (e / 4) + 4 * g + (e % 4);
+      O[(long long)q * d_model + r] = (half_t)o[nt][e];
+    }
+}
+}  // namespace
+
+int SmolgenBiasIndex(int q, int k) {
+  int nt = q / 32, r = q % 32, mt = k / 32, kk = k % 32;
+  int blk = kk / 8, g = (kk % 8) / 4, j = kk % 4;
+  int lane = g * 32 + r;
+  return ((nt * 2 + mt) * 2 + blk / 2) * 512 + lane * 8 + (blk % 2) * 4 + j;
+}
+
+void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int batch, int heads, float scale,
+                     hipStream_t stream) {
+  int total = batch * heads;
+  if (total <= 0) return;
+  hipLaunchKernelGGL(attention_kernel, dim3((total + 3) / 4), dim3(256), 0, stream, qkv, bias, out, total, heads,
+                     scale);
+}
+
+// ---------------------------------------------------------------------------
+// Attention policy tail.
+// ---------------------------------------------------------------------------
+namespace {
+__global__ __launch_bounds__(256) void attn_policy_gather_kernel(const float* __restrict__ logits,
+                                                                 const half_t* __restrict__ kq, int ld_kq,
+                                                                 int key_off, const float* __restrict__ ppo, int pd,
+                                                                 const int16_t* __restrict__ inv_map,
+                                                                 float* __restrict__ out) {
+  __shared__ float off[4][8];
+  const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int u = 0; u < 8; u++) {
+    int t = wave * 8 + u;
+    int i = t / 8, j = t % 8;
+    const half_t* krow = kq + (long long)(b * 64 + 56 + j) * ld_kq + key_off;
+    float s = 0.0f;
+    for (int k = lane; k < pd; k += 64) s += (float)krow[k] * ppo[i * pd + k];
+    s = WaveSum(s);
+    if (lane == 0) off[i][j] = s;
+  }
+  __syncthreads();
+  const float* lg = logits + (long long)b * 4096;
+  for (int o = threadIdx.x; o < 1858; o += 256) {
+    int src = inv_map[o];
+    float v;
+    if (src < 4096) {
+      v = lg[src];
+    } else {
+      int q = src - 4096;
+      int k = q / 24, j = (q % 24) / 3, pc = q % 3;
+      v = lg[(48 + k) * 64 + 56 + j] + off[pc][j] + off[3][j];
+    }
+    out[(long long)b * 1858 + o] = v;
+  }
+}
+}  // namespace
+
+void LaunchAttnPolicyGather(const float* logits, const half_t* kq, int ld_kq, int key_off, const float* ppo, int pd,
+                            const int16_t* inv_map, float* out, int batch, hipStream_t stream) {
+  if (batch <= 0) return;
+  hipLaunchKernelGGL(attn_policy_gather_kernel, dim3(batch), dim3(256), 0, stream, logits, kq, ld_kq, key_off, ppo,
+                     pd, inv_map, out);
+}
+
+}  // namespace lc0mi

@@ -1,0 +1,811 @@
+// MI355X network backend: weight preparation, buffer management and the
+// launch sequence of the forward pass.
+//
+// Forward pass semantics follow lc0's blas backend (reference file:line):
+//   format validation / options        blas/network_blas.cc:983-1072,1115-1182
+//   attention body prologue            blas/network_blas.cc:603-721
+//   encoder layer                      blas/network_blas.cc:271-471
+//   value / moves-left / policy heads  blas/network_blas.cc:725-968
+//   WDL softmax, q = w - l             blas/network_blas.cc:86-111,747-762
+#include "network.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <mutex>
+#include <sstream>
+
+#include "kernels.h"
+#include "tables.h"
+
+namespace lc0mi {
+
+#define HIP_CHECK(expr)                                                                      \
+  do {                                                                                       \
+    hipError_t err__ = (expr);                                                               \
+    if (err__ != hipSuccess) {                                                               \
+      throw Error(std::string("HIP error: ") + hipGetErrorString(err__) + " (" #expr ") at " \
+                  __FILE__ ":" + std::to_string(__LINE__));                                  \
+    }                                                                                        \
+  } while (0)
+
+// ------------------------------------------------------------------ options --
+Options::Options(const std::string& kv) {
+  std::string item;
+  std::stringstream ss(kv);
+  while (std::getline(ss, item, ',')) {
+    size_t b = item.find_first_not_of(" \t");
+    if (b == std::string::npos) continue;
+    size_t e = item.find_last_not_of(" \t");
+    item = item.substr(b, e - b + 1);
+    size_t eq = item.find('=');
+    if (eq == std::string::npos) {
+      kv_[item] = "true";
+    } else {
+      kv_[item.substr(0, eq)] = item.substr(eq + 1);
+    }
+  }
+}
+int Options::GetInt(const std::string& key, int def) {
+  auto it = kv_.find(key);
+  if (it == kv_.end()) return def;
+  read_[key] = true;
+  try {
+    size_t pos = 0;
+    int v = std::stoi(it->second, &pos);
+    if (pos != it->second.size()) throw std::invalid_argument("trailing");
+    return v;
+  } catch (const std::exception&) {
+    throw Error("Option '" + key + "' expects an integer, got '" + it->second + "'.");
+  }
+}
+bool Options::GetBool(const std::string& key, bool def) {
+  auto it = kv_.find(key);
+  if (it == kv_.end()) return def;
+  read_[key] = true;
+  if (it->second == "true" || it->second == "1") return true;
+  if (it->second == "false" || it->second == "0") return false;
+  throw Error("Option '" + key + "' expects true/false, got '" + it->second + "'.");
+}
+std::string Options::GetString(const std::string& key, const std::string& def) {
+  auto it = kv_.find(key);
+  if (it == kv_.end()) return def;
+  read_[key] = true;
+  return it->second;
+}
+void Options::CheckAllOptionsRead(const std::string& backend_name) const {
+  for (const auto& kv : kv_) {
+    if (!read_.count(kv.first)) {
+      throw Error("Unknown option '" + kv.first + "' for backend " + backend_name + ".");
+    }
+  }
+}
+
+namespace {
+
+// -------------------------------------------------------------- device memory --
+class DeviceArena {
+ public:
+  ~DeviceArena() {
+    for (void* p : ptrs_) (void)hipFree(p);
+  }
+  void* Alloc(size_t bytes) {
+    void* p = nullptr;
+    HIP_CHECK(hipMalloc(&p, std::max<size_t>(bytes, 256)));
+    ptrs_.push_back(p);
+    total_ += bytes;
+    return p;
+  }
+  template <typename T>
+  T* Upload(const std::vector<T>& host) {
+    T* d = static_cast<T*>(Alloc(host.size() * sizeof(T)));
+    if (!host.empty()) HIP_CHECK(hipMemcpy(d, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice));
+    return d;
+  }
+  size_t total() const { return total_; }
+
+ private:
+  std::vector<void*> ptrs_;
+  size_t total_ = 0;
+};
+
+struct Linear {
+  half_t* w = nullptr;   // [out][ld] halves, K zero-padded to ld
+  float* b = nullptr;    // [out] or null
+  int out = 0, in = 0, ld = 0;
+};
+
+int RoundUp(int v, int m) { return (v + m - 1) / m * m; }
+
+struct EncoderDev {
+  Linear qkv, dense, ffn1, ffn2;
+  float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
+  bool has_smolgen = false;
+  Linear sg_compress, sg_dense1, sg_dense2;
+  float *sg_ln1_g = nullptr, *sg_ln1_b = nullptr, *sg_ln2_g = nullptr, *sg_ln2_b = nullptr;
+};
+
+// Pinned host staging of one batch (inputs and outputs).
+struct HostSlot {
+  uint64_t* masks = nullptr;
+  float* values = nullptr;
+  float* policy = nullptr;
+  float* wdl = nullptr;   // raw value-head outputs, 3 (WDL) or 1 per sample
+  float* mlh = nullptr;
+  int capacity = 0;
+  ~HostSlot() {
+    if (masks) (void)hipHostFree(masks);
+    if (values) (void)hipHostFree(values);
+    if (policy) (void)hipHostFree(policy);
+    if (wdl) (void)hipHostFree(wdl);
+    if (mlh) (void)hipHostFree(mlh);
+  }
+};
+
+class Mi355xNetwork;
+
+class Mi355xComputation : public NetworkComputation {
+ public:
+  explicit Mi355xComputation(Mi355xNetwork* net) : net_(net) {}
+  ~Mi355xComputation() override;
+  void AddInput(InputPlanes&& input) override;
+  void AddInputs(int n, const uint64_t* masks, const float* values) override;
+  void ComputeBlocking() override;
+  int GetBatchSize() const override { return batch_; }
+  float GetQVal(int sample) const override;
+  float GetDVal(int sample) const override;
+  float GetPVal(int sample, int move_id) const override { return GetPolicyRow(sample)[move_id]; }
+  float GetMVal(int sample) const override;
+  const float* GetPolicyRow(int sample) const override;
+
+ private:
+  void CheckSample(int sample) const {
+    if (sample < 0 || sample >= batch_) throw Error("sample index out of range");
+    if (!computed_) throw Error("ComputeBlocking() has not been called");
+  }
+  HostSlot* SlotFor(int index);
+  Mi355xNetwork* net_;
+  std::vector<std::unique_ptr<HostSlot>> slots_;
+  int batch_ = 0;
+  bool computed_ = false;
+};
+
+class Mi355xNetwork : public Network {
+ public:
+  Mi355xNetwork(const WeightsFile& file, Options& options);
+  ~Mi355xNetwork() override;
+
+  const NetworkCapabilities& GetCapabilities() const override { return caps_; }
+  std::unique_ptr<NetworkComputation> NewComputation() override {
+    return std::make_unique<Mi355xComputation>(this);
+  }
+  int GetMiniBatchSize() const override { return 256; }
+  int GetMaxBatchSize() const override { return max_batch_; }
+  void SetProfiling(bool on) override {
+    std::lock_guard<std::mutex> lock(eval_mutex_);
+    profiling_ = on;
+  }
+  std::vector<KernelTime> TakeProfile() override;
+  double TimeResidentForward(int batch, int iters) override;
+
+  // Used by the computation.
+  std::unique_ptr<HostSlot> GetSlot();
+  void ReleaseSlot(std::unique_ptr<HostSlot> slot);
+  void Evaluate(HostSlot* slot, int batch);
+  bool wdl() const { return wdl_; }
+  bool moves_left() const { return moves_left_; }
+
+ private:
+  void BuildAttentionBody(const WeightsFile& file);
+  void ForwardDevice(int batch);
+  void ForwardAttentionBody(int B);
+  Linear MakeLinear(const Vec& w, const Vec& b, int out, int in);
+  float* UploadF(const Vec& v) { return arena_.Upload(v); }
+  half_t* AllocH(size_t n) { return static_cast<half_t*>(arena_.Alloc(n * sizeof(half_t))); }
+  float* AllocF(size_t n) { return static_cast<float*>(arena_.Alloc(n * sizeof(float))); }
+
+  // Launch helpers (profiling aware).
+  template <typename F>
+  void Timed(const char* name, double flops, double bytes, F&& launch);
+  void Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act,
+            bool out_f32 = false);
+
+  NetworkCapabilities caps_;
+  int device_ = 0;
+  int max_batch_ = 1024;
+  bool wdl_ = false, moves_left_ = false, attn_body_ = false, attn_policy_ = false, conv_policy_ = false;
+  int default_act_ = kActRelu, smolgen_act_ = kActNone, ffn_act_ = kActNone;
+  std::string policy_head_, value_head_;
+  hipStream_t stream_ = nullptr;
+  DeviceArena arena_;
+  std::mutex eval_mutex_;
+  std::mutex slots_mutex_;
+  std::vector<std::unique_ptr<HostSlot>> free_slots_;
+
+  // Attention body dimensions.
+  int emb_ = 0, d_model_ = 0, heads_ = 0, dff_ = 0, in_ld_ = 192;
+  int sg_hc_ = 0, sg_hs_ = 0, sg_gen_ = 0;
+  int pol_emb_ = 0, pol_d_ = 0, val_ch_ = 0, val_fc_ = 0, val_out_ = 0, mov_ch_ = 0, mov_fc_ = 0;
+  float alpha_ = 1.0f, eps_ = 1e-6f;
+  bool any_smolgen_ = false;
+
+  // Device weights.
+  Linear emb_lin_, smolgen_w_, pol_emb_lin_, pol_qk_lin_, val_emb_lin_, val_fc1_, val_fc2_, mov_emb_lin_, mov_fc1_,
+      mov_fc2_;
+  std::vector<EncoderDev> encoders_;
+  half_t* pos_enc_ = nullptr;
+  float* ppo_ = nullptr;
+  int16_t* inv_map_ = nullptr;
+
+  // Device activations (sized for max_batch_).
+  uint64_t* d_masks_ = nullptr;
+  float* d_values_ = nullptr;
+  half_t *in0_ = nullptr, *x_ = nullptr, *t_ = nullptr, *qkv_ = nullptr, *att_ = nullptr, *ffn_ = nullptr;
+  half_t *sg1_ = nullptr, *sg2_ = nullptr, *sg3_ = nullptr, *sbias_ = nullptr;
+  half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
+  float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
+
+  // Profiling.
+  bool profiling_ = false;
+  struct Pending { std::string name; hipEvent_t start, stop; double flops, bytes; };
+  std::vector<Pending> pending_;
+  std::vector<hipEvent_t> event_pool_;
+  std::vector<KernelTime> profile_;
+  hipEvent_t NewEvent();
+  void CollectPending();
+};
+
+// ----------------------------------------------------------------- helpers --
+hipEvent_t Mi355xNetwork::NewEvent() {
+  if (!event_pool_.empty()) {
+    hipEvent_t e = event_pool_.back();
+    event_pool_.pop_back();
+    return e;
+  }
+  hipEvent_t e;
+  HIP_CHECK(hipEventCreate(&e));
+  return e;
+}
+
+template <typename F>
+void Mi355xNetwork::Timed(const char* name, double flops, double bytes, F&& launch) {
+  if (!profiling_) {
+    launch();
+    return;
+  }
+  Pending p{name, NewEvent(), NewEvent(), flops, bytes};
+  HIP_CHECK(hipEventRecord(p.start, stream_));
+  launch();
+  HIP_CHECK(hipEventRecord(p.stop, stream_));
+  pending_.push_back(p);
+}
+
+void Mi355xNetwork::CollectPending() {
+  for (Pending& p : pending_) {
+    float ms = 0.0f;
+    HIP_CHECK(hipEventElapsedTime(&ms, p.start, p.stop));
+    auto it = std::find_if(profile_.begin(), profile_.end(), [&](const KernelTime& k) { return k.name == p.name; });
+    if (it == profile_.end()) {
+      profile_.push_back(KernelTime{p.name, 0.0, 0, 0.0, 0.0});
+      it = profile_.end() - 1;
+    }
+    it->ms += ms;
+    it->launches += 1;
+    it->flops += p.flops;
+    it->bytes += p.bytes;
+    event_pool_.push_back(p.start);
+    event_pool_.push_back(p.stop);
+  }
+  pending_.clear();
+}
+
+std::vector<KernelTime> Mi355xNetwork::TakeProfile() {
+  std::lock_guard<std::mutex> lock(eval_mutex_);
+  std::vector<KernelTime> out;
+  out.swap(profile_);
+  return out;
+}
+
+Linear Mi355xNetwork::MakeLinear(const Vec& w, const Vec& b, int out, int in) {
+  if (static_cast<size_t>(out) * in != w.size()) {
+    throw Error("Weight tensor has " + std::to_string(w.size()) + " elements, expected " + std::to_string(out) +
+                " x " + std::to_string(in) + ".");
+  }
+  if (!b.empty() && static_cast<int>(b.size()) != out) throw Error("Bias size does not match the layer width.");
+  Linear l;
+  l.out = out;
+  l.in = in;
+  l.ld = RoundUp(in, 8);
+  std::vector<half_t> h(static_cast<size_t>(out) * l.ld, (half_t)0.0f);
+  for (int o = 0; o < out; o++)
+    for (int i = 0; i < in; i++) h[static_cast<size_t>(o) * l.ld + i] = (half_t)w[static_cast<size_t>(o) * in + i];
+  l.w = arena_.Upload(h);
+  if (!b.empty()) l.b = arena_.Upload(b);
+  return l;
+}
+
+void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M,
+                         int act, bool out_f32) {
+  GemmArgs g;
+  g.A = A; g.lda = lda;
+  g.W = lin.w; g.ldw = lin.ld;
+  g.C = C; g.ldc = ldc;
+  g.bias = lin.b;
+  g.M = M; g.N = lin.out; g.K = lin.ld;
+  g.act = act;
+  g.out_f32 = out_f32;
+  const double flops = 2.0 * M * lin.out * lin.in;
+  const double bytes = 2.0 * (static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in) +
+                       static_cast<double>(M) * lin.out * (out_f32 ? 4 : 2);
+  Timed(name, flops, bytes, [&] { LaunchGemm(g, stream_); });
+}
+
+// ------------------------------------------------------------- construction --
+Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
+  const NetworkFormat& nf = file.format;
+  caps_.input_format = nf.input;
+  caps_.output_format = nf.output;
+  caps_.moves_left = nf.moves_left;
+
+  device_ = options.GetInt("gpu", 0);
+  max_batch_ = options.GetInt("max_batch", 1024);
+  if (max_batch_ < 1 || max_batch_ > 4096) throw Error("max_batch must be in 1..4096.");
+  const std::string precision = options.GetString("precision", "fp16");
+  if (precision != "fp16") throw Error("Precision '" + precision + "' is not supported (fp16 only).");
+  policy_head_ = options.GetString("policy_head", "vanilla");
+  value_head_ = options.GetString("value_head", "winner");
+  wdl_ = nf.value == kValueWdl;
+  moves_left_ = nf.moves_left == kMovesLeftV1 && options.GetBool("mlh", true);
+  conv_policy_ = nf.policy == kPolicyConvolution;
+  attn_policy_ = nf.policy == kPolicyAttention;
+  attn_body_ = nf.network == kNetworkAttentionBodyWithHeadformat ||
+               nf.network == kNetworkAttentionBodyWithMultiheadformat;
+  default_act_ = nf.default_activation == 1 ? kActMish : kActRelu;
+  if (attn_body_) {
+    smolgen_act_ = nf.smolgen_activation == kActDefault ? default_act_ : nf.smolgen_activation;
+    ffn_act_ = nf.ffn_activation == kActDefault ? default_act_ : nf.ffn_activation;
+  }
+  if (file.weights.policy_heads.count(policy_head_) == 0) {
+    throw Error("The policy head you specified '" + policy_head_ + "' does not exist in this net.");
+  }
+  if (file.weights.value_heads.count(value_head_) == 0) {
+    throw Error("The value head you specified '" + value_head_ + "' does not exist in this net.");
+  }
+
+  int count = 0;
+  hipError_t err = hipGetDeviceCount(&count);
+  if (err != hipSuccess || count == 0) {
+    throw Error("No HIP device is available: the mi355x backend needs a GPU (there is no CPU fallback).");
+  }
+  if (device_ < 0 || device_ >= count) throw Error("Invalid GPU id " + std::to_string(device_) + ".");
+  HIP_CHECK(hipSetDevice(device_));
+  HIP_CHECK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+
+  d_masks_ = static_cast<uint64_t*>(arena_.Alloc(sizeof(uint64_t) * kInputPlanes * max_batch_));
+  d_values_ = AllocF(static_cast<size_t>(kInputPlanes) * max_batch_);
+  d_policy_ = AllocF(static_cast<size_t>(kPolicyOutputs) * max_batch_);
+  d_wdl_ = AllocF(3 * static_cast<size_t>(max_batch_));
+  d_mlh_ = AllocF(max_batch_);
+
+  if (attn_body_) {
+    BuildAttentionBody(file);
+  } else {
+    throw Error("Only attention-body networks are supported by this build of the mi355x backend.");
+  }
+  HIP_CHECK(hipStreamSynchronize(stream_));
+}
+
+Mi355xNetwork::~Mi355xNetwork() {
+  if (stream_) {
+    (void)hipStreamSynchronize(stream_);
+    for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
+    (void)hipStreamDestroy(stream_);
+  }
+}
+
+void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
+  const NetWeights& w = file.weights;
+  const NetworkFormat& nf = file.format;
+  if (!w.residual.empty()) throw Error("Attention body on top of a residual tower is not supported.");
+  if (nf.input_embedding != kInputEmbeddingPeMap) {
+    throw Error("Only the PE_MAP input embedding is supported by the mi355x backend.");
+  }
+  if (!w.ip_mult_gate.empty() || !w.ip_add_gate.empty()) throw Error("Input gating is not supported.");
+  if (!attn_policy_) throw Error("Attention-body networks need the attention policy head.");
+  const PolicyHead& ph = w.policy_heads.at(policy_head_);
+  const ValueHead& vh = w.value_heads.at(value_head_);
+  if (!ph.pol_encoder.empty()) throw Error("Policy encoder layers are not supported.");
+
+  emb_ = static_cast<int>(w.ip_emb_b.size());
+  heads_ = w.encoder_head_count;
+  if (emb_ <= 0 || emb_ % 8 != 0 || emb_ > 8192) throw Error("Embedding size must be a multiple of 8 in 8..8192.");
+  if (w.encoder.empty() || heads_ <= 0) throw Error("Attention body without encoder layers.");
+  d_model_ = static_cast<int>(w.encoder[0].mha.q_b.size());
+  dff_ = static_cast<int>(w.encoder[0].ffn.dense1_b.size());
+  if (d_model_ != heads_ * 32) throw Error("Only attention heads of depth 32 are supported.");
+  if (dff_ % 8 != 0) throw Error("FFN width must be a multiple of 8.");
+  alpha_ = static_cast<float>(std::pow(2.0 * w.encoder.size(), -0.25));
+  eps_ = 1e-6f;
+
+  emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + 64);
+  in_ld_ = emb_lin_.ld;
+  {
+    const std::vector<float>& pe = PosEncoding();
+    std::vector<half_t> h(pe.size());
+    for (size_t i = 0; i < pe.size(); i++) h[i] = (half_t)pe[i];
+    pos_enc_ = arena_.Upload(h);
+  }
+
+  for (const EncoderLayer& l : w.encoder) {
+    EncoderDev e;
+    if (static_cast<int>(l.mha.q_b.size()) != d_model_ || static_cast<int>(l.ffn.dense1_b.size()) != dff_) {
+      throw Error("Encoder layers of different sizes are not supported.");
+    }
+    Vec qkv_w, qkv_b;
+    qkv_w.reserve(3 * l.mha.q_w.size());
+    for (const Vec* v : {&l.mha.q_w, &l.mha.k_w, &l.mha.v_w}) qkv_w.insert(qkv_w.end(), v->begin(), v->end());
+    for (const Vec* v : {&l.mha.q_b, &l.mha.k_b, &l.mha.v_b}) qkv_b.insert(qkv_b.end(), v->begin(), v->end());
+    e.qkv = MakeLinear(qkv_w, qkv_b, 3 * d_model_, emb_);
+    e.dense = MakeLinear(l.mha.dense_w, l.mha.dense_b, emb_, d_model_);
+    e.ffn1 = MakeLinear(l.ffn.dense1_w, l.ffn.dense1_b, dff_, emb_);
+    e.ffn2 = MakeLinear(l.ffn.dense2_w, l.ffn.dense2_b, emb_, dff_);
+    e.ln1_g = UploadF(l.ln1_gammas); e.ln1_b = UploadF(l.ln1_betas);
+    e.ln2_g = UploadF(l.ln2_gammas); e.ln2_b = UploadF(l.ln2_betas);
+    if (static_cast<int>(l.ln1_gammas.size()) != emb_ || static_cast<int>(l.ln2_gammas.size()) != emb_) {
+      throw Error("Layer norm parameters do not match the embedding size.");
+    }
+    e.has_smolgen = l.mha.has_smolgen;
+    if (e.has_smolgen) {
+      const Smolgen& s = l.mha.smolgen;
+      const int hc = static_cast<int>(s.compress.size()) / emb_;
+      const int hs = static_cast<int>(s.dense1_b.size());
+      const int gen = static_cast<int>(s.dense2_b.size());
+      if (!any_smolgen_) {
+        sg_hc_ = hc; sg_hs_ = hs; sg_gen_ = gen;
+      } else if (hc != sg_hc_ || hs != sg_hs_ || gen != sg_gen_) {
+        throw Error("Smolgen layers of different sizes are not supported.");
+      }
+      any_smolgen_ = true;
+      if (hc % 8 || hs % 8 || gen % heads_ || (gen / heads_) % 8 || hs > 8192 || gen > 8192) {
+        throw Error("Unsupported smolgen sizes.");
+      }
+      e.sg_compress = MakeLinear(s.compress, Vec(), hc, emb_);
+      e.sg_dense1 = MakeLinear(s.dense1_w, s.dense1_b, hs, 64 * hc);
+      e.sg_dense2 = MakeLinear(s.dense2_w, s.dense2_b, gen, hs);
+      e.sg_ln1_g = UploadF(s.ln1_gammas); e.sg_ln1_b = UploadF(s.ln1_betas);
+      e.sg_ln2_g = UploadF(s.ln2_gammas); e.sg_ln2_b = UploadF(s.ln2_betas);
+    }
+    encoders_.push_back(e);
+  }
+  if (any_smolgen_) {
+    const int g = sg_gen_ / heads_;
+    if (w.smolgen_w.size() != static_cast<size_t>(4096) * g) throw Error("Global smolgen weights have a wrong size.");
+    // Rows permuted so that the generated logits come out in the layout the
+    // attention kernel reads with one 16-byte load per lane.
+    Vec perm(w.smolgen_w.size());
+    for (int q = 0; q < 64; q++)
+      for (int k = 0; k < 64; k++)
+        std::memcpy(&perm[static_cast<size_t>(SmolgenBiasIndex(q, k)) * g], &w.smolgen_w[static_cast<size_t>(q * 64 + k) * g],
+                    sizeof(float) * g);
+    smolgen_w_ = MakeLinear(perm, Vec(), 4096, g);
+  }
+
+  // Heads.
+  pol_emb_ = static_cast<int>(ph.ip_pol_b.size());
+  pol_d_ = static_cast<int>(ph.ip2_pol_b.size());
+  if (pol_emb_ % 8 || pol_d_ % 8 || pol_d_ <= 0) throw Error("Unsupported policy head sizes.");
+  pol_emb_lin_ = MakeLinear(ph.ip_pol_w, ph.ip_pol_b, pol_emb_, emb_);
+  {
+    Vec qk_w(ph.ip2_pol_w), qk_b(ph.ip2_pol_b);
+    qk_w.insert(qk_w.end(), ph.ip3_pol_w.begin(), ph.ip3_pol_w.end());
+    qk_b.insert(qk_b.end(), ph.ip3_pol_b.begin(), ph.ip3_pol_b.end());
+    pol_qk_lin_ = MakeLinear(qk_w, qk_b, 2 * pol_d_, pol_emb_);
+  }
+  if (ph.ip4_pol_w.size() != static_cast<size_t>(4) * pol_d_) throw Error("Promotion weights have a wrong size.");
+  ppo_ = UploadF(ph.ip4_pol_w);
+  inv_map_ = arena_.Upload(AttnPolicyInverseMap());
+
+  val_ch_ = static_cast<int>(vh.ip_val_b.size());
+  val_fc_ = static_cast<int>(vh.ip1_val_b.size());
+  val_out_ = wdl_ ? 3 : 1;
+  if (val_ch_ % 8 || val_fc_ % 8) throw Error("Unsupported value head sizes.");
+  val_emb_lin_ = MakeLinear(vh.ip_val_w, vh.ip_val_b, val_ch_, emb_);
+  val_fc1_ = MakeLinear(vh.ip1_val_w, vh.ip1_val_b, val_fc_, 64 * val_ch_);
+  val_fc2_ = MakeLinear(vh.ip2_val_w, vh.ip2_val_b, val_out_, val_fc_);
+  if (moves_left_) {
+    mov_ch_ = static_cast<int>(w.ip_mov_b.size());
+    mov_fc_ = static_cast<int>(w.ip1_mov_b.size());
+    if (mov_ch_ % 8 || mov_fc_ % 8) throw Error("Unsupported moves-left head sizes.");
+    mov_emb_lin_ = MakeLinear(w.ip_mov_w, w.ip_mov_b, mov_ch_, emb_);
+    mov_fc1_ = MakeLinear(w.ip1_mov_w, w.ip1_mov_b, mov_fc_, 64 * mov_ch_);
+    mov_fc2_ = MakeLinear(w.ip2_mov_w, w.ip2_mov_b, 1, mov_fc_);
+  }
+
+  // Activations.
+  const size_t T = static_cast<size_t>(max_batch_) * 64;
+  in0_ = AllocH(T * in_ld_);
+  x_ = AllocH(T * emb_);
+  t_ = AllocH(T * emb_);
+  qkv_ = AllocH(T * 3 * d_model_);
+  att_ = AllocH(T * d_model_);
+  ffn_ = AllocH(T * dff_);
+  if (any_smolgen_) {
+    sg1_ = AllocH(T * sg_hc_);
+    sg2_ = AllocH(static_cast<size_t>(max_batch_) * sg_hs_);
+    sg3_ = AllocH(static_cast<size_t>(max_batch_) * sg_gen_);
+    sbias_ = AllocH(static_cast<size_t>(max_batch_) * heads_ * 4096);
+  }
+  pol_e_ = AllocH(T * pol_emb_);
+  pol_qk_ = AllocH(T * 2 * pol_d_);
+  pol_logits_ = AllocF(static_cast<size_t>(max_batch_) * 4096);
+  head1_ = AllocH(T * std::max(val_ch_, mov_ch_));
+  head2_ = AllocH(static_cast<size_t>(max_batch_) * std::max(val_fc_, mov_fc_));
+}
+
+// ------------------------------------------------------------------ forward --
+void Mi355xNetwork::ForwardAttentionBody(int B) {
+  const int T = B * 64;
+  Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * 2),
+        [&] { LaunchExpandPlanesAttn<half_t>(d_masks_, d_values_, pos_enc_, in0_, in_ld_, B, stream_); });
+  Gemm("gemm_embedding", in0_, in_ld_, emb_lin_, x_, emb_, T, default_act_);
+
+  for (const EncoderDev& e : encoders_) {
+    const half_t* bias = nullptr;
+    if (e.has_smolgen) {
+      const int g = sg_gen_ / heads_;
+      Gemm("gemm_smolgen_compress", x_, emb_, e.sg_compress, sg1_, sg_hc_, T, kActNone);
+      Gemm("gemm_smolgen_dense1", sg1_, 64 * sg_hc_, e.sg_dense1, sg2_, sg_hs_, B, smolgen_act_);
+      Timed("layer_norm_smolgen", 0.0, 4.0 * B * sg_hs_, [&] {
+        LaunchLayerNorm(sg2_, nullptr, sg2_, e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f, 1e-3f, stream_);
+      });
+      Gemm("gemm_smolgen_dense2", sg2_, sg_hs_, e.sg_dense2, sg3_, sg_gen_, B, smolgen_act_);
+      Timed("layer_norm_smolgen", 0.0, 4.0 * B * sg_gen_, [&] {
+        LaunchLayerNorm(sg3_, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f, 1e-3f, stream_);
+      });
+      Gemm("gemm_smolgen_global", sg3_, g, smolgen_w_, sbias_, 4096, B * heads_, kActNone);
+      bias = sbias_;
+    }
+    Gemm("gemm_qkv", x_, emb_, e.qkv, qkv_, 3 * d_model_, T, kActNone);
+    Timed("attention", 4.0 * 2 * 64 * 64 * 32 * B * heads_ / 2.0,
+          B * heads_ * (2.0 * (3 * 64 * 32 + 64 * 32) + (bias ? 2.0 * 4096 : 0.0)),
+          [&] { LaunchAttention(qkv_, bias, att_, B, heads_, 1.0f / std::sqrt(32.0f), stream_); });
+    Gemm("gemm_mha_dense", att_, d_model_, e.dense, t_, emb_, T, kActNone);
+    Timed("layer_norm_skip", 0.0, 6.0 * T * emb_, [&] {
+      LaunchLayerNorm(t_, x_, x_, e.ln1_g, e.ln1_b, T, emb_, alpha_, eps_, stream_);
+    });
+    Gemm("gemm_ffn1", x_, emb_, e.ffn1, ffn_, dff_, T, ffn_act_);
+    Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, t_, emb_, T, kActNone);
+    Timed("layer_norm_skip", 0.0, 6.0 * T * emb_, [&] {
+      LaunchLayerNorm(t_, x_, x_, e.ln2_g, e.ln2_b, T, emb_, alpha_, eps_, stream_);
+    });
+  }
+
+  // Value head.
+  Gemm("gemm_value_embed", x_, emb_, val_emb_lin_, head1_, val_ch_, T, default_act_);
+  Gemm("gemm_value_fc1", head1_, 64 * val_ch_, val_fc1_, head2_, val_fc_, B, default_act_);
+  Gemm("gemm_value_fc2", head2_, val_fc_, val_fc2_, d_wdl_, val_out_, B, kActNone, /*out_f32=*/true);
+  // Moves-left head.
+  if (moves_left_) {
+    Gemm("gemm_mlh_embed", x_, emb_, mov_emb_lin_, head1_, mov_ch_, T, default_act_);
+    Gemm("gemm_mlh_fc1", head1_, 64 * mov_ch_, mov_fc1_, head2_, mov_fc_, B, default_act_);
+    Gemm("gemm_mlh_fc2", head2_, mov_fc_, mov_fc2_, d_mlh_, 1, B, kActRelu, /*out_f32=*/true);
+  }
+  // Policy head.
+  Gemm("gemm_policy_embed", x_, emb_, pol_emb_lin_, pol_e_, pol_emb_, T, default_act_);
+  Gemm("gemm_policy_qk", pol_e_, pol_emb_, pol_qk_lin_, pol_qk_, 2 * pol_d_, T, kActNone);
+  {
+    GemmArgs g;
+    g.A = pol_qk_; g.lda = 2 * pol_d_; g.strideA = 64LL * 2 * pol_d_;
+    g.W = pol_qk_ + pol_d_; g.ldw = 2 * pol_d_; g.strideW = 64LL * 2 * pol_d_;
+    g.C = pol_logits_; g.ldc = 64; g.strideC = 4096;
+    g.M = 64; g.N = 64; g.K = pol_d_; g.batch = B;
+    g.scale = 1.0f / std::sqrt(static_cast<float>(pol_d_));
+    g.act = kActNone;
+    g.out_f32 = true;
+    Timed("gemm_policy_logits", 2.0 * 64 * 64 * pol_d_ * B, B * (2.0 * 2 * 64 * pol_d_ + 4.0 * 4096),
+          [&] { LaunchGemm(g, stream_); });
+  }
+  Timed("policy_gather", 0.0, B * (4.0 * 4288 + 4.0 * 1858), [&] {
+    LaunchAttnPolicyGather(pol_logits_, pol_qk_, 2 * pol_d_, pol_d_, ppo_, pol_d_, inv_map_, d_policy_, B, stream_);
+  });
+}
+
+void Mi355xNetwork::ForwardDevice(int batch) {
+  if (attn_body_) ForwardAttentionBody(batch);
+}
+
+void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {
+  if (batch <= 0) return;
+  std::lock_guard<std::mutex> lock(eval_mutex_);
+  HIP_CHECK(hipSetDevice(device_));
+  HIP_CHECK(hipMemcpyAsync(d_masks_, slot->masks, sizeof(uint64_t) * kInputPlanes * batch, hipMemcpyHostToDevice,
+                           stream_));
+  HIP_CHECK(hipMemcpyAsync(d_values_, slot->values, sizeof(float) * kInputPlanes * batch, hipMemcpyHostToDevice,
+                           stream_));
+  ForwardDevice(batch);
+  HIP_CHECK(hipGetLastError());
+  HIP_CHECK(hipMemcpyAsync(slot->policy, d_policy_, sizeof(float) * kPolicyOutputs * batch, hipMemcpyDeviceToHost,
+                           stream_));
+  HIP_CHECK(hipMemcpyAsync(slot->wdl, d_wdl_, sizeof(float) * (wdl_ ? 3 : 1) * batch, hipMemcpyDeviceToHost,
+                           stream_));
+  if (moves_left_) {
+    HIP_CHECK(hipMemcpyAsync(slot->mlh, d_mlh_, sizeof(float) * batch, hipMemcpyDeviceToHost, stream_));
+  }
+  HIP_CHECK(hipStreamSynchronize(stream_));
+  if (profiling_) CollectPending();
+  // Value post-processing on the host (3 numbers per sample).
+  for (int i = 0; i < batch; i++) {
+    if (wdl_) {
+      float* v = slot->wdl + 3 * i;
+      float m = std::max(v[0], std::max(v[1], v[2]));
+      float e0 = std::exp(v[0] - m), e1 = std::exp(v[1] - m), e2 = std::exp(v[2] - m);
+      float s = e0 + e1 + e2;
+      v[0] = e0 / s; v[1] = e1 / s; v[2] = e2 / s;
+    } else {
+      slot->wdl[i] = std::tanh(slot->wdl[i]);
+    }
+  }
+}
+
+double Mi355xNetwork::TimeResidentForward(int batch, int iters) {
+  if (batch < 1 || batch > max_batch_) throw Error("batch out of range");
+  if (iters < 1) throw Error("iters must be positive");
+  std::lock_guard<std::mutex> lock(eval_mutex_);
+  HIP_CHECK(hipSetDevice(device_));
+  const bool was_profiling = profiling_;
+  profiling_ = false;
+  hipEvent_t start = NewEvent(), stop = NewEvent();
+  HIP_CHECK(hipEventRecord(start, stream_));
+  for (int i = 0; i < iters; i++) ForwardDevice(batch);
+  HIP_CHECK(hipEventRecord(stop, stream_));
+  HIP_CHECK(hipStreamSynchronize(stream_));
+  HIP_CHECK(hipGetLastError());
+  float ms = 0.0f;
+  HIP_CHECK(hipEventElapsedTime(&ms, start, stop));
+  event_pool_.push_back(start);
+  event_pool_.push_back(stop);
+  profiling_ = was_profiling;
+  return ms / iters;
+}
+
+std::unique_ptr<HostSlot> Mi355xNetwork::GetSlot() {
+  {
+    std::lock_guard<std::mutex> lock(slots_mutex_);
+    if (!free_slots_.empty()) {
+      auto s = std::move(free_slots_.back());
+      free_slots_.pop_back();
+      return s;
+    }
+  }
+  HIP_CHECK(hipSetDevice(device_));
+  auto s = std::make_unique<HostSlot>();
+  s->capacity = max_batch_;
+  HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&s->masks), sizeof(uint64_t) * kInputPlanes * max_batch_));
+  HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&s->values), sizeof(float) * kInputPlanes * max_batch_));
+  HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&s->policy), sizeof(float) * kPolicyOutputs * max_batch_));
+  HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&s->wdl), sizeof(float) * 3 * max_batch_));
+  HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&s->mlh), sizeof(float) * max_batch_));
+  return s;
+}
+
+void Mi355xNetwork::ReleaseSlot(std::unique_ptr<HostSlot> slot) {
+  std::lock_guard<std::mutex> lock(slots_mutex_);
+  free_slots_.push_back(std::move(slot));
+}
+
+// -------------------------------------------------------------- computation --
+Mi355xComputation::~Mi355xComputation() {
+  for (auto& s : slots_) net_->ReleaseSlot(std::move(s));
+}
+
+HostSlot* Mi355xComputation::SlotFor(int index) {
+  const int cap = net_->GetMaxBatchSize();
+  const size_t si = static_cast<size_t>(index / cap);
+  while (slots_.size() <= si) slots_.push_back(net_->GetSlot());
+  return slots_[si].get();
+}
+
+void Mi355xComputation::AddInput(InputPlanes&& input) {
+  if (input.size() != static_cast<size_t>(kInputPlanes)) {
+    throw Error("AddInput expects exactly 112 input planes, got " + std::to_string(input.size()) + ".");
+  }
+  HostSlot* s = SlotFor(batch_);
+  const int at = batch_ % net_->GetMaxBatchSize();
+  uint64_t* m = s->masks + static_cast<size_t>(at) * kInputPlanes;
+  float* v = s->values + static_cast<size_t>(at) * kInputPlanes;
+  for (int i = 0; i < kInputPlanes; i++) {
+    m[i] = input[i].mask;
+    v[i] = input[i].value;
+  }
+  batch_++;
+  computed_ = false;
+}
+
+void Mi355xComputation::AddInputs(int n, const uint64_t* masks, const float* values) {
+  if (n < 0) throw Error("negative input count");
+  for (int i = 0; i < n; i++) {
+    HostSlot* s = SlotFor(batch_);
+    const int at = batch_ % net_->GetMaxBatchSize();
+    std::memcpy(s->masks + static_cast<size_t>(at) * kInputPlanes, masks + static_cast<size_t>(i) * kInputPlanes,
+                sizeof(uint64_t) * kInputPlanes);
+    std::memcpy(s->values + static_cast<size_t>(at) * kInputPlanes, values + static_cast<size_t>(i) * kInputPlanes,
+                sizeof(float) * kInputPlanes);
+    batch_++;
+  }
+  computed_ = false;
+}
+
+void Mi355xComputation::ComputeBlocking() {
+  const int cap = net_->GetMaxBatchSize();
+  for (size_t si = 0; si < slots_.size(); si++) {
+    const int n = std::min(cap, batch_ - static_cast<int>(si) * cap);
+    net_->Evaluate(slots_[si].get(), n);
+  }
+  computed_ = true;
+}
+
+const float* Mi355xComputation::GetPolicyRow(int sample) const {
+  CheckSample(sample);
+  const int cap = net_->GetMaxBatchSize();
+  return slots_[sample / cap]->policy + static_cast<size_t>(sample % cap) * kPolicyOutputs;
+}
+
+float Mi355xComputation::GetQVal(int sample) const {
+  CheckSample(sample);
+  const int cap = net_->GetMaxBatchSize();
+  const float* w = slots_[sample / cap]->wdl;
+  if (net_->wdl()) return w[3 * (sample % cap)] - w[3 * (sample % cap) + 2];
+  return w[sample % cap];
+}
+
+float Mi355xComputation::GetDVal(int sample) const {
+  CheckSample(sample);
+  if (!net_->wdl()) return 0.0f;
+  const int cap = net_->GetMaxBatchSize();
+  return slots_[sample / cap]->wdl[3 * (sample % cap) + 1];
+}
+
+float Mi355xComputation::GetMVal(int sample) const {
+  CheckSample(sample);
+  if (!net_->moves_left()) return 0.0f;
+  const int cap = net_->GetMaxBatchSize();
+  return slots_[sample / cap]->mlh[sample % cap];
+}
+
+}  // namespace
+
+std::unique_ptr<Network> MakeMi355xNetwork(const WeightsFile& weights, Options& options) {
+  const NetworkFormat& nf = weights.format;
+  switch (nf.network) {
+    case kNetworkClassicalWithHeadformat:
+    case kNetworkSeWithHeadformat:
+    case kNetworkAttentionBodyWithHeadformat:
+    case kNetworkAttentionBodyWithMultiheadformat:
+      break;
+    default:
+      throw Error("Network format " + std::to_string(nf.network) + " is not supported by the mi355x backend.");
+  }
+  if (nf.policy != kPolicyClassical && nf.policy != kPolicyConvolution && nf.policy != kPolicyAttention) {
+    throw Error("Policy format " + std::to_string(nf.policy) + " is not supported by the mi355x backend.");
+  }
+  if (nf.value != kValueClassical && nf.value != kValueWdl) {
+    throw Error("Value format " + std::to_string(nf.value) + " is not supported by the mi355x backend.");
+  }
+  if (nf.moves_left != kMovesLeftNone && nf.moves_left != kMovesLeftV1) {
+    throw Error("Moves left head format " + std::to_string(nf.moves_left) + " is not supported by the mi355x backend.");
+  }
+  if (nf.default_activation != 0 && nf.default_activation != 1) {
+    throw Error("Default activation " + std::to_string(nf.default_activation) + " is not supported by the mi355x backend.");
+  }
+  if (nf.input_embedding != kInputEmbeddingNone && nf.input_embedding != kInputEmbeddingPeMap &&
+      nf.input_embedding != kInputEmbeddingPeDense) {
+    throw Error("Input embedding " + std::to_string(nf.input_embedding) + " is not supported by the mi355x backend.");
+  }
+  auto net = std::make_unique<Mi355xNetwork>(weights, options);
+  options.CheckAllOptionsRead("mi355x");
+  return net;
+}
+
+}  // namespace lc0mi

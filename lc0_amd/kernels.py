@@ -1,0 +1,121 @@
+"""numpy front end of the single-kernel entry points (include/lc0mi_kernels.h).
+
+Each function runs exactly one gfx950 kernel of the forward pass on host
+arrays; used by the per-kernel parity tests and micro-benchmarks.
+"""
+import ctypes as C
+
+import numpy as np
+
+from .backend import BackendError, load_library
+
+ACT_MISH, ACT_RELU, ACT_NONE, ACT_TANH, ACT_SIGMOID, ACT_SELU, ACT_SWISH, ACT_RELU_2 = 1, 2, 3, 4, 5, 6, 7, 8
+
+
+def _lib():
+    lib = load_library()
+    if not getattr(lib, "_k_ready", False):
+        vp, ci, ll, cf, cd = C.c_void_p, C.c_int, C.c_longlong, C.c_float, C.POINTER(C.c_double)
+        lib.lc0mi_k_gemm.argtypes = [vp, ci, ll, vp, ci, ll, vp, ci, ci, ci, ci, cf, ci, ci, vp, ci, ll, ci, cd]
+        lib.lc0mi_k_gemm_f32.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, ci, vp, ci]
+        lib.lc0mi_k_layer_norm.argtypes = [vp, vp, vp, vp, ci, ci, cf, cf, vp, ci, cd]
+        lib.lc0mi_k_attention.argtypes = [vp, vp, ci, ci, cf, vp, ci, cd]
+        lib.lc0mi_k_expand_planes_attn.argtypes = [vp, vp, ci, ci, vp, ci, cd]
+        lib.lc0mi_k_expand_planes_nchw.argtypes = [vp, vp, ci, vp]
+        lib.lc0mi_k_attn_policy_gather.argtypes = [vp, vp, vp, ci, ci, vp]
+        lib._k_ready = True
+    return lib
+
+
+def _check(rc):
+    if rc:
+        raise BackendError(load_library().lc0mi_last_error().decode(errors="replace"))
+
+
+def _h(a):
+    return np.ascontiguousarray(a, dtype=np.float16)
+
+
+def _ptr(a):
+    return a.ctypes.data if a is not None else None
+
+
+def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
+    """a [batch?, M, K], w [batch?, N, K] (any float dtype, rounded to fp16) ->
+    act(scale * a @ w^T + bias). Returns (C, ms) if time_iters else C."""
+    a, w = _h(a), _h(w)
+    batched = a.ndim == 3
+    if not batched:
+        a, w = a[None], w[None]
+    batch, m, k = a.shape
+    n = w.shape[1]
+    out = np.zeros((batch, m, n), np.float32 if out_f32 else np.float16)
+    b = np.ascontiguousarray(bias, np.float32) if bias is not None else None
+    ms = C.c_double(0)
+    _check(_lib().lc0mi_k_gemm(_ptr(a), k, m * k, _ptr(w), k, n * k, _ptr(b), m, n, k, batch, scale, act,
+                               int(out_f32), _ptr(out), n, m * n, time_iters, C.byref(ms)))
+    out = out if batched else out[0]
+    return (out, ms.value) if time_iters else out
+
+
+def gemm_f32(a, w, bias=None, scale=1.0, act=ACT_NONE):
+    a = np.ascontiguousarray(a, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    m, k = a.shape
+    n = w.shape[0]
+    out = np.zeros((m, n), np.float32)
+    b = np.ascontiguousarray(bias, np.float32) if bias is not None else None
+    _check(_lib().lc0mi_k_gemm_f32(_ptr(a), k, _ptr(w), k, _ptr(b), m, n, k, scale, act, _ptr(out), n))
+    return out
+
+
+def layer_norm(x, skip, gamma, beta, alpha, eps, time_iters=0):
+    x = _h(x)
+    s = _h(skip) if skip is not None else None
+    g = np.ascontiguousarray(gamma, np.float32)
+    b = np.ascontiguousarray(beta, np.float32)
+    y = np.zeros_like(x)
+    ms = C.c_double(0)
+    _check(_lib().lc0mi_k_layer_norm(_ptr(x), _ptr(s), _ptr(g), _ptr(b), x.shape[0], x.shape[1], alpha, eps,
+                                     _ptr(y), time_iters, C.byref(ms)))
+    return (y, ms.value) if time_iters else y
+
+
+def attention(qkv, bias, batch, heads, scale, time_iters=0):
+    """qkv [B*64, 3*heads*32], bias [B, heads, 64, 64] or None -> [B*64, heads*32]."""
+    qkv = _h(qkv)
+    b = _h(bias) if bias is not None else None
+    out = np.zeros((batch * 64, heads * 32), np.float16)
+    ms = C.c_double(0)
+    _check(_lib().lc0mi_k_attention(_ptr(qkv), _ptr(b), batch, heads, scale, _ptr(out), time_iters, C.byref(ms)))
+    return (out, ms.value) if time_iters else out
+
+
+def expand_planes_attn(masks, values, ld=176, time_iters=0):
+    masks = np.ascontiguousarray(masks, np.uint64)
+    values = np.ascontiguousarray(values, np.float32)
+    n = masks.shape[0]
+    out = np.zeros((n * 64, ld), np.float16)
+    ms = C.c_double(0)
+    _check(_lib().lc0mi_k_expand_planes_attn(_ptr(masks), _ptr(values), n, ld, _ptr(out), time_iters, C.byref(ms)))
+    return (out, ms.value) if time_iters else out
+
+
+def expand_planes_nchw(masks, values):
+    masks = np.ascontiguousarray(masks, np.uint64)
+    values = np.ascontiguousarray(values, np.float32)
+    n = masks.shape[0]
+    out = np.zeros((n, 112, 64), np.float32)
+    _check(_lib().lc0mi_k_expand_planes_nchw(_ptr(masks), _ptr(values), n, _ptr(out)))
+    return out
+
+
+def attn_policy_gather(logits, keys, ppo):
+    """logits f32 [B,64,64], keys [B*64, pd], ppo f32 [4, pd] -> [B, 1858]."""
+    logits = np.ascontiguousarray(logits, np.float32)
+    keys = _h(keys)
+    ppo = np.ascontiguousarray(ppo, np.float32)
+    n = logits.shape[0]
+    out = np.zeros((n, 1858), np.float32)
+    _check(_lib().lc0mi_k_attn_policy_gather(_ptr(logits), _ptr(keys), _ptr(ppo), keys.shape[1], n, _ptr(out)))
+    return out

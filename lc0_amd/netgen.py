@@ -160,7 +160,7 @@ CONFIGS = {
     # tiny nets for fast parity tests
     "tiny_resnet": lambda: se_resnet(32, 2, 8, seed=2000, moves_left=True),
     "tiny_attn": lambda: attention_body(64, 2, 2, 96, seed=2001, smolgen=(8, 32, 32), perturb_ln=True),
-    "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 4, 128, seed=2002, perturb_ln=True),
+    "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True),
 }
 
 

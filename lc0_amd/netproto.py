@@ -174,7 +174,7 @@ def serialize_net(net, layer_encoding=FLOAT32):
     return encode_message("Net", full, layer_encoding)
 
 
-def write_pb_gz(path, net, layer_encoding=FLOAT32, compresslevel=1):
+def write_pb_gz(path, net, layer_encoding=FLOAT32, compresslevel=0):
     data = serialize_net(net, layer_encoding)
     with gzip.GzipFile(path, "wb", compresslevel=compresslevel, mtime=0) as f:
         f.write(data)

@@ -1,0 +1,127 @@
+"""Per-kernel parity on the GPU: each hand-written kernel, called through the C
+ABI (include/lc0mi_kernels.h), against the oracle function it replaces on the
+same seeded tensors. fp16 tolerances are stated per test."""
+import numpy as np
+import pytest
+
+from oracle import netread as nr
+from oracle import nn as onn
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+def _h(a):
+    """Round to fp16 and back: what the kernel actually sees."""
+    return np.asarray(a, np.float16).astype(f32)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 64, 64), (128, 128, 128), (192, 96, 176), (300, 3, 128), (7, 1858 // 2, 72),
+                                   (1024, 256, 1024), (5, 8, 16)])
+@pytest.mark.parametrize("act", [nr.ACT_NONE, nr.ACT_MISH, nr.ACT_SWISH, nr.ACT_RELU])
+def test_gemm_vs_oracle_fc(m, n, k, act):
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(m * 7 + n * 3 + k + act)
+    a = _h(rng.standard_normal((m, k)) * 0.5)
+    w = _h(rng.standard_normal((n, k)) * 0.2)
+    b = rng.standard_normal(n).astype(f32)
+    want = onn.fc(a, w.reshape(-1), b, act)
+    got = K.gemm(a, w, b, act=act, out_f32=True)
+    # fp16 operands, fp32 accumulation, fp32 output: only summation order differs.
+    np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
+    got16 = K.gemm(a, w, b, act=act).astype(f32)
+    np.testing.assert_allclose(got16, want, rtol=2e-3, atol=2e-3)  # + one fp16 rounding of the output
+
+
+def test_gemm_no_bias_scale_and_batched():
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(1)
+    a = _h(rng.standard_normal((5, 64, 96)))
+    w = _h(rng.standard_normal((5, 64, 96)))
+    got = K.gemm(a, w, None, scale=0.125, out_f32=True)
+    want = np.matmul(a, w.transpose(0, 2, 1)) * 0.125
+    np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
+
+
+def test_gemm_f32_vs_oracle_fc():
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(2)
+    for m, n, k in [(64, 64, 64), (70, 33, 20), (513, 130, 256)]:
+        a = rng.standard_normal((m, k)).astype(f32)
+        w = rng.standard_normal((n, k)).astype(f32)
+        b = rng.standard_normal(n).astype(f32)
+        np.testing.assert_allclose(K.gemm_f32(a, w, b, act=nr.ACT_MISH), onn.fc(a, w, b, nr.ACT_MISH),
+                                   rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("rows,c", [(64, 64), (300, 256), (128, 1024), (9, 8192), (5, 32)])
+@pytest.mark.parametrize("with_skip", [True, False])
+def test_layer_norm_vs_oracle(rows, c, with_skip):
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(rows + c)
+    x = _h(rng.standard_normal((rows, c)))
+    s = _h(rng.standard_normal((rows, c))) if with_skip else None
+    g = (1 + 0.1 * rng.standard_normal(c)).astype(f32)
+    b = (0.1 * rng.standard_normal(c)).astype(f32)
+    want = onn.layer_norm_skip(x, 0.427, s, g, b, 1e-6)
+    got = K.layer_norm(x, s, g, b, 0.427, 1e-6).astype(f32)
+    np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3)  # fp16 output rounding
+
+
+@pytest.mark.parametrize("batch,heads", [(1, 1), (3, 2), (5, 8), (2, 32)])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_attention_vs_oracle(batch, heads, with_bias):
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(batch * 100 + heads)
+    d = heads * 32
+    qkv = _h(rng.standard_normal((batch * 64, 3 * d)))
+    bias = _h(rng.standard_normal((batch, heads, 64, 64)) * 2) if with_bias else None
+    scale = 1.0 / np.sqrt(32.0)
+    got = K.attention(qkv, bias, batch, heads, scale).astype(f32)
+    q = qkv[:, :d].reshape(batch, 64, heads, 32).transpose(0, 2, 1, 3)
+    k = qkv[:, d:2 * d].reshape(batch, 64, heads, 32).transpose(0, 2, 1, 3)
+    v = qkv[:, 2 * d:].reshape(batch, 64, heads, 32).transpose(0, 2, 1, 3)
+    s = np.matmul(q, k.transpose(0, 1, 3, 2)) * f32(scale)
+    if bias is not None:
+        s = bias + s
+    p = onn.softmax_rows(s)
+    want = np.matmul(p, v).transpose(0, 2, 1, 3).reshape(batch * 64, d)
+    # probabilities are rounded to fp16 before P.V and the output is fp16.
+    np.testing.assert_allclose(got, want, rtol=4e-3, atol=4e-3)
+
+
+def test_expand_planes_bit_exact():
+    from lc0_amd import kernels as K
+    from oracle import chess as oc
+    pos = oc.random_positions(33, seed=5)
+    want = onn.encode_planes(pos["masks"], pos["values"])           # [B,112,64]
+    got_nchw = K.expand_planes_nchw(pos["masks"], pos["values"])
+    assert np.array_equal(got_nchw, want)
+    got = K.expand_planes_attn(pos["masks"], pos["values"], 176).astype(f32).reshape(33, 64, 176)
+    assert np.array_equal(got[:, :, :112], want.transpose(0, 2, 1))  # values <= 99 are exact in fp16
+    assert np.array_equal(got[:, :, 112:176], np.broadcast_to(onn.POS_ENCODING, (33, 64, 64)))
+    got_pad = K.expand_planes_attn(pos["masks"], pos["values"], 192).astype(f32).reshape(33, 64, 192)
+    assert np.array_equal(got_pad[:, :, :176], got) and (got_pad[:, :, 176:] == 0).all()
+
+
+def test_attn_policy_gather_vs_oracle():
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(3)
+    B, pd = 4, 64
+    logits = rng.standard_normal((B, 64, 64)).astype(f32)
+    keys = _h(rng.standard_normal((B * 64, pd)))
+    ppo = rng.standard_normal((4, pd)).astype(f32)
+    got = K.attn_policy_gather(logits, keys, ppo)
+    k3 = keys.reshape(B, 64, pd)
+    off = np.einsum("bjk,ik->bij", k3[:, 56:64], ppo)
+    off3 = off[:, :3] + off[:, 3:4]
+    promo = logits[:, 48:56, 56:64][:, :, :, None] + off3.transpose(0, 2, 1)[:, None]
+    buf = np.concatenate([logits.reshape(B, 4096), promo.reshape(B, 192)], axis=1)
+    want = np.zeros((B, 1858), f32)
+    sel = onn.ATTN_POLICY_MAP >= 0
+    want[:, onn.ATTN_POLICY_MAP[sel]] = buf[:, sel]
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+    # plain from->to logits are moved bit-exactly
+    plain = onn.ATTN_POLICY_MAP[:4096]
+    ps = plain >= 0
+    assert np.array_equal(got[:, plain[ps]], logits.reshape(B, 4096)[:, ps])

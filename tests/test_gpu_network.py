@@ -1,0 +1,158 @@
+"""Whole-network parity on the GPU through the C ABI (Network /
+NetworkComputation mirror) against the blas-backend restatement in oracle/nn.py,
+on identical seeded weights and seeded random-playout positions.
+
+Tolerances (fp16 configuration): 5e-3 max-abs on the softmaxed policy (all 1858
+moves and legal moves only), on W/D/L and q; the moves-left value is compared
+relatively. Raw logits are also compared so that a near-uniform softmax cannot
+hide an error."""
+import numpy as np
+import pytest
+
+from lc0_amd import netgen
+from oracle import chess as oc
+from oracle import netread as nr
+from oracle import nn as onn
+
+pytestmark = pytest.mark.gpu
+TOL = 5e-3
+
+
+@pytest.fixture(scope="module")
+def positions():
+    return oc.random_positions(320, seed=20240)
+
+
+def _run_gpu(path, masks, values, options=""):
+    from lc0_amd import Network
+    net = Network(path, options)
+    comp = net.NewComputation()
+    comp.AddInputs(masks, values)
+    comp.ComputeBlocking()
+    assert comp.GetBatchSize() == masks.shape[0]
+    res = comp.results()
+    comp.close()
+    return net, res
+
+
+def _compare(res, want, legal, tol=TOL):
+    pol_g, pol_o = res["policy"], want["policy"]
+    sm_g, sm_o = onn.softmax_rows(pol_g), onn.softmax_rows(pol_o)
+    stats = dict(policy_softmax=np.abs(sm_g - sm_o).max(),
+                 logits=np.abs(pol_g - pol_o).max(),
+                 wdl_q=np.abs(res["q"] - (want["wdl"][:, 0] - want["wdl"][:, 2])).max(),
+                 wdl_d=np.abs(res["d"] - want["wdl"][:, 1]).max(),
+                 mlh_rel=(np.abs(res["m"] - want["m"]) / np.maximum(np.abs(want["m"]), 1.0)).max())
+    legal_err = 0.0
+    top1 = 0
+    for i, lg in enumerate(legal):
+        a, b = onn.check_softmax_legal(pol_g[i], lg), onn.check_softmax_legal(pol_o[i], lg)
+        legal_err = max(legal_err, float(np.abs(a - b).max()))
+        top1 += int(a.argmax() == b.argmax())
+    stats["policy_legal_softmax"] = legal_err
+    stats["top1_agreement"] = top1 / len(legal)
+    print("parity:", {k: float(v) for k, v in stats.items()})
+    assert stats["policy_softmax"] <= tol
+    assert stats["policy_legal_softmax"] <= tol
+    assert stats["wdl_q"] <= tol and stats["wdl_d"] <= tol
+    assert stats["mlh_rel"] <= 2e-2
+    # logits of a random-init net are O(1): 3e-2 absolute is ~1e-2 relative
+    assert stats["logits"] <= 3e-2 * max(1.0, float(np.abs(pol_o).max()))
+    return stats
+
+
+@pytest.mark.parametrize("name,batch", [("tiny_attn", 37), ("tiny_attn_nosmolgen", 64), ("c1_attn_10x256", 64)])
+def test_attention_nets_match_oracle(name, batch, positions):
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    net, res = _run_gpu(path, masks, values)
+    caps = net.GetCapabilities()
+    assert (caps.input_format, caps.output_format, caps.moves_left) == (1, 2, 1)
+    assert not net.IsCpu()
+    _compare(res, want, positions["legal"][:batch])
+    # getter-level API on one sample
+    comp = net.NewComputation()
+    comp.AddInput([(int(m), float(v)) for m, v in zip(masks[3], values[3])])
+    comp.ComputeBlocking()
+    assert comp.GetBatchSize() == 1
+    np.testing.assert_allclose(comp.GetPVal(0, 100), res["policy"][3, 100], rtol=0, atol=2e-3)
+    np.testing.assert_allclose(comp.GetQVal(0), res["q"][3], atol=2e-3)
+    np.testing.assert_allclose(comp.GetDVal(0) + 0 * comp.GetMVal(0), res["d"][3], atol=2e-3)
+
+
+@pytest.mark.timeout(900)
+def test_bt4_shape_batch_256(positions):
+    """configs[2]: oracle comparison on the first 48 positions (seconds of CPU
+    time), then size-independent properties at the full batch of 256: rows are
+    independent, so the full-batch rows equal the small-batch rows, and a
+    permuted batch gives permuted outputs."""
+    path = netgen.cached_config("c2_bt4_15x1024")
+    masks, values = positions["masks"][:256], positions["values"][:256]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks[:48], values[:48])
+    net, res48 = _run_gpu(path, masks[:48], values[:48])
+    _compare(res48, want, positions["legal"][:48])
+    comp = net.NewComputation()
+    comp.AddInputs(masks, values)
+    comp.ComputeBlocking()
+    full = comp.results()
+    assert np.isfinite(full["policy"]).all()
+    np.testing.assert_allclose(full["policy"][:48], res48["policy"], rtol=0, atol=1e-5)
+    np.testing.assert_allclose(full["q"][:48], res48["q"], rtol=0, atol=1e-6)
+    perm = np.random.default_rng(0).permutation(256)
+    comp2 = net.NewComputation()
+    comp2.AddInputs(masks[perm], values[perm])
+    comp2.ComputeBlocking()
+    np.testing.assert_allclose(comp2.results()["policy"], full["policy"][perm], rtol=0, atol=1e-5)
+
+
+def test_ragged_and_oversized_batches(positions):
+    """Batch sizes that are not tile multiples, a batch larger than max_batch
+    (split into device passes) and an empty computation."""
+    path = netgen.cached_config("tiny_attn")
+    from lc0_amd import Network
+    net = Network(path, "max_batch=16")
+    assert net.GetMaxBatchSize() == 16
+    ref = None
+    for n in (1, 2, 15, 16, 17, 40):
+        comp = net.NewComputation()
+        comp.AddInputs(positions["masks"][:n], positions["values"][:n])
+        comp.ComputeBlocking()
+        r = comp.results()
+        if ref is None:
+            big = net.NewComputation()
+            big.AddInputs(positions["masks"][:40], positions["values"][:40])
+            big.ComputeBlocking()
+            ref = big.results()
+        np.testing.assert_allclose(r["policy"], ref["policy"][:n], rtol=0, atol=1e-5)
+        np.testing.assert_allclose(r["m"], ref["m"][:n], rtol=0, atol=1e-5)
+    empty = net.NewComputation()
+    empty.ComputeBlocking()
+    assert empty.GetBatchSize() == 0
+
+
+def test_error_behaviour(positions, tmp_path):
+    from lc0_amd import BackendError, Network, netproto
+    path = netgen.cached_config("tiny_attn")
+    with pytest.raises(BackendError, match="Unknown option"):
+        Network(path, "no_such_option=1")
+    with pytest.raises(BackendError, match="does not exist in this net"):
+        Network(path, "policy_head=soft")
+    with pytest.raises(BackendError, match="Cannot read weights"):
+        Network(str(tmp_path / "missing.pb.gz"))
+    raw = netproto.serialize_net(netgen.CONFIGS["tiny_attn"]())
+    with pytest.raises(BackendError, match="bad header"):
+        Network(raw.replace(b"\xc0\x01\x00\x00", b"\xc1\x01\x00\x00", 1))
+    net = Network(raw, "mlh=false")          # from a buffer, moves-left switched off
+    comp = net.NewComputation()
+    with pytest.raises(BackendError, match="112"):
+        comp.AddInput([(0, 1.0)] * 5)
+    comp.AddInputs(positions["masks"][:2], positions["values"][:2])
+    with pytest.raises(BackendError, match="ComputeBlocking"):
+        comp.GetQVal(0)
+    comp.ComputeBlocking()
+    assert comp.GetMVal(0) == 0.0
+    with pytest.raises(BackendError, match="out of range"):
+        comp.GetQVal(2)
+    with pytest.raises(BackendError, match="out of range"):
+        comp.GetPVal(0, 1858)
