@@ -27,6 +27,8 @@ struct GemmArgs {
   bool out_f32 = false;
 };
 void LaunchGemm(const GemmArgs& args, hipStream_t stream);
+// Name of the kernel variant LaunchGemm picks for these arguments (tile shape).
+const char* GemmVariantName(const GemmArgs& args);
 
 // Same contract in float: C = act(scale * A.W^T + bias) with float A, W, C.
 // K % 4 == 0, lda % 4 == 0, ldw % 4 == 0.

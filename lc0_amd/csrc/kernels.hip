@@ -40,6 +40,31 @@ __device__ __forceinline__ float Activate(float v, int act) {
   }
 }
 
+// Calls f with a branch-free functor for the activation, so that unrolled
+// epilogue loops do not carry a per-element switch.
+template <typename F>
+__device__ __forceinline__ void DispatchAct(int act, F&& f) {
+  switch (act) {
+    case 1: f([](float v) { return ActMish(v); }); break;
+    case 2: f([](float v) { return v > 0.0f ? v : 0.0f; }); break;
+    case 7: f([](float v) { return v / (1.0f + __expf(-v)); }); break;
+    case 8: f([](float v) { return v > 0.0f ? v * v : 0.0f; }); break;
+    case 3: f([](float v) { return v; }); break;
+    default: f([act](float v) { return Activate(v, act); }); break;
+  }
+}
+
+// bias[n..n+3] (zeros when there is no bias or past N).
+__device__ __forceinline__ void LoadBias4(const float* bias, int n, int N, float out[4]) {
+  if (bias != nullptr && n + 3 < N) {
+    floatx4 b = *reinterpret_cast<const floatx4*>(bias + n);
+    out[0] = b[0]; out[1] = b[1]; out[2] = b[2]; out[3] = b[3];
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; r++) out[r] = (bias != nullptr && n + r < N) ? bias[n + r] : 0.0f;
+  }
+}
+
 __device__ __forceinline__ float WaveSum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -145,40 +170,200 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
   // Epilogue. Accumulator element e of a tile: n = 8*(e/4) + 4*(lane/32) + e%4, m = lane%32.
   OutT* C = reinterpret_cast<OutT*>(p.C) + (long long)blockIdx.z * p.strideC;
   const bool vec_ok = (p.ldc % 4 == 0);
-#pragma unroll
-  for (int i = 0; i < TM; i++) {
-    const int m = m0 + wm * WM + i * 32 + frag_row;
-    if (m >= M) continue;
+  DispatchAct(p.act, [&](auto act_fn) {
 #pragma unroll
     for (int j = 0; j < TN; j++) {
 #pragma unroll
       for (int blk = 0; blk < 4; blk++) {
         const int n = n0 + wn * WN + j * 32 + blk * 8 + (lane >> 5) * 4;
         if (n >= N) continue;
-        float v[4];
+        float b4[4];
+        LoadBias4(p.bias, n, N, b4);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          float x = acc[i][j][blk * 4 + r] * p.scale;
-          if (p.bias != nullptr && n + r < N) x += p.bias[n + r];
-          v[r] = Activate(x, p.act);
-        }
-        OutT* dst = C + (long long)m * p.ldc + n;
-        if (vec_ok && n + 3 < N) {
-          if constexpr (sizeof(OutT) == 2) {
-            half4 h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-            *reinterpret_cast<half4*>(dst) = h;
+        for (int i = 0; i < TM; i++) {
+          const int m = m0 + wm * WM + i * 32 + frag_row;
+          if (m >= M) continue;
+          float v[4];
+#pragma unroll
+          for (int r = 0; r < 4; r++) v[r] = act_fn(acc[i][j][blk * 4 + r] * p.scale + b4[r]);
+          OutT* dst = C + (long long)m * p.ldc + n;
+          if (vec_ok && n + 3 < N) {
+            if constexpr (sizeof(OutT) == 2) {
+              half4 h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+              *reinterpret_cast<half4*>(dst) = h;
+            } else {
+              floatx4 f = {v[0], v[1], v[2], v[3]};
+              *reinterpret_cast<floatx4*>(dst) = f;
+            }
           } else {
-            floatx4 f = {v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<floatx4*>(dst) = f;
-          }
-        } else {
 #pragma unroll
-          for (int r = 0; r < 4; r++)
-            if (n + r < N) dst[r] = (OutT)v[r];
+            for (int r = 0; r < 4; r++)
+              if (n + r < N) dst[r] = (OutT)v[r];
+          }
         }
       }
     }
+  });
+}
+
+// ---------------------------------------------------------------------------
+// Large-shape GEMM: same contract as gemm_kernel for K % BK == 0 and half output.
+//
+// Operand tiles travel from global memory straight into LDS (16 bytes per lane,
+// global_load_lds_dwordx4), double-buffered, with one barrier per k-tile: the
+// fetch of k-tile t+1 is in flight while the MFMAs of k-tile t run, and no VGPR
+// is spent on staging. One such instruction fills 1 KiB of LDS in lane order, so
+// LDS rows are unpadded; the 16-byte chunk c of tile row r is stored at chunk
+// slot c ^ swizzle(r), which makes the ds_read_b128 fragment reads (32 rows x
+// one chunk column) hit all banks evenly. The epilogue applies scale, bias and
+// activation in registers, stages 32-row strips through LDS and writes rows of
+// the output as 16-byte vectors.
+// ---------------------------------------------------------------------------
+#define LC0MI_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// 16 bytes per lane from global memory into LDS at lds_base + lane * 16
+// (lds_base must be wave-uniform). Completion is visible through vmcnt only:
+// callers wait with s_waitcnt vmcnt(0) plus a barrier before reading the data.
+__device__ __forceinline__ void DmaToLds16(const half_t* gptr, half_t* lds_base) {
+  unsigned lds_addr = (unsigned)(size_t)LC0MI_LDS_PTR(lds_base);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory", "m0");
+}
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(GemmArgs p) {
+  constexpr int NWAVES = WAVES_M * WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int CPR = BK / 8;                     // 16-byte chunks per tile row
+  constexpr int ROWS_PER_CHUNK = 64 / CPR;        // tile rows per 1 KiB transfer
+  constexpr int SWZ_SHIFT = (BK == 64) ? 1 : 2;   // log2(rows per 256 bytes of LDS)
+  constexpr int A_CPW = BM / ROWS_PER_CHUNK / NWAVES, W_CPW = BN / ROWS_PER_CHUNK / NWAVES;
+  static_assert(BK == 64 || BK == 32, "BK must be 32 or 64");
+  static_assert(A_CPW >= 1 && W_CPW >= 1, "tile too small for the wave count");
+  constexpr int STAGE = (BM + BN) * BK;
+  constexpr int EPI_STRIDE = WN + 8;
+  constexpr int EPI_HALVES = NWAVES * 32 * EPI_STRIDE;
+  constexpr int SMEM = (2 * STAGE > EPI_HALVES) ? 2 * STAGE : EPI_HALVES;
+  __shared__ __attribute__((aligned(1024))) half_t smem[SMEM];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const half_t* A = p.A + (long long)blockIdx.z * p.strideA;
+  const half_t* W = p.W + (long long)blockIdx.z * p.strideW;
+  const int M = p.M, N = p.N, K = p.K;
+
+  const half_t* a_ptr[A_CPW];
+  const half_t* w_ptr[W_CPW];
+#pragma unroll
+  for (int i = 0; i < A_CPW; i++) {
+    const int row = (wave * A_CPW + i) * ROWS_PER_CHUNK + lane / CPR;
+    const int c = (lane % CPR) ^ ((row >> SWZ_SHIFT) % CPR);
+    a_ptr[i] = A + (long long)min(m0 + row, M - 1) * p.lda + c * 8;
   }
+#pragma unroll
+  for (int i = 0; i < W_CPW; i++) {
+    const int row = (wave * W_CPW + i) * ROWS_PER_CHUNK + lane / CPR;
+    const int c = (lane % CPR) ^ ((row >> SWZ_SHIFT) % CPR);
+    w_ptr[i] = W + (long long)min(n0 + row, N - 1) * p.ldw + c * 8;
+  }
+  auto issue = [&](half_t* As, half_t* Ws, int k0) {
+#pragma unroll
+    for (int i = 0; i < A_CPW; i++) DmaToLds16(a_ptr[i] + k0, As + (wave * A_CPW + i) * 512);
+#pragma unroll
+    for (int i = 0; i < W_CPW; i++) DmaToLds16(w_ptr[i] + k0, Ws + (wave * W_CPW + i) * 512);
+  };
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+  const int r = lane & 31, g = lane >> 5;
+  const int swz = (r >> SWZ_SHIFT) % CPR;
+  const int a_row = (wm * WM + r) * BK, w_row = (wn * WN + r) * BK;
+
+  const int nk = K / BK;
+  issue(smem, smem + BM * BK, 0);
+  for (int kt = 0; kt < nk; kt++) {
+    const half_t* As = smem + (kt & 1) * STAGE;
+    const half_t* Ws = As + BM * BK;
+    half_t* nxt = smem + ((kt + 1) & 1) * STAGE;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of k-tile kt have landed
+    __syncthreads();                     // ... and everybody's; everybody is done reading the other stage
+    if (kt + 1 < nk) issue(nxt, nxt + BM * BK, (kt + 1) * BK);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      const int coff = ((2 * ks + g) ^ swz) * 8;
+      half8 af[TM], wf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) af[i] = *reinterpret_cast<const half8*>(As + a_row + i * 32 * BK + coff);
+#pragma unroll
+      for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const half8*>(Ws + w_row + j * 32 * BK + coff);
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // Epilogue through LDS (the stage buffers are free after the barrier).
+  __syncthreads();
+  half_t* C = reinterpret_cast<half_t*>(p.C) + (long long)blockIdx.z * p.strideC;
+  half_t* strip = smem + wave * 32 * EPI_STRIDE;
+  constexpr int CHUNKS_PER_ROW = WN / 8;
+  constexpr int ROWS_PER_PASS = 64 / CHUNKS_PER_ROW;
+  const bool vec_ok = (p.ldc % 8 == 0);
+  float bias_v[TN][4][4];
+#pragma unroll
+  for (int j = 0; j < TN; j++)
+#pragma unroll
+    for (int blk = 0; blk < 4; blk++) LoadBias4(p.bias, n0 + wn * WN + j * 32 + blk * 8 + g * 4, N, bias_v[j][blk]);
+  DispatchAct(p.act, [&](auto act_fn) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int blk = 0; blk < 4; blk++) {
+          half4 h;
+#pragma unroll
+          for (int rr = 0; rr < 4; rr++) h[rr] = (half_t)act_fn(acc[i][j][blk * 4 + rr] * p.scale + bias_v[j][blk][rr]);
+          *reinterpret_cast<half4*>(&strip[r * EPI_STRIDE + j * 32 + blk * 8 + g * 4]) = h;
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0); the strip is private to this wave
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int pass = 0; pass < 32 / ROWS_PER_PASS; pass++) {
+        const int row = pass * ROWS_PER_PASS + lane / CHUNKS_PER_ROW;
+        const int ch = lane % CHUNKS_PER_ROW;
+        const int m = m0 + wm * WM + i * 32 + row;
+        const int n = n0 + wn * WN + ch * 8;
+        if (m < M && n < N) {
+          half_t* dst = C + (long long)m * p.ldc + n;
+          if (vec_ok && n + 7 < N) {
+            *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&strip[row * EPI_STRIDE + ch * 8]);
+          } else {
+            for (int e = 0; e < 8 && n + e < N; e++) dst[e] = strip[row * EPI_STRIDE + ch * 8 + e];
+          }
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_wave_barrier();
+    }
+  });
+}
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
+  dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch);
+  hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK, WAVES_M, WAVES_N>), grid, dim3(WAVES_M * WAVES_N * 64), 0, stream, a);
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
@@ -193,10 +378,30 @@ void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
 
 }  // namespace
 
+const char* GemmVariantName(const GemmArgs& a) {
+  const long long tiles256 = (long long)((a.M + 255) / 256) * ((a.N + 255) / 256) * a.batch;
+  const long long big_tiles = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
+  if (!a.out_f32 && a.K % 64 == 0 && a.K >= 128 && a.N >= 192 && tiles256 >= 128) {
+    // A last partial round of 256x256 tiles wastes up to a whole round; halve the tile then.
+    const long long rem = tiles256 % 256;
+    if (tiles256 < 1024 && rem != 0 && rem <= 160) return "gemm_dma_256x128x32";
+    return "gemm_dma_256x256x64";
+  }
+  return big_tiles >= 192 ? "gemm_128x128x64" : "gemm_64x64x64";
+}
+
 void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
-  const long long big_tiles = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
-  if (big_tiles >= 192) {
+  const char* variant = GemmVariantName(a);
+  if (variant[5] == 'd') {
+    if (variant[13] == '2') {
+      LaunchGemmDma<256, 256, 64, 2, 4>(a, stream);
+    } else {
+      LaunchGemmDma<256, 128, 32, 4, 2>(a, stream);
+    }
+    return;
+  }
+  if (variant[5] == '1') {
     LaunchGemmTile<128, 128, 64, 2, 2>(a, stream);
   } else {
     LaunchGemmTile<64, 64, 64, 2, 2>(a, stream);

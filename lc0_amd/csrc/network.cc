@@ -339,7 +339,8 @@ void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linea
   const double flops = 2.0 * M * lin.out * lin.in;
   const double bytes = 2.0 * (static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in) +
                        static_cast<double>(M) * lin.out * (out_f32 ? 4 : 2);
-  Timed(name, flops, bytes, [&] { LaunchGemm(g, stream_); });
+  const std::string label = std::string(name) + "|" + GemmVariantName(g);
+  Timed(label.c_str(), flops, bytes, [&] { LaunchGemm(g, stream_); });
 }
 
 // ------------------------------------------------------------- construction --
@@ -604,7 +605,8 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     g.scale = 1.0f / std::sqrt(static_cast<float>(pol_d_));
     g.act = kActNone;
     g.out_f32 = true;
-    Timed("gemm_policy_logits", 2.0 * 64 * 64 * pol_d_ * B, B * (2.0 * 2 * 64 * pol_d_ + 4.0 * 4096),
+    const std::string label = std::string("gemm_policy_logits|") + GemmVariantName(g);
+    Timed(label.c_str(), 2.0 * 64 * 64 * pol_d_ * B, B * (2.0 * 2 * 64 * pol_d_ + 4.0 * 4096),
           [&] { LaunchGemm(g, stream_); });
   }
   Timed("policy_gather", 0.0, B * (4.0 * 4288 + 4.0 * 1858), [&] {

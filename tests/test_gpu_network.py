@@ -97,8 +97,10 @@ def test_bt4_shape_batch_256(positions):
     comp.ComputeBlocking()
     full = comp.results()
     assert np.isfinite(full["policy"]).all()
-    np.testing.assert_allclose(full["policy"][:48], res48["policy"], rtol=0, atol=1e-5)
-    np.testing.assert_allclose(full["q"][:48], res48["q"], rtol=0, atol=1e-6)
+    # Different batch sizes may run different GEMM tile shapes (another summation
+    # order, then fp16 rounding of activations): equal to fp16 accuracy, not bitwise.
+    np.testing.assert_allclose(full["policy"][:48], res48["policy"], rtol=0, atol=5e-3)
+    np.testing.assert_allclose(full["q"][:48], res48["q"], rtol=0, atol=5e-3)
     perm = np.random.default_rng(0).permutation(256)
     comp2 = net.NewComputation()
     comp2.AddInputs(masks[perm], values[perm])
