@@ -21,6 +21,13 @@ extern "C" {
 int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* W, int ldw, long long strideW,
                  const float* bias, int M, int N, int K, int batch, float scale, int act, int out_f32, void* C,
                  int ldc, long long strideC, int time_iters, double* ms);
+/* Split-K form: K is cut into split_k slices whose float partial sums are added in
+ * slice order (bias added once, no activation). C is float [M][N]. */
+int lc0mi_k_gemm_splitk(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,
+                        int K, int split_k, float scale, float* C, int ldc);
+/* Forces the GEMM tile variant of subsequent calls (-1 automatic; 0 256x256x64,
+ * 1 256x192x64, 2 256x128x32 direct-to-LDS kernels, 3 128x128x64, 4 64x64x64). */
+int lc0mi_k_set_gemm_variant(int variant);
 /* float variant (fp32 configuration). */
 int lc0mi_k_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, int M, int N, int K,
                      float scale, int act, float* C, int ldc);
@@ -28,6 +35,11 @@ int lc0mi_k_gemm_f32(const float* A, int lda, const float* W, int ldw, const flo
  * (LayerNorm2DWithSkipConnection, src/neural/backends/blas/encoder.h:29-66) */
 int lc0mi_k_layer_norm(const uint16_t* x, const uint16_t* skip, const float* gamma, const float* beta, int rows,
                        int C, float alpha, float eps, uint16_t* y, int time_iters, double* ms);
+/* One-workgroup-per-row layer norm with an activation applied first:
+ * y = LN(act(x) * alpha + skip); x is float (x_f32) or half (x_f16), one of them NULL. */
+int lc0mi_k_layer_norm_rows(const float* x_f32, const uint16_t* x_f16, int pre_act, const uint16_t* skip,
+                            const float* gamma, const float* beta, int rows, int C, float alpha, float eps,
+                            uint16_t* y);
 /* Fused attention: qkv [B*64][3*heads*32] halves, bias [B][heads][64 q][64 k]
  * halves in natural order (may be NULL), out [B*64][heads*32]
  * (src/neural/backends/blas/network_blas.cc:352-439). */

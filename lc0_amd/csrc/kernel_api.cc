@@ -108,6 +108,64 @@ int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* 
   });
 }
 
+int lc0mi_k_gemm_splitk(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,
+                        int K, int split_k, float scale, float* C, int ldc) {
+  return Guard([&] {
+    RequireDevice();
+    if (K % 8 || lda % 8 || ldw % 8) throw Error("K, lda and ldw must be multiples of 8");
+    if (M < 1 || N < 1 || split_k < 1 || lda < K || ldw < K || ldc < N) throw Error("bad gemm shape");
+    Dev dev;
+    lc0mi::GemmArgs g;
+    g.A = reinterpret_cast<const half_t*>(dev.Put(A, (size_t)(M - 1) * lda + K)); g.lda = lda;
+    g.W = reinterpret_cast<const half_t*>(dev.Put(W, (size_t)(N - 1) * ldw + K)); g.ldw = ldw;
+    const size_t c_elems = (size_t)M * ldc;
+    float* dC = static_cast<float*>(dev.Alloc(c_elems * 4 * split_k));
+    g.C = dC; g.ldc = ldc;
+    g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
+    g.M = M; g.N = N; g.K = K; g.scale = scale; g.act = 3; g.out_f32 = true;
+    g.split_k = split_k; g.split_stride = (long long)c_elems;
+    lc0mi::LaunchGemm(g, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    // Add the slices on the host in slice order.
+    std::vector<float> part(c_elems * split_k);
+    K_CHECK(hipMemcpy(part.data(), dC, part.size() * 4, hipMemcpyDeviceToHost));
+    for (int m = 0; m < M; m++)
+      for (int n = 0; n < N; n++) {
+        float s = 0.0f;
+        for (int z = 0; z < split_k; z++) s += part[(size_t)z * c_elems + (size_t)m * ldc + n];
+        C[(size_t)m * ldc + n] = s;
+      }
+  });
+}
+
+int lc0mi_k_layer_norm_rows(const float* x_f32, const uint16_t* x_f16, int pre_act, const uint16_t* skip,
+                            const float* gamma, const float* beta, int rows, int C, float alpha, float eps,
+                            uint16_t* y) {
+  return Guard([&] {
+    RequireDevice();
+    if (C % 8 || C < 8 || C > 8192 || rows < 1) throw Error("bad layer norm shape");
+    if ((x_f32 == nullptr) == (x_f16 == nullptr)) throw Error("exactly one of x_f32 / x_f16 must be given");
+    Dev dev;
+    const size_t n = (size_t)rows * C;
+    const float* dxf = x_f32 ? dev.Put(x_f32, n) : nullptr;
+    const half_t* dxh = x_f16 ? reinterpret_cast<const half_t*>(dev.Put(x_f16, n)) : nullptr;
+    const half_t* ds = skip ? reinterpret_cast<const half_t*>(dev.Put(skip, n)) : nullptr;
+    auto* dy = reinterpret_cast<half_t*>(dev.Alloc(n * 2));
+    float* dg = dev.Put(gamma, (size_t)C);
+    float* db = dev.Put(beta, (size_t)C);
+    lc0mi::LaunchLayerNormRows(dxf, dxf ? 1 : 0, 0, dxh, pre_act, ds, dy, dg, db, rows, C, alpha, eps, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(y, dy, n * 2, hipMemcpyDeviceToHost));
+  });
+}
+
+int lc0mi_k_set_gemm_variant(int variant) {
+  lc0mi::SetGemmVariantOverride(variant);
+  return 0;
+}
+
 int lc0mi_k_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, int M, int N, int K,
                      float scale, int act, float* C, int ldc) {
   return Guard([&] {

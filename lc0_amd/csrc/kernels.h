@@ -25,6 +25,12 @@ struct GemmArgs {
   float scale = 1.0f;
   int act = 3;  // Activation enum value (3 = none)
   bool out_f32 = false;
+  // split_k > 1: the K range is cut into split_k slices computed by different
+  // workgroups; slice s stores its partial sums (float, out_f32 required, no
+  // activation, bias only in slice 0) at C + s * split_stride. The consumer adds
+  // the slices.
+  int split_k = 1;
+  long long split_stride = 0;
 };
 void LaunchGemm(const GemmArgs& args, hipStream_t stream);
 // Name of the kernel variant LaunchGemm picks for these arguments (tile shape).
@@ -52,6 +58,21 @@ void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T*
 // Input planes -> NCHW dense planes out[b][c][sq] (T = half_t or float).
 template <typename T>
 void LaunchExpandPlanesNchw(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream);
+
+// Sets n floats to zero (a kernel, so that it can be captured into a graph).
+void LaunchZero(float* p, long long n, hipStream_t stream);
+// Forces LaunchGemm to use one kernel variant (-1 = automatic choice): 0 256x256x64,
+// 1 256x192x64, 2 256x128x32 (direct-to-LDS, need K % 64 == 0 and half output),
+// 3 128x128x64, 4 64x64x64. For tests and tuning only.
+void SetGemmVariantOverride(int variant);
+
+// Layer norm for few, long rows (one workgroup per row): t = act(x) * alpha + skip,
+// where x is half (x_f16) or the sum of n_partials float arrays x_f32 + i * partial_stride
+// (split-K partial sums); exactly one of x_f32 / x_f16 is non-null. pre_act is an
+// Activation enum value applied before the norm. C % 8 == 0, C <= 8192.
+void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_stride, const half_t* x_f16,
+                         int pre_act, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows,
+                         int C, float alpha, float eps, hipStream_t stream);
 
 // rows x C layer norm: y = beta + gamma * (t - mean) / sqrt(var + eps) with
 // t = x * alpha + skip (skip may be null). x, skip, y may alias. C % 8 == 0, C <= 8192.

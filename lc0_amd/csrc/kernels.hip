@@ -98,9 +98,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
-  const half_t* A = p.A + (long long)blockIdx.z * p.strideA;
-  const half_t* W = p.W + (long long)blockIdx.z * p.strideW;
-  const int M = p.M, N = p.N, K = p.K;
+  const int zb = blockIdx.z / p.split_k, zs = blockIdx.z - zb * p.split_k;
+  const half_t* A = p.A + (long long)zb * p.strideA;
+  const half_t* W = p.W + (long long)zb * p.strideW;
+  const int M = p.M, N = p.N;
+  // This workgroup's slice of the reduction dimension.
+  const int k_slice = ((p.K + p.split_k - 1) / p.split_k + BK - 1) / BK * BK;
+  const int k_begin = zs * k_slice;
+  const int K = min(p.K, k_begin + k_slice);
 
   uint4 ra[A_VECS], rw[W_VECS];
   auto load_tile = [&](int k0) {
@@ -142,13 +147,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-  const int nk = (K + BK - 1) / BK;
+  const int nk = K > k_begin ? (K - k_begin + BK - 1) / BK : 0;
   const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
-  load_tile(0);
+  if (nk > 0) load_tile(k_begin);
   for (int kt = 0; kt < nk; kt++) {
     store_tile();
     __syncthreads();
-    if (kt + 1 < nk) load_tile((kt + 1) * BK);
+    if (kt + 1 < nk) load_tile(k_begin + (kt + 1) * BK);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ks++) {
       half8 af[TM], wf[TN];
@@ -168,7 +173,30 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
   }
 
   // Epilogue. Accumulator element e of a tile: n = 8*(e/4) + 4*(lane/32) + e%4, m = lane%32.
-  OutT* C = reinterpret_cast<OutT*>(p.C) + (long long)blockIdx.z * p.strideC;
+  OutT* C = reinterpret_cast<OutT*>(p.C) + (long long)zb * p.strideC;
+  if constexpr (sizeof(OutT) == 4) {
+    if (p.split_k > 1) {
+      // Every slice stores its own partial sums (no atomics: the consumer adds the
+      // slices in a fixed order, so results do not depend on scheduling).
+      C += (long long)zs * p.split_stride;
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int blk = 0; blk < 4; blk++) {
+          const int n = n0 + wn * WN + j * 32 + blk * 8 + (lane >> 5) * 4;
+          float b4[4];
+          LoadBias4(zs == 0 ? p.bias : nullptr, n, N, b4);
+#pragma unroll
+          for (int i = 0; i < TM; i++) {
+            const int m = m0 + wm * WM + i * 32 + frag_row;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+              if (m < M && n + r < N) C[(long long)m * p.ldc + n + r] = acc[i][j][blk * 4 + r] * p.scale + b4[r];
+          }
+        }
+      return;
+    }
+  }
   const bool vec_ok = (p.ldc % 4 == 0);
   DispatchAct(p.act, [&](auto act_fn) {
 #pragma unroll
@@ -317,7 +345,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(GemmArg
   half_t* C = reinterpret_cast<half_t*>(p.C) + (long long)blockIdx.z * p.strideC;
   half_t* strip = smem + wave * 32 * EPI_STRIDE;
   constexpr int CHUNKS_PER_ROW = WN / 8;
-  constexpr int ROWS_PER_PASS = 64 / CHUNKS_PER_ROW;
+  constexpr int STRIP_CHUNKS = 32 * CHUNKS_PER_ROW;
   const bool vec_ok = (p.ldc % 8 == 0);
   float bias_v[TN][4][4];
 #pragma unroll
@@ -340,12 +368,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(GemmArg
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0); the strip is private to this wave
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
-      for (int pass = 0; pass < 32 / ROWS_PER_PASS; pass++) {
-        const int row = pass * ROWS_PER_PASS + lane / CHUNKS_PER_ROW;
-        const int ch = lane % CHUNKS_PER_ROW;
+      for (int pass = 0; pass < (STRIP_CHUNKS + 63) / 64; pass++) {
+        const int idx = pass * 64 + lane;
+        const int row = idx / CHUNKS_PER_ROW;
+        const int ch = idx - row * CHUNKS_PER_ROW;
         const int m = m0 + wm * WM + i * 32 + row;
         const int n = n0 + wn * WN + ch * 8;
-        if (m < M && n < N) {
+        if (idx < STRIP_CHUNKS && m < M && n < N) {
           half_t* dst = C + (long long)m * p.ldc + n;
           if (vec_ok && n + 7 < N) {
             *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&strip[row * EPI_STRIDE + ch * 8]);
@@ -368,7 +397,7 @@ void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
-  dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch);
+  dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch * a.split_k);
   if (a.out_f32) {
     hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, float>), grid, dim3(256), 0, stream, a);
   } else {
@@ -378,33 +407,54 @@ void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
 
 }  // namespace
 
-const char* GemmVariantName(const GemmArgs& a) {
+namespace {
+enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64 };
+
+int g_variant_override = -1;
+
+GemmVariant PickGemmVariant(const GemmArgs& a) {
+  if (g_variant_override >= 0) {
+    const bool dma_ok = !a.out_f32 && a.split_k == 1 && a.K % 64 == 0;
+    if (g_variant_override >= kTile128 || dma_ok) return static_cast<GemmVariant>(g_variant_override);
+  }
   const long long tiles256 = (long long)((a.M + 255) / 256) * ((a.N + 255) / 256) * a.batch;
   const long long big_tiles = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
-  if (!a.out_f32 && a.K % 64 == 0 && a.K >= 128 && a.N >= 192 && tiles256 >= 128) {
-    // A last partial round of 256x256 tiles wastes up to a whole round; halve the tile then.
-    const long long rem = tiles256 % 256;
-    if (tiles256 < 1024 && rem != 0 && rem <= 160) return "gemm_dma_256x128x32";
-    return "gemm_dma_256x256x64";
+  if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= 128 && a.N >= 192 && tiles256 >= 128) {
+    // One workgroup per CU at a time: time ~ rounds over 256 CUs x tile width,
+    // with a small efficiency penalty for the narrower tiles.
+    const long long m_tiles = (a.M + 255) / 256;
+    auto cost = [&](int bn, double penalty) {
+      const long long tiles = m_tiles * ((a.N + bn - 1) / bn) * a.batch;
+      return (double)((tiles + 255) / 256) * bn * penalty;
+    };
+    const double c256 = cost(256, 1.0), c192 = cost(192, 1.04), c128 = cost(128, 1.15);
+    if (c256 <= c192 && c256 <= c128) return kDma256x256;
+    return c192 <= c128 ? kDma256x192 : kDma256x128;
   }
-  return big_tiles >= 192 ? "gemm_128x128x64" : "gemm_64x64x64";
+  return big_tiles >= 192 ? kTile128 : kTile64;
+}
+}  // namespace
+
+void SetGemmVariantOverride(int variant) { g_variant_override = variant; }
+
+const char* GemmVariantName(const GemmArgs& a) {
+  switch (PickGemmVariant(a)) {
+    case kDma256x256: return "gemm_dma_256x256x64";
+    case kDma256x192: return "gemm_dma_256x192x64";
+    case kDma256x128: return "gemm_dma_256x128x32";
+    case kTile128: return "gemm_128x128x64";
+    default: return a.split_k > 1 ? "gemm_64x64x64_splitk" : "gemm_64x64x64";
+  }
 }
 
 void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
-  const char* variant = GemmVariantName(a);
-  if (variant[5] == 'd') {
-    if (variant[13] == '2') {
-      LaunchGemmDma<256, 256, 64, 2, 4>(a, stream);
-    } else {
-      LaunchGemmDma<256, 128, 32, 4, 2>(a, stream);
-    }
-    return;
-  }
-  if (variant[5] == '1') {
-    LaunchGemmTile<128, 128, 64, 2, 2>(a, stream);
-  } else {
-    LaunchGemmTile<64, 64, 64, 2, 2>(a, stream);
+  switch (PickGemmVariant(a)) {
+    case kDma256x256: LaunchGemmDma<256, 256, 64, 2, 4>(a, stream); break;
+    case kDma256x192: LaunchGemmDma<256, 192, 64, 4, 2>(a, stream); break;
+    case kDma256x128: LaunchGemmDma<256, 128, 32, 4, 2>(a, stream); break;
+    case kTile128: LaunchGemmTile<128, 128, 64, 2, 2>(a, stream); break;
+    default: LaunchGemmTile<64, 64, 64, 2, 2>(a, stream); break;
   }
 }
 
@@ -593,6 +643,96 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restric
   }
 }
 }  // namespace
+
+namespace {
+__global__ __launch_bounds__(256) void zero_kernel(float* p, long long n) {
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0.0f;
+}
+
+// One workgroup per row; every thread keeps up to 4 vectors of 8 elements.
+__global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __restrict__ xf, int n_partials,
+                                                              long long partial_stride, const half_t* xh,
+                                                              int pre_act, const half_t* skip, half_t* y,
+                                                              const float* __restrict__ gamma,
+                                                              const float* __restrict__ beta, int C, float alpha,
+                                                              float eps) {
+  __shared__ float red[4];
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nvec = C / 8;
+  float t[4][8];
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int v = tid + i * 256;
+#pragma unroll
+    for (int e = 0; e < 8; e++) t[i][e] = 0.0f;
+    if (v < nvec) {
+      const long long off = (long long)row * C + v * 8;
+      if (xf != nullptr) {
+        for (int part = 0; part < n_partials; part++) {
+          floatx4 a = *reinterpret_cast<const floatx4*>(xf + part * partial_stride + off);
+          floatx4 b = *reinterpret_cast<const floatx4*>(xf + part * partial_stride + off + 4);
+#pragma unroll
+          for (int e = 0; e < 4; e++) { t[i][e] += a[e]; t[i][4 + e] += b[e]; }
+        }
+      } else {
+        half8 h = *reinterpret_cast<const half8*>(xh + off);
+#pragma unroll
+        for (int e = 0; e < 8; e++) t[i][e] = (float)h[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e++) t[i][e] = Activate(t[i][e], pre_act) * alpha;
+      if (skip != nullptr) {
+        half8 hs = *reinterpret_cast<const half8*>(skip + off);
+#pragma unroll
+        for (int e = 0; e < 8; e++) t[i][e] += (float)hs[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e++) sum += t[i][e];
+    }
+  }
+  sum = WaveSum(sum);
+  if (lane == 0) red[wave] = sum;
+  __syncthreads();
+  const float mean = (red[0] + red[1] + red[2] + red[3]) / (float)C;
+  __syncthreads();
+  float var = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    if (tid + i * 256 < nvec) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) { float d = t[i][e] - mean; var += d * d; }
+    }
+  var = WaveSum(var);
+  if (lane == 0) red[wave] = var;
+  __syncthreads();
+  const float den = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)C + eps);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int v = tid + i * 256;
+    if (v < nvec) {
+      half8 o;
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = (half_t)(beta[v * 8 + e] + gamma[v * 8 + e] * (t[i][e] - mean) * den);
+      *reinterpret_cast<half8*>(y + (long long)row * C + v * 8) = o;
+    }
+  }
+}
+}  // namespace
+
+void LaunchZero(float* p, long long n, hipStream_t stream) {
+  if (n <= 0) return;
+  hipLaunchKernelGGL(zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, n);
+}
+
+void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_stride, const half_t* x_f16,
+                         int pre_act, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows,
+                         int C, float alpha, float eps, hipStream_t stream) {
+  if (rows <= 0) return;
+  hipLaunchKernelGGL(layer_norm_rows_kernel, dim3(rows), dim3(256), 0, stream, x_f32, n_partials, partial_stride,
+                     x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps);
+}
 
 void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
                      int rows, int C, float alpha, float eps, hipStream_t stream) {

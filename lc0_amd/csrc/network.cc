@@ -146,9 +146,18 @@ struct HostSlot {
 
 class Mi355xNetwork;
 
+// Free list of pinned staging slots. Shared by the network and its computations
+// so that a computation destroyed after its network still has a valid place to
+// return its slots to.
+struct SlotPool {
+  std::mutex mutex;
+  std::vector<std::unique_ptr<HostSlot>> free_slots;
+  bool network_alive = true;
+};
+
 class Mi355xComputation : public NetworkComputation {
  public:
-  explicit Mi355xComputation(Mi355xNetwork* net) : net_(net) {}
+  Mi355xComputation(Mi355xNetwork* net, std::shared_ptr<SlotPool> pool) : net_(net), pool_(std::move(pool)) {}
   ~Mi355xComputation() override;
   void AddInput(InputPlanes&& input) override;
   void AddInputs(int n, const uint64_t* masks, const float* values) override;
@@ -166,7 +175,14 @@ class Mi355xComputation : public NetworkComputation {
     if (!computed_) throw Error("ComputeBlocking() has not been called");
   }
   HostSlot* SlotFor(int index);
+  Mi355xNetwork* Net() const {
+    if (!pool_->network_alive) throw Error("the network of this computation has been destroyed");
+    return net_;
+  }
   Mi355xNetwork* net_;
+  std::shared_ptr<SlotPool> pool_;
+  int max_batch_ = 0;
+  bool wdl_ = false, moves_left_ = false;
   std::vector<std::unique_ptr<HostSlot>> slots_;
   int batch_ = 0;
   bool computed_ = false;
@@ -179,7 +195,7 @@ class Mi355xNetwork : public Network {
 
   const NetworkCapabilities& GetCapabilities() const override { return caps_; }
   std::unique_ptr<NetworkComputation> NewComputation() override {
-    return std::make_unique<Mi355xComputation>(this);
+    return std::make_unique<Mi355xComputation>(this, pool_);
   }
   int GetMiniBatchSize() const override { return 256; }
   int GetMaxBatchSize() const override { return max_batch_; }
@@ -208,9 +224,9 @@ class Mi355xNetwork : public Network {
 
   // Launch helpers (profiling aware).
   template <typename F>
-  void Timed(const char* name, double flops, double bytes, F&& launch);
+  void Timed(const char* name, double flops, double bytes, F&& launch, hipStream_t st = nullptr);
   void Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act,
-            bool out_f32 = false);
+            bool out_f32 = false, hipStream_t st = nullptr, int split_k = 1);
 
   NetworkCapabilities caps_;
   int device_ = 0;
@@ -219,10 +235,11 @@ class Mi355xNetwork : public Network {
   int default_act_ = kActRelu, smolgen_act_ = kActNone, ffn_act_ = kActNone;
   std::string policy_head_, value_head_;
   hipStream_t stream_ = nullptr;
+  hipStream_t side_stream_ = nullptr;  // smolgen chain, overlapped with the QKV projection
+  std::vector<hipEvent_t> fork_events_, join_events_;
   DeviceArena arena_;
   std::mutex eval_mutex_;
-  std::mutex slots_mutex_;
-  std::vector<std::unique_ptr<HostSlot>> free_slots_;
+  std::shared_ptr<SlotPool> pool_ = std::make_shared<SlotPool>();
 
   // Attention body dimensions.
   int emb_ = 0, d_model_ = 0, heads_ = 0, dff_ = 0, in_ld_ = 192;
@@ -244,6 +261,7 @@ class Mi355xNetwork : public Network {
   float* d_values_ = nullptr;
   half_t *in0_ = nullptr, *x_ = nullptr, *t_ = nullptr, *qkv_ = nullptr, *att_ = nullptr, *ffn_ = nullptr;
   half_t *sg1_ = nullptr, *sg2_ = nullptr, *sg3_ = nullptr, *sbias_ = nullptr;
+  float* sg2f_ = nullptr;  // split-K accumulator of smolgen dense1
   half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
   float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
 
@@ -270,15 +288,16 @@ hipEvent_t Mi355xNetwork::NewEvent() {
 }
 
 template <typename F>
-void Mi355xNetwork::Timed(const char* name, double flops, double bytes, F&& launch) {
+void Mi355xNetwork::Timed(const char* name, double flops, double bytes, F&& launch, hipStream_t st) {
   if (!profiling_) {
     launch();
     return;
   }
+  if (st == nullptr) st = stream_;
   Pending p{name, NewEvent(), NewEvent(), flops, bytes};
-  HIP_CHECK(hipEventRecord(p.start, stream_));
+  HIP_CHECK(hipEventRecord(p.start, st));
   launch();
-  HIP_CHECK(hipEventRecord(p.stop, stream_));
+  HIP_CHECK(hipEventRecord(p.stop, st));
   pending_.push_back(p);
 }
 
@@ -327,8 +346,11 @@ Linear Mi355xNetwork::MakeLinear(const Vec& w, const Vec& b, int out, int in) {
 }
 
 void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M,
-                         int act, bool out_f32) {
+                         int act, bool out_f32, hipStream_t st, int split_k) {
+  if (st == nullptr) st = stream_;
   GemmArgs g;
+  g.split_k = split_k;
+  g.split_stride = static_cast<long long>(M) * ldc;
   g.A = A; g.lda = lda;
   g.W = lin.w; g.ldw = lin.ld;
   g.C = C; g.ldc = ldc;
@@ -340,7 +362,7 @@ void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linea
   const double bytes = 2.0 * (static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in) +
                        static_cast<double>(M) * lin.out * (out_f32 ? 4 : 2);
   const std::string label = std::string(name) + "|" + GemmVariantName(g);
-  Timed(label.c_str(), flops, bytes, [&] { LaunchGemm(g, stream_); });
+  Timed(label.c_str(), flops, bytes, [&] { LaunchGemm(g, st); }, st);
 }
 
 // ------------------------------------------------------------- construction --
@@ -383,6 +405,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   if (device_ < 0 || device_ >= count) throw Error("Invalid GPU id " + std::to_string(device_) + ".");
   HIP_CHECK(hipSetDevice(device_));
   HIP_CHECK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+  HIP_CHECK(hipStreamCreateWithFlags(&side_stream_, hipStreamNonBlocking));
 
   d_masks_ = static_cast<uint64_t*>(arena_.Alloc(sizeof(uint64_t) * kInputPlanes * max_batch_));
   d_values_ = AllocF(static_cast<size_t>(kInputPlanes) * max_batch_);
@@ -399,9 +422,20 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
 }
 
 Mi355xNetwork::~Mi355xNetwork() {
+  {
+    std::lock_guard<std::mutex> lock(pool_->mutex);
+    pool_->network_alive = false;
+    pool_->free_slots.clear();
+  }
   if (stream_) {
     (void)hipStreamSynchronize(stream_);
     for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
+    for (hipEvent_t e : fork_events_) (void)hipEventDestroy(e);
+    for (hipEvent_t e : join_events_) (void)hipEventDestroy(e);
+    if (side_stream_) {
+      (void)hipStreamSynchronize(side_stream_);
+      (void)hipStreamDestroy(side_stream_);
+    }
     (void)hipStreamDestroy(stream_);
   }
 }
@@ -535,6 +569,14 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   if (any_smolgen_) {
     sg1_ = AllocH(T * sg_hc_);
     sg2_ = AllocH(static_cast<size_t>(max_batch_) * sg_hs_);
+    sg2f_ = AllocF(static_cast<size_t>(max_batch_) * sg_hs_ * 16);  // up to 16 split-K slices
+    for (size_t i = 0; i < encoders_.size(); i++) {
+      hipEvent_t a, b;
+      HIP_CHECK(hipEventCreateWithFlags(&a, hipEventDisableTiming));
+      HIP_CHECK(hipEventCreateWithFlags(&b, hipEventDisableTiming));
+      fork_events_.push_back(a);
+      join_events_.push_back(b);
+    }
     sg3_ = AllocH(static_cast<size_t>(max_batch_) * sg_gen_);
     sbias_ = AllocH(static_cast<size_t>(max_batch_) * heads_ * 4096);
   }
@@ -552,23 +594,38 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
         [&] { LaunchExpandPlanesAttn<half_t>(d_masks_, d_values_, pos_enc_, in0_, in_ld_, B, stream_); });
   Gemm("gemm_embedding", in0_, in_ld_, emb_lin_, x_, emb_, T, default_act_);
 
-  for (const EncoderDev& e : encoders_) {
+  for (size_t li = 0; li < encoders_.size(); li++) {
+    const EncoderDev& e = encoders_[li];
     const half_t* bias = nullptr;
+    // The smolgen chain depends only on x: it runs on the side stream next to the
+    // QKV projection (on the main stream when profiling, for clean per-kernel times).
+    hipStream_t ss = profiling_ ? stream_ : side_stream_;
     if (e.has_smolgen) {
       const int g = sg_gen_ / heads_;
-      Gemm("gemm_smolgen_compress", x_, emb_, e.sg_compress, sg1_, sg_hc_, T, kActNone);
-      Gemm("gemm_smolgen_dense1", sg1_, 64 * sg_hc_, e.sg_dense1, sg2_, sg_hs_, B, smolgen_act_);
-      Timed("layer_norm_smolgen", 0.0, 4.0 * B * sg_hs_, [&] {
-        LaunchLayerNorm(sg2_, nullptr, sg2_, e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f, 1e-3f, stream_);
-      });
-      Gemm("gemm_smolgen_dense2", sg2_, sg_hs_, e.sg_dense2, sg3_, sg_gen_, B, smolgen_act_);
-      Timed("layer_norm_smolgen", 0.0, 4.0 * B * sg_gen_, [&] {
-        LaunchLayerNorm(sg3_, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f, 1e-3f, stream_);
-      });
-      Gemm("gemm_smolgen_global", sg3_, g, smolgen_w_, sbias_, 4096, B * heads_, kActNone);
+      if (ss != stream_) {
+        HIP_CHECK(hipEventRecord(fork_events_[li], stream_));
+        HIP_CHECK(hipStreamWaitEvent(ss, fork_events_[li], 0));
+      }
+      Gemm("gemm_smolgen_compress", x_, emb_, e.sg_compress, sg1_, sg_hc_, T, kActNone, false, ss);
+      // dense1 has a long reduction and few outputs: split K, accumulate in float,
+      // and let the layer norm kernel apply the activation.
+      const int split = std::max(1, std::min(16, (64 * sg_hc_) / 256));
+      Gemm("gemm_smolgen_dense1", sg1_, 64 * sg_hc_, e.sg_dense1, sg2f_, sg_hs_, B, kActNone, true, ss, split);
+      Timed("layer_norm_rows", 0.0, (4.0 * split + 2.0) * B * sg_hs_, [&] {
+        LaunchLayerNormRows(sg2f_, split, static_cast<long long>(B) * sg_hs_, nullptr, smolgen_act_, nullptr, sg2_,
+                            e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f, 1e-3f, ss);
+      }, ss);
+      Gemm("gemm_smolgen_dense2", sg2_, sg_hs_, e.sg_dense2, sg3_, sg_gen_, B, smolgen_act_, false, ss);
+      Timed("layer_norm_rows", 0.0, 4.0 * B * sg_gen_, [&] {
+        LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f, 1e-3f,
+                            ss);
+      }, ss);
+      Gemm("gemm_smolgen_global", sg3_, g, smolgen_w_, sbias_, 4096, B * heads_, kActNone, false, ss);
+      if (ss != stream_) HIP_CHECK(hipEventRecord(join_events_[li], ss));
       bias = sbias_;
     }
     Gemm("gemm_qkv", x_, emb_, e.qkv, qkv_, 3 * d_model_, T, kActNone);
+    if (e.has_smolgen && ss != stream_) HIP_CHECK(hipStreamWaitEvent(stream_, join_events_[li], 0));
     Timed("attention", 4.0 * 2 * 64 * 64 * 32 * B * heads_ / 2.0,
           B * heads_ * (2.0 * (3 * 64 * 32 + 64 * 32) + (bias ? 2.0 * 4096 : 0.0)),
           [&] { LaunchAttention(qkv_, bias, att_, B, heads_, 1.0f / std::sqrt(32.0f), stream_); });
@@ -674,10 +731,10 @@ double Mi355xNetwork::TimeResidentForward(int batch, int iters) {
 
 std::unique_ptr<HostSlot> Mi355xNetwork::GetSlot() {
   {
-    std::lock_guard<std::mutex> lock(slots_mutex_);
-    if (!free_slots_.empty()) {
-      auto s = std::move(free_slots_.back());
-      free_slots_.pop_back();
+    std::lock_guard<std::mutex> lock(pool_->mutex);
+    if (!pool_->free_slots.empty()) {
+      auto s = std::move(pool_->free_slots.back());
+      pool_->free_slots.pop_back();
       return s;
     }
   }
@@ -693,19 +750,28 @@ std::unique_ptr<HostSlot> Mi355xNetwork::GetSlot() {
 }
 
 void Mi355xNetwork::ReleaseSlot(std::unique_ptr<HostSlot> slot) {
-  std::lock_guard<std::mutex> lock(slots_mutex_);
-  free_slots_.push_back(std::move(slot));
+  std::lock_guard<std::mutex> lock(pool_->mutex);
+  pool_->free_slots.push_back(std::move(slot));
 }
 
 // -------------------------------------------------------------- computation --
 Mi355xComputation::~Mi355xComputation() {
-  for (auto& s : slots_) net_->ReleaseSlot(std::move(s));
+  std::lock_guard<std::mutex> lock(pool_->mutex);
+  if (pool_->network_alive) {
+    for (auto& s : slots_) pool_->free_slots.push_back(std::move(s));
+  }
+  // Otherwise the slots are simply freed here (pinned memory outlives the network object).
 }
 
 HostSlot* Mi355xComputation::SlotFor(int index) {
-  const int cap = net_->GetMaxBatchSize();
-  const size_t si = static_cast<size_t>(index / cap);
-  while (slots_.size() <= si) slots_.push_back(net_->GetSlot());
+  Mi355xNetwork* net = Net();
+  if (max_batch_ == 0) {
+    max_batch_ = net->GetMaxBatchSize();
+    wdl_ = net->wdl();
+    moves_left_ = net->moves_left();
+  }
+  const size_t si = static_cast<size_t>(index / max_batch_);
+  while (slots_.size() <= si) slots_.push_back(net->GetSlot());
   return slots_[si].get();
 }
 
@@ -714,7 +780,7 @@ void Mi355xComputation::AddInput(InputPlanes&& input) {
     throw Error("AddInput expects exactly 112 input planes, got " + std::to_string(input.size()) + ".");
   }
   HostSlot* s = SlotFor(batch_);
-  const int at = batch_ % net_->GetMaxBatchSize();
+  const int at = batch_ % max_batch_;
   uint64_t* m = s->masks + static_cast<size_t>(at) * kInputPlanes;
   float* v = s->values + static_cast<size_t>(at) * kInputPlanes;
   for (int i = 0; i < kInputPlanes; i++) {
@@ -729,7 +795,7 @@ void Mi355xComputation::AddInputs(int n, const uint64_t* masks, const float* val
   if (n < 0) throw Error("negative input count");
   for (int i = 0; i < n; i++) {
     HostSlot* s = SlotFor(batch_);
-    const int at = batch_ % net_->GetMaxBatchSize();
+    const int at = batch_ % max_batch_;
     std::memcpy(s->masks + static_cast<size_t>(at) * kInputPlanes, masks + static_cast<size_t>(i) * kInputPlanes,
                 sizeof(uint64_t) * kInputPlanes);
     std::memcpy(s->values + static_cast<size_t>(at) * kInputPlanes, values + static_cast<size_t>(i) * kInputPlanes,
@@ -740,39 +806,39 @@ void Mi355xComputation::AddInputs(int n, const uint64_t* masks, const float* val
 }
 
 void Mi355xComputation::ComputeBlocking() {
-  const int cap = net_->GetMaxBatchSize();
+  Mi355xNetwork* net = Net();
   for (size_t si = 0; si < slots_.size(); si++) {
-    const int n = std::min(cap, batch_ - static_cast<int>(si) * cap);
-    net_->Evaluate(slots_[si].get(), n);
+    const int n = std::min(max_batch_, batch_ - static_cast<int>(si) * max_batch_);
+    net->Evaluate(slots_[si].get(), n);
   }
   computed_ = true;
 }
 
 const float* Mi355xComputation::GetPolicyRow(int sample) const {
   CheckSample(sample);
-  const int cap = net_->GetMaxBatchSize();
+  const int cap = max_batch_;
   return slots_[sample / cap]->policy + static_cast<size_t>(sample % cap) * kPolicyOutputs;
 }
 
 float Mi355xComputation::GetQVal(int sample) const {
   CheckSample(sample);
-  const int cap = net_->GetMaxBatchSize();
+  const int cap = max_batch_;
   const float* w = slots_[sample / cap]->wdl;
-  if (net_->wdl()) return w[3 * (sample % cap)] - w[3 * (sample % cap) + 2];
+  if (wdl_) return w[3 * (sample % cap)] - w[3 * (sample % cap) + 2];
   return w[sample % cap];
 }
 
 float Mi355xComputation::GetDVal(int sample) const {
   CheckSample(sample);
-  if (!net_->wdl()) return 0.0f;
-  const int cap = net_->GetMaxBatchSize();
+  if (!wdl_) return 0.0f;
+  const int cap = max_batch_;
   return slots_[sample / cap]->wdl[3 * (sample % cap) + 1];
 }
 
 float Mi355xComputation::GetMVal(int sample) const {
   CheckSample(sample);
-  if (!net_->moves_left()) return 0.0f;
-  const int cap = net_->GetMaxBatchSize();
+  if (!moves_left_) return 0.0f;
+  const int cap = max_batch_;
   return slots_[sample / cap]->mlh[sample % cap];
 }
 

@@ -17,6 +17,8 @@ def _lib():
     if not getattr(lib, "_k_ready", False):
         vp, ci, ll, cf, cd = C.c_void_p, C.c_int, C.c_longlong, C.c_float, C.POINTER(C.c_double)
         lib.lc0mi_k_gemm.argtypes = [vp, ci, ll, vp, ci, ll, vp, ci, ci, ci, ci, cf, ci, ci, vp, ci, ll, ci, cd]
+        lib.lc0mi_k_gemm_splitk.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, ci, cf, vp, ci]
+        lib.lc0mi_k_layer_norm_rows.argtypes = [vp, vp, ci, vp, vp, vp, ci, ci, cf, cf, vp]
         lib.lc0mi_k_gemm_f32.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, ci, vp, ci]
         lib.lc0mi_k_layer_norm.argtypes = [vp, vp, vp, vp, ci, ci, cf, cf, vp, ci, cd]
         lib.lc0mi_k_attention.argtypes = [vp, vp, ci, ci, cf, vp, ci, cd]
@@ -56,6 +58,36 @@ def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
                                int(out_f32), _ptr(out), n, m * n, time_iters, C.byref(ms)))
     out = out if batched else out[0]
     return (out, ms.value) if time_iters else out
+
+
+def set_gemm_variant(variant):
+    """-1 automatic, 0..2 direct-to-LDS 256x{256,192,128} tiles, 3 128x128, 4 64x64."""
+    _lib().lc0mi_k_set_gemm_variant(int(variant))
+
+
+def gemm_splitk(a, w, bias=None, split_k=4, scale=1.0):
+    """a [M,K], w [N,K] -> float32 a @ w^T * scale + bias, reduced over split_k K-slices."""
+    a, w = _h(a), _h(w)
+    m, k = a.shape
+    n = w.shape[0]
+    out = np.zeros((m, n), np.float32)
+    b = np.ascontiguousarray(bias, np.float32) if bias is not None else None
+    _check(_lib().lc0mi_k_gemm_splitk(_ptr(a), k, _ptr(w), k, _ptr(b), m, n, k, split_k, scale, _ptr(out), n))
+    return out
+
+
+def layer_norm_rows(x, skip, gamma, beta, alpha, eps, pre_act=ACT_NONE, x_is_f32=False):
+    """One workgroup per row: LN(act(x) * alpha + skip)."""
+    xf = np.ascontiguousarray(x, np.float32) if x_is_f32 else None
+    xh = None if x_is_f32 else _h(x)
+    s = _h(skip) if skip is not None else None
+    g = np.ascontiguousarray(gamma, np.float32)
+    b = np.ascontiguousarray(beta, np.float32)
+    rows, c = np.shape(x)
+    y = np.zeros((rows, c), np.float16)
+    _check(_lib().lc0mi_k_layer_norm_rows(_ptr(xf), _ptr(xh), pre_act, _ptr(s), _ptr(g), _ptr(b), rows, c, alpha, eps,
+                                          _ptr(y)))
+    return y
 
 
 def gemm_f32(a, w, bias=None, scale=1.0, act=ACT_NONE):

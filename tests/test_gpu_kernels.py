@@ -43,6 +43,51 @@ def test_gemm_no_bias_scale_and_batched():
     np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
 
 
+@pytest.mark.parametrize("m,n,k,split", [(256, 256, 2048, 8), (37, 130, 520, 3), (64, 64, 64, 4), (300, 8, 4096, 16)])
+def test_gemm_splitk_vs_oracle_fc(m, n, k, split):
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(m + n + k)
+    a = _h(rng.standard_normal((m, k)) * 0.5)
+    w = _h(rng.standard_normal((n, k)) * 0.1)
+    b = rng.standard_normal(n).astype(f32)
+    got = K.gemm_splitk(a, w, b, split_k=split)
+    np.testing.assert_allclose(got, onn.fc(a, w.reshape(-1), b, nr.ACT_NONE), rtol=3e-4, atol=3e-4)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("m,n,k", [(2048, 1024, 256), (777, 200, 128), (300, 1858, 64), (64, 64, 192)])
+def test_every_gemm_variant_vs_oracle_fc(variant, m, n, k):
+    """Every tile variant (the three direct-to-LDS kernels and the two
+    register-staged ones) on full and ragged M / N."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(m + n)
+    a = _h(rng.standard_normal((m, k)) * 0.5)
+    w = _h(rng.standard_normal((n, k)) * 0.1)
+    b = rng.standard_normal(n).astype(f32)
+    K.set_gemm_variant(variant)
+    try:
+        got = K.gemm(a, w, b, act=nr.ACT_MISH).astype(f32)
+    finally:
+        K.set_gemm_variant(-1)
+    np.testing.assert_allclose(got, onn.fc(a, w.reshape(-1), b, nr.ACT_MISH), rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("rows,c,f32_in,act", [(256, 256, True, nr.ACT_SWISH), (256, 8192, False, nr.ACT_NONE),
+                                               (3, 32, True, nr.ACT_MISH), (17, 1024, False, nr.ACT_RELU)])
+def test_layer_norm_rows_vs_oracle(rows, c, f32_in, act):
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(rows * 3 + c)
+    x = rng.standard_normal((rows, c)).astype(f32)
+    if not f32_in:
+        x = _h(x)
+    s = _h(rng.standard_normal((rows, c)))
+    g = (1 + 0.1 * rng.standard_normal(c)).astype(f32)
+    b = (0.1 * rng.standard_normal(c)).astype(f32)
+    want = onn.layer_norm_skip(onn.activate(x, act), 0.7, s, g, b, 1e-3)
+    got = K.layer_norm_rows(x, s, g, b, 0.7, 1e-3, pre_act=act, x_is_f32=f32_in).astype(f32)
+    np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3)
+
+
 def test_gemm_f32_vs_oracle_fc():
     from lc0_amd import kernels as K
     rng = np.random.default_rng(2)
