@@ -56,6 +56,20 @@ int lc0mi_k_expand_planes_nchw(const uint64_t* masks, const float* values, int b
 int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const float* ppo, int pd, int batch,
                                float* out);
 
+/* One 3x3 convolution of the residual tower through the winograd F(4x4,3x3) path
+ * (input transform, 36 batched GEMMs, output transform with the fused tail):
+ *   out = act(conv(x) + bias (+ skip))                      when se_k == 0
+ *   out = ApplySEUnit(conv(x), bias, skip, w1,b1,w2,b2)     when se_k > 0
+ * (WinogradConvolution3::Forward + BiasActivate / BiasResidual / ApplySEUnit,
+ *  src/neural/backends/blas/winograd_convolution3.cc:47-324, se_unit.cc:31-91).
+ * x, skip, out: [B][64][C] floats (NHWC); filter: [cout][cin][3][3]; use_fp16 selects
+ * the half-precision kernels (operands rounded to fp16 on the way in). */
+int lc0mi_k_winograd_conv(const float* x, const float* filter, const float* bias, const float* skip,
+                          const float* se_w1, const float* se_b1, const float* se_w2, const float* se_b2, int se_k,
+                          int batch, int cin, int cout, int act, int use_fp16, float* out);
+/* Input planes -> [B][64][112] floats (NHWC form of EncodePlanes). */
+int lc0mi_k_expand_planes_nhwc(const uint64_t* masks, const float* values, int batch, float* out);
+
 #ifdef __cplusplus
 }
 #endif

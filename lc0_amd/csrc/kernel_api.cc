@@ -293,4 +293,96 @@ int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const 
   });
 }
 
+
+}  // extern "C"
+
+namespace {
+template <typename T>
+void WinogradConvHost(const float* x, const float* filter, const float* bias, const float* skip, const float* se_w1,
+                      const float* se_b1, const float* se_w2, const float* se_b2, int se_k, int batch, int cin,
+                      int cout, int act, float* out) {
+  Dev dev;
+  const int ld = (cin + 7) / 8 * 8;
+  const size_t nx = (size_t)batch * 64 * cin, no = (size_t)batch * 64 * cout;
+  std::vector<T> hx(nx);
+  for (size_t i = 0; i < nx; i++) hx[i] = (T)x[i];
+  T* dx = dev.Put(hx.data(), nx);
+  T* dskip = nullptr;
+  if (skip) {
+    std::vector<T> hs(no);
+    for (size_t i = 0; i < no; i++) hs[i] = (T)skip[i];
+    dskip = dev.Put(hs.data(), no);
+  }
+  std::vector<float> u((size_t)36 * cout * ld);
+  lc0mi::WinogradFilterTransform4x4(filter, cout, cin, ld, u.data());
+  std::vector<T> ut(u.size());
+  for (size_t i = 0; i < u.size(); i++) ut[i] = (T)u[i];
+  T* du = dev.Put(ut.data(), ut.size());
+  float* dbias = dev.Put(bias, (size_t)cout);
+  float *w1 = nullptr, *b1 = nullptr, *w2 = nullptr, *b2 = nullptr;
+  if (se_k > 0) {
+    w1 = dev.Put(se_w1, (size_t)se_k * cout); b1 = dev.Put(se_b1, (size_t)se_k);
+    w2 = dev.Put(se_w2, (size_t)2 * cout * se_k); b2 = dev.Put(se_b2, (size_t)2 * cout);
+  }
+  const int tiles = batch * 4;
+  T* dv = static_cast<T*>(dev.Alloc(sizeof(T) * 36 * tiles * ld));
+  K_CHECK(hipMemset(dv, 0, sizeof(T) * 36 * tiles * ld));
+  float* dm = static_cast<float*>(dev.Alloc(sizeof(float) * 36 * tiles * cout));
+  T* dout = static_cast<T*>(dev.Alloc(sizeof(T) * no));
+  lc0mi::LaunchWinogradInputTransform<T>(dx, dv, batch, cin, ld, nullptr);
+  if constexpr (sizeof(T) == 2) {
+    lc0mi::GemmArgs g;
+    g.A = dv; g.lda = ld; g.strideA = (long long)tiles * ld;
+    g.W = du; g.ldw = ld; g.strideW = (long long)cout * ld;
+    g.C = dm; g.ldc = cout; g.strideC = (long long)tiles * cout;
+    g.M = tiles; g.N = cout; g.K = ld; g.batch = 36; g.out_f32 = true;
+    lc0mi::LaunchGemm(g, nullptr);
+  } else {
+    lc0mi::GemmArgsF32 g;
+    g.A = dv; g.lda = ld; g.strideA = (long long)tiles * ld;
+    g.W = du; g.ldw = ld; g.strideW = (long long)cout * ld;
+    g.C = dm; g.ldc = cout; g.strideC = (long long)tiles * cout;
+    g.M = tiles; g.N = cout; g.K = ld; g.batch = 36;
+    lc0mi::LaunchGemmF32(g, nullptr);
+  }
+  lc0mi::LaunchWinogradOutputTransform<T, float>(dm, dbias, dskip, w1, b1, w2, b2, se_k, dout, batch, cout, act, nullptr);
+  K_CHECK(hipDeviceSynchronize());
+  K_CHECK(hipGetLastError());
+  std::vector<T> ho(no);
+  K_CHECK(hipMemcpy(ho.data(), dout, sizeof(T) * no, hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < no; i++) out[i] = (float)ho[i];
+}
+}  // namespace
+
+extern "C" {
+
+int lc0mi_k_winograd_conv(const float* x, const float* filter, const float* bias, const float* skip,
+                          const float* se_w1, const float* se_b1, const float* se_w2, const float* se_b2, int se_k,
+                          int batch, int cin, int cout, int act, int use_fp16, float* out) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1 || cin < 1 || cout < 1 || cout > 1024 || se_k < 0 || se_k > 256) throw Error("bad convolution shape");
+    if (use_fp16) {
+      WinogradConvHost<half_t>(x, filter, bias, skip, se_w1, se_b1, se_w2, se_b2, se_k, batch, cin, cout, act, out);
+    } else {
+      WinogradConvHost<float>(x, filter, bias, skip, se_w1, se_b1, se_w2, se_b2, se_k, batch, cin, cout, act, out);
+    }
+  });
+}
+
+int lc0mi_k_expand_planes_nhwc(const uint64_t* masks, const float* values, int batch, float* out) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1) throw Error("bad expand shape");
+    Dev dev;
+    uint64_t* dm = dev.Put(masks, (size_t)batch * 112);
+    float* dv = dev.Put(values, (size_t)batch * 112);
+    auto* dout = static_cast<float*>(dev.Alloc((size_t)batch * 64 * 112 * 4));
+    lc0mi::LaunchExpandPlanesNhwc<float>(dm, dv, dout, batch, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(out, dout, (size_t)batch * 64 * 112 * 4, hipMemcpyDeviceToHost));
+  });
+}
+
 }  // extern "C"

@@ -95,3 +95,43 @@ void LaunchAttnPolicyGather(const float* logits, const half_t* kq, int ld_kq, in
                             int pd, const int16_t* inv_map, float* out, int batch, hipStream_t stream);
 
 }  // namespace lc0mi
+
+// ---------------------------------------------------------------------------
+// SE-ResNet tower: winograd F(4x4,3x3) convolution on the 8x8 board.
+// Activations are NHWC: x[b][sq][c]. T = half_t or float.
+// ---------------------------------------------------------------------------
+namespace lc0mi {
+
+// Input planes -> out[b][sq][c], c < 112 (T = half_t or float).
+template <typename T>
+void LaunchExpandPlanesNhwc(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream);
+
+// Host side: filter [cout][cin][3][3] -> U[36][cout][ld_cin] = (G g G^T), with the
+// row-scaled G = diag(4,6,6,24,24,1) * G_lavin (integer entries); ld_cin >= cin is the
+// zero-padded row length.
+void WinogradFilterTransform4x4(const float* filter, int cout, int cin, int ld_cin, float* u);
+
+// V[k][b*4+t][c] = (B^T d B)[k] of the 6x6 input patch of tile t (2x2 tiles of 4x4
+// outputs, zero padding), with B^T row-scaled by 1/diag(4,6,6,24,24,1).
+// x: [B][64][C], v: [36][B*4][ldv].
+template <typename T>
+void LaunchWinogradInputTransform(const T* x, T* v, int batch, int C, int ldv, hipStream_t stream);
+
+// Output transform y = A^T m A per tile with the fused tail of a residual block:
+//   plain:  out = act(y + bias (+ skip))
+//   SE:     pool = mean64(y) + bias; h = act(W1 pool + b1); s = W2 h + b2;
+//           gamma = sigmoid(s[0:C]); beta = s[C:2C] + gamma * bias;
+//           out = act(gamma * y + skip + beta)
+// m: [36][B*4][C] (M_IS_F32 selects float m for T = half_t), out/skip: [B][64][C].
+// se_w1: [K][C], se_w2: [2C][K] floats. C <= 1024, K <= 256.
+template <typename T, typename MT>
+void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip, const float* se_w1,
+                                   const float* se_b1, const float* se_w2, const float* se_b2, int se_k, T* out,
+                                   int batch, int C, int act, hipStream_t stream);
+
+// Gather of the convolutional policy head: out[b][j] = t[b][sq][plane] for
+// kConvPolicyMap[plane*64+sq] = j. t: [B][64][ld] (NHWC), inv_map: [1858] holding plane*64+sq.
+template <typename T>
+void LaunchConvPolicyGather(const T* t, int ld, const int16_t* inv_map, float* out, int batch, hipStream_t stream);
+
+}  // namespace lc0mi

@@ -119,6 +119,27 @@ struct Linear {
 
 int RoundUp(int v, int m) { return (v + m - 1) / m * m; }
 
+// Residual-tower device weights (element type chosen by the precision option).
+struct ConvDev {
+  void* u = nullptr;      // [36][cout][ld] winograd-domain filter
+  float* bias = nullptr;  // [cout]
+  int cin = 0, cout = 0, ld = 0;
+};
+struct SeDev {
+  float *w1 = nullptr, *b1 = nullptr, *w2 = nullptr, *b2 = nullptr;
+  int k = 0;
+};
+struct ResBlockDev {
+  ConvDev conv1, conv2;
+  bool has_se = false;
+  SeDev se;
+};
+struct LinearT {
+  void* w = nullptr;      // [out][ld]
+  float* b = nullptr;
+  int out = 0, in = 0, ld = 0;
+};
+
 struct EncoderDev {
   Linear qkv, dense, ffn1, ffn2;
   float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
@@ -215,8 +236,21 @@ class Mi355xNetwork : public Network {
 
  private:
   void BuildAttentionBody(const WeightsFile& file);
+  template <typename T>
+  void BuildResnet(const WeightsFile& file);
   void ForwardDevice(int batch);
   void ForwardAttentionBody(int B);
+  template <typename T>
+  void ForwardResnet(int B);
+  template <typename T>
+  void WinogradConv(const char* name, const struct ConvDev& conv, const void* x, const void* skip, const struct SeDev* se,
+                    int act, void* out, int B);
+  template <typename T>
+  void GemmT(const char* name, const void* A, int lda, long long strideA, const void* W, int ldw, long long strideW,
+             void* C, int ldc, long long strideC, const float* bias, int M, int N, int K, int batch, int act,
+             bool out_f32);
+  template <typename T>
+  struct LinearT MakeLinearT(const Vec& w, const Vec& b, int out, int in);
   Linear MakeLinear(const Vec& w, const Vec& b, int out, int in);
   float* UploadF(const Vec& v) { return arena_.Upload(v); }
   half_t* AllocH(size_t n) { return static_cast<half_t*>(arena_.Alloc(n * sizeof(half_t))); }
@@ -264,6 +298,18 @@ class Mi355xNetwork : public Network {
   float* sg2f_ = nullptr;  // split-K accumulator of smolgen dense1
   half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
   float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
+
+  // Residual tower.
+  bool fp32_ = false;
+  int filters_ = 0;
+  bool classical_value_ = false;
+  ConvDev res_input_, res_policy1_, res_policy_conv_;
+  std::vector<ResBlockDev> res_blocks_;
+  LinearT res_pol_conv1x1_, res_pol_fc_, res_val_conv_, res_val_fc1_, res_val_fc2_, res_mov_conv_, res_mov_fc1_,
+      res_mov_fc2_;
+  int16_t* conv_inv_map_ = nullptr;
+  void *r_in_ = nullptr, *r_x_ = nullptr, *r_y_ = nullptr, *r_v_ = nullptr, *r_m_ = nullptr, *r_h1_ = nullptr,
+       *r_h2_ = nullptr;
 
   // Profiling.
   bool profiling_ = false;
@@ -376,7 +422,10 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   max_batch_ = options.GetInt("max_batch", 1024);
   if (max_batch_ < 1 || max_batch_ > 4096) throw Error("max_batch must be in 1..4096.");
   const std::string precision = options.GetString("precision", "fp16");
-  if (precision != "fp16") throw Error("Precision '" + precision + "' is not supported (fp16 only).");
+  if (precision != "fp16" && precision != "fp32") {
+    throw Error("Precision '" + precision + "' is not supported (fp16 or fp32).");
+  }
+  fp32_ = precision == "fp32";
   policy_head_ = options.GetString("policy_head", "vanilla");
   value_head_ = options.GetString("value_head", "winner");
   wdl_ = nf.value == kValueWdl;
@@ -414,9 +463,12 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   d_mlh_ = AllocF(max_batch_);
 
   if (attn_body_) {
+    if (fp32_) throw Error("precision=fp32 is available for residual-tower networks only.");
     BuildAttentionBody(file);
+  } else if (fp32_) {
+    BuildResnet<float>(file);
   } else {
-    throw Error("Only attention-body networks are supported by this build of the mi355x backend.");
+    BuildResnet<half_t>(file);
   }
   HIP_CHECK(hipStreamSynchronize(stream_));
 }
@@ -587,6 +639,217 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   head2_ = AllocH(static_cast<size_t>(max_batch_) * std::max(val_fc_, mov_fc_));
 }
 
+
+// ------------------------------------------------------------ residual tower --
+template <typename T>
+LinearT Mi355xNetwork::MakeLinearT(const Vec& w, const Vec& b, int out, int in) {
+  if (static_cast<size_t>(out) * in != w.size()) {
+    throw Error("Weight tensor has " + std::to_string(w.size()) + " elements, expected " + std::to_string(out) +
+                " x " + std::to_string(in) + ".");
+  }
+  if (!b.empty() && static_cast<int>(b.size()) != out) throw Error("Bias size does not match the layer width.");
+  LinearT l;
+  l.out = out; l.in = in; l.ld = RoundUp(in, 8);
+  std::vector<T> h(static_cast<size_t>(out) * l.ld, (T)0.0f);
+  for (int o = 0; o < out; o++)
+    for (int i = 0; i < in; i++) h[static_cast<size_t>(o) * l.ld + i] = (T)w[static_cast<size_t>(o) * in + i];
+  l.w = arena_.Upload(h);
+  if (!b.empty()) l.b = arena_.Upload(b);
+  return l;
+}
+
+template <typename T>
+void Mi355xNetwork::GemmT(const char* name, const void* A, int lda, long long strideA, const void* W, int ldw,
+                          long long strideW, void* C, int ldc, long long strideC, const float* bias, int M, int N,
+                          int K, int batch, int act, bool out_f32) {
+  const double flops = 2.0 * M * N * K * batch;
+  const double bytes = sizeof(T) * batch * (static_cast<double>(M) * K + static_cast<double>(N) * K) +
+                       static_cast<double>(batch) * M * N * (out_f32 ? 4 : sizeof(T));
+  if constexpr (sizeof(T) == 2) {
+    GemmArgs g;
+    g.A = static_cast<const half_t*>(A); g.lda = lda; g.strideA = strideA;
+    g.W = static_cast<const half_t*>(W); g.ldw = ldw; g.strideW = strideW;
+    g.C = C; g.ldc = ldc; g.strideC = strideC;
+    g.bias = bias; g.M = M; g.N = N; g.K = K; g.batch = batch; g.act = act; g.out_f32 = out_f32;
+    const std::string label = std::string(name) + "|" + GemmVariantName(g);
+    Timed(label.c_str(), flops, bytes, [&] { LaunchGemm(g, stream_); });
+  } else {
+    GemmArgsF32 g;
+    g.A = static_cast<const float*>(A); g.lda = lda; g.strideA = strideA;
+    g.W = static_cast<const float*>(W); g.ldw = ldw; g.strideW = strideW;
+    g.C = static_cast<float*>(C); g.ldc = ldc; g.strideC = strideC;
+    g.bias = bias; g.M = M; g.N = N; g.K = K; g.batch = batch; g.act = act;
+    const std::string label = std::string(name) + "|gemm_f32_64x64x16";
+    Timed(label.c_str(), flops, bytes, [&] { LaunchGemmF32(g, stream_); });
+  }
+}
+
+template <typename T>
+void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
+  const NetWeights& w = file.weights;
+  const NetworkFormat& nf = file.format;
+  if (attn_policy_) throw Error("The attention policy head on a residual tower is not supported.");
+  if (w.residual.empty() && w.input.weights.empty()) throw Error("Network has no input convolution.");
+  const PolicyHead& ph = w.policy_heads.at(policy_head_);
+  const ValueHead& vh = w.value_heads.at(value_head_);
+  filters_ = static_cast<int>(w.input.biases.size());
+  if (filters_ <= 0 || filters_ % 8 != 0 || filters_ > 1024) {
+    throw Error("The number of filters must be a multiple of 8 in 8..1024.");
+  }
+  classical_value_ = nf.value == kValueClassical;
+
+  auto make_conv = [&](const ConvBlock& cb, int cout, int cin) {
+    if (cb.weights.size() != static_cast<size_t>(cout) * cin * 9 || static_cast<int>(cb.biases.size()) != cout) {
+      throw Error("3x3 convolution weights have an unexpected size.");
+    }
+    ConvDev c;
+    c.cin = cin; c.cout = cout; c.ld = RoundUp(cin, 8);
+    std::vector<float> u(static_cast<size_t>(36) * cout * c.ld);
+    WinogradFilterTransform4x4(cb.weights.data(), cout, cin, c.ld, u.data());
+    std::vector<T> ut(u.size());
+    for (size_t i = 0; i < u.size(); i++) ut[i] = (T)u[i];
+    c.u = arena_.Upload(ut);
+    c.bias = arena_.Upload(cb.biases);
+    return c;
+  };
+  res_input_ = make_conv(w.input, filters_, kInputPlanes);
+  for (const Residual& r : w.residual) {
+    ResBlockDev b;
+    b.conv1 = make_conv(r.conv1, filters_, filters_);
+    b.conv2 = make_conv(r.conv2, filters_, filters_);
+    b.has_se = r.has_se;
+    if (r.has_se) {
+      b.se.k = static_cast<int>(r.se.b1.size());
+      if (b.se.k <= 0 || b.se.k > 256 || r.se.w1.size() != static_cast<size_t>(b.se.k) * filters_ ||
+          r.se.w2.size() != static_cast<size_t>(2) * filters_ * b.se.k || r.se.b2.size() != 2u * filters_) {
+        throw Error("SE unit weights have an unexpected size.");
+      }
+      b.se.w1 = arena_.Upload(r.se.w1); b.se.b1 = arena_.Upload(r.se.b1);
+      b.se.w2 = arena_.Upload(r.se.w2); b.se.b2 = arena_.Upload(r.se.b2);
+    }
+    res_blocks_.push_back(b);
+  }
+
+  // A dense layer fed by a flattened [C][64] head tensor: this backend keeps heads as
+  // [64][C], so the columns are reordered once here (c*64+sq -> sq*C+c).
+  auto make_fc_from_nchw = [&](const Vec& fw, const Vec& fb, int out, int channels) {
+    if (fw.size() != static_cast<size_t>(out) * channels * 64) throw Error("Head dense layer has an unexpected size.");
+    Vec perm(fw.size());
+    for (int o = 0; o < out; o++)
+      for (int c = 0; c < channels; c++)
+        for (int sq = 0; sq < 64; sq++)
+          perm[(static_cast<size_t>(o) * 64 + sq) * channels + c] = fw[(static_cast<size_t>(o) * channels + c) * 64 + sq];
+    return MakeLinearT<T>(perm, fb, out, channels * 64);
+  };
+  auto make_conv1x1 = [&](const ConvBlock& cb, int cin) {
+    const int cout = static_cast<int>(cb.biases.size());
+    if (cout <= 0 || cout % 8 != 0 || cb.weights.size() != static_cast<size_t>(cout) * cin) {
+      throw Error("1x1 head convolution has an unexpected size.");
+    }
+    return MakeLinearT<T>(cb.weights, cb.biases, cout, cin);
+  };
+
+  int max_head_ch = 8;
+  if (conv_policy_) {
+    res_policy1_ = make_conv(ph.policy1, filters_, filters_);
+    const int pol_out = static_cast<int>(ph.policy.biases.size());
+    if (pol_out < 73 || pol_out > 1024) throw Error("Convolutional policy head has an unexpected size.");
+    res_policy_conv_ = make_conv(ph.policy, pol_out, filters_);
+    conv_inv_map_ = arena_.Upload(ConvPolicyInverseMap());
+    max_head_ch = std::max(max_head_ch, pol_out);
+  } else {
+    res_pol_conv1x1_ = make_conv1x1(ph.policy, filters_);
+    res_pol_fc_ = make_fc_from_nchw(ph.ip_pol_w, ph.ip_pol_b, kPolicyOutputs, res_pol_conv1x1_.out);
+    max_head_ch = std::max(max_head_ch, res_pol_conv1x1_.out);
+  }
+  res_val_conv_ = make_conv1x1(vh.value, filters_);
+  val_fc_ = static_cast<int>(vh.ip1_val_b.size());
+  val_out_ = wdl_ ? 3 : 1;
+  if (val_fc_ <= 0 || val_fc_ % 8) throw Error("Unsupported value head sizes.");
+  res_val_fc1_ = make_fc_from_nchw(vh.ip1_val_w, vh.ip1_val_b, val_fc_, res_val_conv_.out);
+  res_val_fc2_ = MakeLinearT<T>(vh.ip2_val_w, vh.ip2_val_b, val_out_, val_fc_);
+  max_head_ch = std::max(max_head_ch, res_val_conv_.out);
+  int max_fc = val_fc_;
+  if (moves_left_) {
+    res_mov_conv_ = make_conv1x1(w.moves_left, filters_);
+    mov_fc_ = static_cast<int>(w.ip1_mov_b.size());
+    if (mov_fc_ <= 0 || mov_fc_ % 8) throw Error("Unsupported moves-left head sizes.");
+    res_mov_fc1_ = make_fc_from_nchw(w.ip1_mov_w, w.ip1_mov_b, mov_fc_, res_mov_conv_.out);
+    res_mov_fc2_ = MakeLinearT<T>(w.ip2_mov_w, w.ip2_mov_b, 1, mov_fc_);
+    max_head_ch = std::max(max_head_ch, res_mov_conv_.out);
+    max_fc = std::max(max_fc, mov_fc_);
+  }
+
+  const size_t B = static_cast<size_t>(max_batch_);
+  const size_t cmax = static_cast<size_t>(std::max(filters_, max_head_ch));
+  r_in_ = arena_.Alloc(sizeof(T) * B * 64 * kInputPlanes);
+  r_x_ = arena_.Alloc(sizeof(T) * B * 64 * cmax);
+  r_y_ = arena_.Alloc(sizeof(T) * B * 64 * cmax);
+  r_v_ = arena_.Alloc(sizeof(T) * 36 * B * 4 * std::max<size_t>(filters_, kInputPlanes));
+  r_m_ = arena_.Alloc(sizeof(float) * 36 * B * 4 * cmax);
+  r_h1_ = arena_.Alloc(sizeof(T) * B * 64 * cmax);
+  r_h2_ = arena_.Alloc(sizeof(T) * B * static_cast<size_t>(max_fc));
+}
+
+// One 3x3 convolution: input transform, 36 batched GEMMs, output transform with the fused tail.
+template <typename T>
+void Mi355xNetwork::WinogradConv(const char* name, const ConvDev& conv, const void* x, const void* skip,
+                                 const SeDev* se, int act, void* out, int B) {
+  const int tiles = B * 4;
+  Timed("winograd_input_transform", 0.0, sizeof(T) * B * (64.0 + 144.0) * conv.cin, [&] {
+    LaunchWinogradInputTransform<T>(static_cast<const T*>(x), static_cast<T*>(r_v_), B, conv.cin, conv.ld, stream_);
+  });
+  // Winograd-domain products are kept in float when the tower runs in fp16: the output
+  // transform sums 36 of them with weights up to 64.
+  constexpr bool kHalf = sizeof(T) == 2;
+  GemmT<T>(name, r_v_, conv.ld, static_cast<long long>(tiles) * conv.ld, conv.u, conv.ld,
+           static_cast<long long>(conv.cout) * conv.ld, r_m_, conv.cout, static_cast<long long>(tiles) * conv.cout,
+           nullptr, tiles, conv.cout, conv.ld, 36, kActNone, /*out_f32=*/kHalf);
+  Timed("winograd_output_transform", 0.0, B * conv.cout * (144.0 * 4 + sizeof(T) * 64.0 * (skip ? 2 : 1)), [&] {
+    LaunchWinogradOutputTransform<T, float>(static_cast<const float*>(r_m_), conv.bias, static_cast<const T*>(skip),
+                                            se ? se->w1 : nullptr, se ? se->b1 : nullptr, se ? se->w2 : nullptr,
+                                            se ? se->b2 : nullptr, se ? se->k : 0, static_cast<T*>(out), B, conv.cout,
+                                            act, stream_);
+  });
+}
+
+template <typename T>
+void Mi355xNetwork::ForwardResnet(int B) {
+  const int T64 = B * 64;
+  Timed("expand_planes", 0.0, B * (112.0 * 12 + sizeof(T) * 64.0 * 112), [&] {
+    LaunchExpandPlanesNhwc<T>(d_masks_, d_values_, static_cast<T*>(r_in_), B, stream_);
+  });
+  WinogradConv<T>("gemm_winograd_input", res_input_, r_in_, nullptr, nullptr, default_act_, r_x_, B);
+  for (const ResBlockDev& blk : res_blocks_) {
+    WinogradConv<T>("gemm_winograd", blk.conv1, r_x_, nullptr, nullptr, default_act_, r_y_, B);
+    WinogradConv<T>("gemm_winograd", blk.conv2, r_y_, r_x_, blk.has_se ? &blk.se : nullptr, default_act_, r_x_, B);
+  }
+  auto fc = [&](const char* name, const void* a, const LinearT& l, void* c, int m, int act, bool out_f32) {
+    GemmT<T>(name, a, l.ld, 0, l.w, l.ld, 0, c, l.out, 0, l.b, m, l.out, l.ld, 1, act, out_f32);
+  };
+  // Value head.
+  fc("gemm_value_conv", r_x_, res_val_conv_, r_h1_, T64, default_act_, false);
+  fc("gemm_value_fc1", r_h1_, res_val_fc1_, r_h2_, B, default_act_, false);
+  fc("gemm_value_fc2", r_h2_, res_val_fc2_, d_wdl_, B, kActNone, true);
+  if (moves_left_) {
+    fc("gemm_mlh_conv", r_x_, res_mov_conv_, r_h1_, T64, default_act_, false);
+    fc("gemm_mlh_fc1", r_h1_, res_mov_fc1_, r_h2_, B, default_act_, false);
+    fc("gemm_mlh_fc2", r_h2_, res_mov_fc2_, d_mlh_, B, kActRelu, true);
+  }
+  // Policy head.
+  if (conv_policy_) {
+    WinogradConv<T>("gemm_winograd_policy", res_policy1_, r_x_, nullptr, nullptr, default_act_, r_y_, B);
+    WinogradConv<T>("gemm_winograd_policy", res_policy_conv_, r_y_, nullptr, nullptr, kActNone, r_h1_, B);
+    Timed("policy_gather", 0.0, B * (sizeof(T) * 73.0 * 64 + 4.0 * 1858), [&] {
+      LaunchConvPolicyGather<T>(static_cast<const T*>(r_h1_), res_policy_conv_.cout, conv_inv_map_, d_policy_, B,
+                                stream_);
+    });
+  } else {
+    fc("gemm_policy_conv", r_x_, res_pol_conv1x1_, r_h1_, T64, default_act_, false);
+    fc("gemm_policy_fc", r_h1_, res_pol_fc_, d_policy_, B, kActNone, true);
+  }
+}
+
 // ------------------------------------------------------------------ forward --
 void Mi355xNetwork::ForwardAttentionBody(int B) {
   const int T = B * 64;
@@ -672,7 +935,13 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
 }
 
 void Mi355xNetwork::ForwardDevice(int batch) {
-  if (attn_body_) ForwardAttentionBody(batch);
+  if (attn_body_) {
+    ForwardAttentionBody(batch);
+  } else if (fp32_) {
+    ForwardResnet<float>(batch);
+  } else {
+    ForwardResnet<half_t>(batch);
+  }
 }
 
 void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {

@@ -19,6 +19,8 @@ def _lib():
         lib.lc0mi_k_gemm.argtypes = [vp, ci, ll, vp, ci, ll, vp, ci, ci, ci, ci, cf, ci, ci, vp, ci, ll, ci, cd]
         lib.lc0mi_k_gemm_splitk.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, ci, cf, vp, ci]
         lib.lc0mi_k_layer_norm_rows.argtypes = [vp, vp, ci, vp, vp, vp, ci, ci, cf, cf, vp]
+        lib.lc0mi_k_winograd_conv.argtypes = [vp] * 8 + [ci] * 6 + [vp]
+        lib.lc0mi_k_expand_planes_nhwc.argtypes = [vp, vp, ci, vp]
         lib.lc0mi_k_gemm_f32.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, ci, vp, ci]
         lib.lc0mi_k_layer_norm.argtypes = [vp, vp, vp, vp, ci, ci, cf, cf, vp, ci, cd]
         lib.lc0mi_k_attention.argtypes = [vp, vp, ci, ci, cf, vp, ci, cd]
@@ -150,4 +152,33 @@ def attn_policy_gather(logits, keys, ppo):
     n = logits.shape[0]
     out = np.zeros((n, 1858), np.float32)
     _check(_lib().lc0mi_k_attn_policy_gather(_ptr(logits), _ptr(keys), _ptr(ppo), keys.shape[1], n, _ptr(out)))
+    return out
+
+
+def winograd_conv(x, filt, bias, skip=None, se=None, act=ACT_RELU, fp16=False):
+    """x [B,64,Cin] (NHWC), filt [Cout,Cin,3,3], se = (w1 [K,C], b1, w2 [2C,K], b2) or None -> [B,64,Cout]."""
+    x = np.ascontiguousarray(x, np.float32)
+    filt = np.ascontiguousarray(filt, np.float32)
+    bias = np.ascontiguousarray(bias, np.float32)
+    b, _, cin = x.shape
+    cout = filt.shape[0]
+    sk = np.ascontiguousarray(skip, np.float32) if skip is not None else None
+    if se is not None:
+        w1, b1, w2, b2 = [np.ascontiguousarray(a, np.float32) for a in se]
+        k = w1.shape[0]
+    else:
+        w1 = b1 = w2 = b2 = None
+        k = 0
+    out = np.zeros((b, 64, cout), np.float32)
+    _check(_lib().lc0mi_k_winograd_conv(_ptr(x), _ptr(filt), _ptr(bias), _ptr(sk), _ptr(w1), _ptr(b1), _ptr(w2),
+                                        _ptr(b2), k, b, cin, cout, act, int(fp16), _ptr(out)))
+    return out
+
+
+def expand_planes_nhwc(masks, values):
+    masks = np.ascontiguousarray(masks, np.uint64)
+    values = np.ascontiguousarray(values, np.float32)
+    n = masks.shape[0]
+    out = np.zeros((n, 64, 112), np.float32)
+    _check(_lib().lc0mi_k_expand_planes_nhwc(_ptr(masks), _ptr(values), n, _ptr(out)))
     return out

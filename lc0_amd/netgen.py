@@ -159,6 +159,8 @@ CONFIGS = {
     "c3_resnet_20x256": lambda: se_resnet(256, 20, 64, seed=1003),
     # tiny nets for fast parity tests
     "tiny_resnet": lambda: se_resnet(32, 2, 8, seed=2000, moves_left=True),
+    "tiny_resnet_convpolicy": lambda: se_resnet(32, 2, 8, seed=2003, conv_policy=True),
+    "tiny_resnet_nose": lambda: se_resnet(24, 3, 0, seed=2004, moves_left=True),
     "tiny_attn": lambda: attention_body(64, 2, 2, 96, seed=2001, smolgen=(8, 32, 32), perturb_ln=True),
     "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True),
 }

@@ -170,3 +170,43 @@ def test_attn_policy_gather_vs_oracle():
     plain = onn.ATTN_POLICY_MAP[:4096]
     ps = plain >= 0
     assert np.array_equal(got[:, plain[ps]], logits.reshape(B, 4096)[:, ps])
+
+
+@pytest.mark.parametrize("fp16", [False, True])
+@pytest.mark.parametrize("batch,cin,cout,se_k,with_skip", [(3, 112, 32, 0, False), (2, 32, 32, 8, True),
+                                                            (5, 64, 64, 16, True), (2, 16, 80, 0, False),
+                                                            (1, 24, 24, 0, True)])
+def test_winograd_conv_vs_oracle(batch, cin, cout, se_k, with_skip, fp16):
+    """F(4x4,3x3) convolution with its fused tail against the oracle's convolution
+    (itself checked against direct 3x3 correlation) and ApplySEUnit."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(batch + cin + cout + se_k)
+    rnd = (lambda a: _h(a)) if fp16 else (lambda a: np.asarray(a, f32))
+    x = rnd(rng.standard_normal((batch, cin, 8, 8)))                 # NCHW for the oracle
+    filt = rnd(rng.standard_normal((cout, cin, 3, 3)) * (cin * 9) ** -0.5)
+    bias = (0.1 * rng.standard_normal(cout)).astype(f32)
+    skip = rnd(rng.standard_normal((batch, cout, 64))) if with_skip else None
+    u = onn.winograd_filter_transform(filt, cout, cin)
+    y = onn.winograd_conv3(x, u, cin, cout).reshape(batch, cout, 64)
+    if se_k:
+        se = (rng.standard_normal((se_k, cout)).astype(f32) * 0.3, rng.standard_normal(se_k).astype(f32) * 0.1,
+              rng.standard_normal((2 * cout, se_k)).astype(f32) * 0.3, rng.standard_normal(2 * cout).astype(f32) * 0.1)
+        want = onn.apply_se_unit(y, bias, skip if with_skip else np.zeros_like(y), *se, nr.ACT_RELU)
+    else:
+        se = None
+        t = y + bias[None, :, None]
+        if with_skip:
+            t = t + skip
+        want = onn.activate(t, nr.ACT_RELU)
+    got = K.winograd_conv(x.reshape(batch, cin, 64).transpose(0, 2, 1), filt, bias,
+                          skip.transpose(0, 2, 1) if with_skip else None, se, act=nr.ACT_RELU, fp16=fp16)
+    tol = 2e-2 if fp16 else 2e-4   # fp16: transformed operands are rounded to 11 bits
+    np.testing.assert_allclose(got.transpose(0, 2, 1), want, rtol=tol, atol=tol)
+
+
+def test_expand_planes_nhwc_bit_exact():
+    from lc0_amd import kernels as K
+    from oracle import chess as oc
+    pos = oc.random_positions(9, seed=6)
+    want = onn.encode_planes(pos["masks"], pos["values"]).transpose(0, 2, 1)
+    assert np.array_equal(K.expand_planes_nhwc(pos["masks"], pos["values"]), want)

@@ -43,6 +43,7 @@ def _compare(res, want, legal, tol=TOL):
                  wdl_q=np.abs(res["q"] - (want["wdl"][:, 0] - want["wdl"][:, 2])).max(),
                  wdl_d=np.abs(res["d"] - want["wdl"][:, 1]).max(),
                  mlh_rel=(np.abs(res["m"] - want["m"]) / np.maximum(np.abs(want["m"]), 1.0)).max())
+    stats["m_max"] = float(np.abs(want["m"]).max())
     legal_err = 0.0
     top1 = 0
     for i, lg in enumerate(legal):
@@ -79,6 +80,19 @@ def test_attention_nets_match_oracle(name, batch, positions):
     np.testing.assert_allclose(comp.GetPVal(0, 100), res["policy"][3, 100], rtol=0, atol=2e-3)
     np.testing.assert_allclose(comp.GetQVal(0), res["q"][3], atol=2e-3)
     np.testing.assert_allclose(comp.GetDVal(0) + 0 * comp.GetMVal(0), res["d"][3], atol=2e-3)
+
+
+@pytest.mark.parametrize("name,batch,options,tol", [
+    ("tiny_resnet", 19, "precision=fp32", 1e-3), ("tiny_resnet", 19, "precision=fp16", 5e-3),
+    ("tiny_resnet_convpolicy", 8, "precision=fp32", 1e-3), ("tiny_resnet_nose", 8, "precision=fp32", 1e-3),
+    ("c0_resnet_6x64", 32, "precision=fp32", 1e-3), ("c0_resnet_6x64", 32, "precision=fp16", 5e-3)])
+def test_residual_tower_nets_match_oracle(name, batch, options, tol, positions):
+    """SE-ResNet family through the winograd F(4x4,3x3) path; configs[0] in fp32 within 1e-3."""
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    net, res = _run_gpu(path, masks, values, options)
+    _compare(res, want, positions["legal"][:batch], tol=tol)
 
 
 @pytest.mark.timeout(900)
