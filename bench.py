@@ -24,6 +24,9 @@ WORKLOADS = {
     "c2_bt4_15x1024": dict(batch=256, desc="BT4-shape attention body: 15 layers, d=1024, 32 heads, dff 1536, "
                                            "smolgen 32/256/256, fp16 with fp32 accumulation"),
     "c1_attn_10x256": dict(batch=64, desc="attention body: 10 layers, d=256, 8 heads, dff 1024, fp16"),
+    "c0_resnet_6x64": dict(batch=32, options="precision=fp32", dtype="fp32",
+                           desc="SE-ResNet 6x64, SE ratio 4, classical policy, WDL, fp32"),
+    "c3_resnet_20x256": dict(batch=512, desc="SE-ResNet 20x256, SE ratio 4, winograd F(4x4,3x3), fp16"),
     "tiny_attn": dict(batch=64, desc="tiny smolgen attention body (test net)"),
 }
 
@@ -74,7 +77,7 @@ def main():
     pos = oc.random_positions(max(batch, args.cpu_sample), seed=20240)
     masks, values = pos["masks"], pos["values"]
 
-    net = Network(path, "gpu=0,max_batch=%d" % max(batch, 16))
+    net = Network(path, "gpu=0,max_batch=%d" % max(batch, 16) + ("," + wl["options"] if wl.get("options") else ""))
     comp = net.NewComputation()
     comp.AddInputs(masks[:batch], values[:batch])
     comp.ComputeBlocking()          # stages the batch into HBM and warms everything up
@@ -128,12 +131,12 @@ def main():
                     "avg_launch_ms": dom.ms / dom.launches, "launches_per_step": dom.launches // prof_iters}
 
     result = {
-        "metric": "NN evals/sec at batch 256, BT4-shape fp16",
+        "metric": "NN evals/sec at batch 256, BT4-shape fp16" if args.config == "c2_bt4_15x1024" else "NN evals/sec",
         "value": batch / (wall_ms * 1e-3),
         "unit": "evals/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
+        "vs_baseline": None, "dtype": wl.get("dtype", "fp16"), "data": "synthetic",
         "config": {"workload": args.config, "description": wl["desc"], "batch": batch,
                    "inputs": "seeded random-playout positions, classical 112 planes"},
         "roofline": roofline,

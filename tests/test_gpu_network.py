@@ -122,6 +122,25 @@ def test_bt4_shape_batch_256(positions):
     np.testing.assert_allclose(comp2.results()["policy"], full["policy"][perm], rtol=0, atol=1e-5)
 
 
+@pytest.mark.timeout(600)
+def test_resnet_20x256_batch_512():
+    """configs[3]: oracle comparison on 24 positions, then the full batch of 512
+    through row-independence (same rows in a small and in the full batch)."""
+    pos = oc.random_positions(512, seed=777)
+    path = netgen.cached_config("c3_resnet_20x256")
+    masks, values = pos["masks"], pos["values"]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks[:24], values[:24])
+    net, res24 = _run_gpu(path, masks[:24], values[:24], "precision=fp16")
+    _compare(res24, want, pos["legal"][:24])
+    comp = net.NewComputation()
+    comp.AddInputs(masks, values)
+    comp.ComputeBlocking()
+    full = comp.results()
+    assert np.isfinite(full["policy"]).all()
+    np.testing.assert_allclose(onn.softmax_rows(full["policy"][:24]), onn.softmax_rows(res24["policy"]), rtol=0, atol=5e-3)
+    np.testing.assert_allclose(full["q"][:24], res24["q"], rtol=0, atol=5e-3)
+
+
 def test_ragged_and_oversized_batches(positions):
     """Batch sizes that are not tile multiples, a batch larger than max_batch
     (split into device passes) and an empty computation."""
