@@ -67,6 +67,10 @@ int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const 
 int lc0mi_k_winograd_conv(const float* x, const float* filter, const float* bias, const float* skip,
                           const float* se_w1, const float* se_b1, const float* se_w2, const float* se_b2, int se_k,
                           int batch, int cin, int cout, int act, int use_fp16, float* out);
+/* Plain device-to-device copy of `bytes` bytes (16-byte vectors), launched `iters`
+ * times: the known-traffic kernel used to calibrate HBM byte counters. *ms receives
+ * the mean HIP-event time per launch. */
+int lc0mi_k_copy(long long bytes, int iters, double* ms);
 /* Input planes -> [B][64][112] floats (NHWC form of EncodePlanes). */
 int lc0mi_k_expand_planes_nhwc(const uint64_t* masks, const float* values, int batch, float* out);
 

@@ -370,6 +370,19 @@ int lc0mi_k_winograd_conv(const float* x, const float* filter, const float* bias
   });
 }
 
+int lc0mi_k_copy(long long bytes, int iters, double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (bytes < 16 || iters < 1) throw Error("bad copy size");
+    Dev dev;
+    void* src = dev.Alloc((size_t)bytes);
+    void* dst = dev.Alloc((size_t)bytes);
+    K_CHECK(hipMemset(src, 1, (size_t)bytes));
+    double t = TimeLaunches(iters, [&] { lc0mi::LaunchCopy(src, dst, bytes / 16, nullptr); });
+    if (ms) *ms = t;
+  });
+}
+
 int lc0mi_k_expand_planes_nhwc(const uint64_t* masks, const float* values, int batch, float* out) {
   return Guard([&] {
     RequireDevice();

@@ -59,6 +59,8 @@ void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T*
 template <typename T>
 void LaunchExpandPlanesNchw(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream);
 
+// dst[i] = src[i] for n 16-byte vectors (traffic calibration kernel).
+void LaunchCopy(const void* src, void* dst, long long n_vec16, hipStream_t stream);
 // Sets n floats to zero (a kernel, so that it can be captured into a graph).
 void LaunchZero(float* p, long long n, hipStream_t stream);
 // Forces LaunchGemm to use one kernel variant (-1 = automatic choice): 0 256x256x64,

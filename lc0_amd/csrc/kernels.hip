@@ -721,6 +721,19 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __res
 }
 }  // namespace
 
+namespace {
+__global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, long long n) {
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+}  // namespace
+
+void LaunchCopy(const void* src, void* dst, long long n_vec16, hipStream_t stream) {
+  if (n_vec16 <= 0) return;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)((n_vec16 + 255) / 256)), dim3(256), 0, stream,
+                     static_cast<const uint4*>(src), static_cast<uint4*>(dst), n_vec16);
+}
+
 void LaunchZero(float* p, long long n, hipStream_t stream) {
   if (n <= 0) return;
   hipLaunchKernelGGL(zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, n);
