@@ -18,7 +18,17 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA peak
+PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA peak
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
+
+# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration) measured with
+# rocprofv3 --pmc on this same command; counters cannot be read from inside the process, so the figures
+# recorded under profiles/ are repeated here: (workload, batch, kernel) -> bytes.
+MEASURED_TRAFFIC = {
+    ("c2_bt4_15x1024", 256, "gemm_dma_256x256x64"): (74036 + 57080) * 1024,
+    ("c2_bt4_15x1024", 256, "gemm_dma_256x192x64"): (90618 + 49152) * 1024,
+    ("c2_bt4_15x1024", 256, "attention"): (163959 + 32769) * 1024,
+}
 
 WORKLOADS = {
     "c2_bt4_15x1024": dict(batch=256, desc="BT4-shape attention body: 15 layers, d=1024, 32 heads, dff 1536, "
@@ -27,6 +37,9 @@ WORKLOADS = {
     "c0_resnet_6x64": dict(batch=32, options="precision=fp32", dtype="fp32",
                            desc="SE-ResNet 6x64, SE ratio 4, classical policy, WDL, fp32"),
     "c3_resnet_20x256": dict(batch=512, desc="SE-ResNet 20x256, SE ratio 4, winograd F(4x4,3x3), fp16"),
+    "c4_bt4_fp8": dict(batch=1024, net="c2_bt4_15x1024", options="precision=fp8", dtype="fp8_e4m3",
+                       desc="BT4-shape attention body with e4m3 operands (fp32 accumulation) in the QKV, attention-output "
+                            "and FFN GEMMs; weights scaled per output row, activations per tensor; the rest fp16"),
     "tiny_attn": dict(batch=64, desc="tiny smolgen attention body (test net)"),
 }
 
@@ -73,7 +86,7 @@ def main():
 
     wl = WORKLOADS[args.config]
     batch = args.batch or wl["batch"]
-    path = netgen.cached_config(args.config)
+    path = netgen.cached_config(wl.get("net", args.config))
     pos = oc.random_positions(max(batch, args.cpu_sample), seed=20240)
     masks, values = pos["masks"], pos["values"]
 
@@ -121,14 +134,18 @@ def main():
     dom = max(groups.values(), key=lambda g: g.ms)
     if dom.flops > 0:
         achieved = dom.flops / dom.launches / (dom.ms / dom.launches * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": dom.name, "achieved": achieved, "peak": PEAK_FP16_TFLOPS,
-                    "unit": "TFLOP/s", "frac": achieved / PEAK_FP16_TFLOPS, "traffic": None,
+        peak = PEAK_FP8_TFLOPS if dom.name.startswith("gemm_f8") else PEAK_FP16_TFLOPS
+        roofline = {"bound": "mfma", "kernel": dom.name, "achieved": achieved, "peak": peak,
+                    "unit": "TFLOP/s", "frac": achieved / peak, "traffic": None,
                     "avg_launch_ms": dom.ms / dom.launches, "launches_per_step": dom.launches // prof_iters}
     else:
         achieved = dom.bytes / dom.launches / (dom.ms / dom.launches * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": dom.name, "achieved": achieved, "peak": PEAK_HBM_GBS,
                     "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
                     "avg_launch_ms": dom.ms / dom.launches, "launches_per_step": dom.launches // prof_iters}
+
+    roofline["traffic"] = MEASURED_TRAFFIC.get((args.config, batch, dom.name))
+    roofline["algorithmic_bytes"] = dom.bytes / dom.launches if dom.bytes else None
 
     result = {
         "metric": "NN evals/sec at batch 256, BT4-shape fp16" if args.config == "c2_bt4_15x1024" else "NN evals/sec",

@@ -67,6 +67,21 @@ int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const 
 int lc0mi_k_winograd_conv(const float* x, const float* filter, const float* bias, const float* skip,
                           const float* se_w1, const float* se_b1, const float* se_w2, const float* se_b2, int se_k,
                           int batch, int cin, int cout, int act, int use_fp16, float* out);
+/* e4m3 GEMM: C = act(col_scale[n] * A.W^T + bias[n]); A [M][lda], W [N][ldw] e4m3 bytes, K % 128 == 0.
+ * out_f8 != 0: C receives e4m3(C * out_mul) bytes, else halves. Counterpart of FullyConnectedLayer::Forward1D
+ * (src/neural/backends/blas/fully_connected_layer.cc:66-106) on quantised operands. */
+int lc0mi_k_gemm_f8(const uint8_t* A, int lda, const uint8_t* W, int ldw, const float* col_scale, const float* bias,
+                    int M, int N, int K, int act, int out_f8, float out_mul, void* C, int ldc, int time_iters,
+                    double* ms);
+/* y[i] = e4m3(x[i] * mul): round to nearest even, saturating at +-448 (FP32toFP8E4M3FN,
+ * src/utils/fp8_utils.h:111-138, applied to half inputs). n % 8 == 0. */
+int lc0mi_k_quantize_f8(const uint16_t* x, long long n, float mul, uint8_t* y);
+/* lc0mi_k_layer_norm with a second, e4m3 output y_f8 = e4m3(y * f8_mul). */
+int lc0mi_k_layer_norm_f8(const uint16_t* x, const uint16_t* skip, const float* gamma, const float* beta, int rows,
+                          int C, float alpha, float eps, float f8_mul, uint16_t* y, uint8_t* y_f8);
+/* lc0mi_k_attention with e4m3 output e4m3(out * out_mul). */
+int lc0mi_k_attention_f8(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, float scale, float out_mul,
+                         uint8_t* out);
 /* Plain device-to-device copy of `bytes` bytes (16-byte vectors), launched `iters`
  * times: the known-traffic kernel used to calibrate HBM byte counters. *ms receives
  * the mean HIP-event time per launch. */

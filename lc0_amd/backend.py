@@ -63,6 +63,7 @@ def load_library():
     lib.lc0mi_net_set_profiling.argtypes = [vp, ci]
     lib.lc0mi_net_take_profile.argtypes = [vp, C.c_char_p, ci]
     lib.lc0mi_net_time_resident_forward.argtypes = [vp, ci, ci, C.POINTER(C.c_double)]
+    lib.lc0mi_net_calibrate_fp8.argtypes = [vp, ci, vp, vp]
     for name, typ in (("lc0mi_attn_policy_map", C.c_int16), ("lc0mi_conv_policy_map", C.c_int16),
                       ("lc0mi_pos_encoding", cf)):
         getattr(lib, name).argtypes = [C.POINTER(ci)]
@@ -157,6 +158,15 @@ class Network:
             name, ms, n, fl, by = line.split()
             out.append(KernelTime(name, float(ms), int(n), float(fl), float(by)))
         return out
+
+    def CalibrateFp8(self, masks, values):
+        """precision=fp8: activation scales from these positions (uint64 [n,112], float32 [n,112])."""
+        import numpy as np
+        masks = np.ascontiguousarray(masks, np.uint64)
+        values = np.ascontiguousarray(values, np.float32)
+        if masks.shape != values.shape or masks.ndim != 2 or masks.shape[1] != 112:
+            raise BackendError("masks and values must both be [n, 112]")
+        _check(load_library().lc0mi_net_calibrate_fp8(self._h, masks.shape[0], masks.ctypes.data, values.ctypes.data))
 
     def TimeResidentForward(self, batch, iters):
         ms = C.c_double()

@@ -195,6 +195,13 @@ int lc0mi_net_time_resident_forward(lc0mi_net* net, int batch, int iters, double
   });
 }
 
+int lc0mi_net_calibrate_fp8(lc0mi_net* net, int n, const uint64_t* masks, const float* values) {
+  return Guard([&] {
+    if (!net) throw lc0mi::Error("null network");
+    net->impl->CalibrateFp8(n, masks, values);
+  });
+}
+
 const int16_t* lc0mi_attn_policy_map(int* count) {
   const auto& m = lc0mi::AttnPolicyMap();
   if (count) *count = static_cast<int>(m.size());

@@ -370,6 +370,90 @@ int lc0mi_k_winograd_conv(const float* x, const float* filter, const float* bias
   });
 }
 
+int lc0mi_k_gemm_f8(const uint8_t* A, int lda, const uint8_t* W, int ldw, const float* col_scale, const float* bias,
+                    int M, int N, int K, int act, int out_f8, float out_mul, void* C, int ldc, int time_iters,
+                    double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (K % 128 || lda % 16 || ldw % 16) throw Error("K must be a multiple of 128, lda and ldw of 16");
+    if (M < 1 || N < 1 || lda < K || ldw < K || ldc < N || !col_scale) throw Error("bad gemm shape");
+    Dev dev;
+    lc0mi::GemmF8Args g;
+    g.A = dev.Put(A, (size_t)(M - 1) * lda + K); g.lda = lda;
+    g.W = dev.Put(W, (size_t)(N - 1) * ldw + K); g.ldw = ldw;
+    const size_t c_bytes = ((size_t)(M - 1) * ldc + N) * (out_f8 ? 1 : 2);
+    g.C = dev.Alloc(c_bytes); g.ldc = ldc;
+    K_CHECK(hipMemcpy(g.C, C, c_bytes, hipMemcpyHostToDevice));
+    g.col_scale = dev.Put(col_scale, (size_t)N);
+    g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
+    g.M = M; g.N = N; g.K = K; g.act = act; g.out_f8 = out_f8 != 0; g.out_mul = out_mul;
+    lc0mi::LaunchGemmF8(g, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(C, g.C, c_bytes, hipMemcpyDeviceToHost));
+    if (time_iters > 0 && ms) *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchGemmF8(g, nullptr); });
+  });
+}
+
+int lc0mi_k_quantize_f8(const uint16_t* x, long long n, float mul, uint8_t* y) {
+  return Guard([&] {
+    RequireDevice();
+    if (n < 8 || n % 8) throw Error("n must be a positive multiple of 8");
+    Dev dev;
+    auto* dx = reinterpret_cast<half_t*>(dev.Put(x, (size_t)n));
+    auto* dy = static_cast<uint8_t*>(dev.Alloc((size_t)n));
+    lc0mi::LaunchQuantizeF8(dx, dy, n, mul, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(y, dy, (size_t)n, hipMemcpyDeviceToHost));
+  });
+}
+
+int lc0mi_k_layer_norm_f8(const uint16_t* x, const uint16_t* skip, const float* gamma, const float* beta, int rows,
+                          int C, float alpha, float eps, float f8_mul, uint16_t* y, uint8_t* y_f8) {
+  return Guard([&] {
+    RequireDevice();
+    if (C % 8 || C < 8 || C > 8192 || rows < 1) throw Error("bad layer norm shape");
+    Dev dev;
+    const size_t n = (size_t)rows * C;
+    auto* dx = reinterpret_cast<half_t*>(dev.Put(x, n));
+    auto* ds = skip ? reinterpret_cast<half_t*>(dev.Put(skip, n)) : nullptr;
+    auto* dy = reinterpret_cast<half_t*>(dev.Alloc(n * 2));
+    auto* dq = static_cast<uint8_t*>(dev.Alloc(n));
+    float* dg = dev.Put(gamma, (size_t)C);
+    float* db = dev.Put(beta, (size_t)C);
+    lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr, dq, f8_mul);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(y, dy, n * 2, hipMemcpyDeviceToHost));
+    K_CHECK(hipMemcpy(y_f8, dq, n, hipMemcpyDeviceToHost));
+  });
+}
+
+int lc0mi_k_attention_f8(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, float scale, float out_mul,
+                         uint8_t* out) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1 || heads < 1) throw Error("bad attention shape");
+    Dev dev;
+    const int d = heads * 32;
+    auto* dq = reinterpret_cast<half_t*>(dev.Put(qkv, (size_t)batch * 64 * 3 * d));
+    half_t* db = nullptr;
+    if (bias) {
+      std::vector<uint16_t> perm((size_t)batch * heads * 4096);
+      for (size_t bh = 0; bh < (size_t)batch * heads; bh++)
+        for (int q = 0; q < 64; q++)
+          for (int k = 0; k < 64; k++) perm[bh * 4096 + lc0mi::SmolgenBiasIndex(q, k)] = bias[bh * 4096 + q * 64 + k];
+      db = reinterpret_cast<half_t*>(dev.Put(perm.data(), perm.size()));
+    }
+    auto* dout = static_cast<uint8_t*>(dev.Alloc((size_t)batch * 64 * d));
+    lc0mi::LaunchAttentionF8Out(dq, db, dout, out_mul, batch, heads, scale, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(out, dout, (size_t)batch * 64 * d, hipMemcpyDeviceToHost));
+  });
+}
+
 int lc0mi_k_copy(long long bytes, int iters, double* ms) {
   return Guard([&] {
     RequireDevice();

@@ -36,6 +36,30 @@ void LaunchGemm(const GemmArgs& args, hipStream_t stream);
 // Name of the kernel variant LaunchGemm picks for these arguments (tile shape).
 const char* GemmVariantName(const GemmArgs& args);
 
+// e4m3 (OCP fp8, "fn": max 448, no infinities) GEMM with fp32 accumulation:
+//   C[m][n] = act(col_scale[n] * sum_k A[m][k] * W[n][k] + bias[n])
+// A, W hold e4m3 bytes, K-contiguous; col_scale[n] = (activation scale) x (scale of weight row n).
+// out_f8: C receives e4m3 bytes of C * out_mul (saturating, round to nearest even), else half.
+// Requirements: K % 128 == 0, lda % 16 == 0, ldw % 16 == 0, 16-byte aligned bases.
+struct GemmF8Args {
+  const uint8_t* A = nullptr; int lda = 0;
+  const uint8_t* W = nullptr; int ldw = 0;
+  void* C = nullptr; int ldc = 0;
+  const float* col_scale = nullptr;
+  const float* bias = nullptr;
+  int M = 0, N = 0, K = 0;
+  int act = 3;
+  bool out_f8 = false;
+  float out_mul = 1.0f;
+};
+void LaunchGemmF8(const GemmF8Args& args, hipStream_t stream);
+const char* GemmF8VariantName(const GemmF8Args& args);
+
+// *out = max(*out, max_i |x[i]|) (n % 8 == 0; *out must hold a non-negative float).
+void LaunchAbsMax(const half_t* x, long long n, float* out, hipStream_t stream);
+// y[i] = e4m3(x[i] * mul), saturating; n % 8 == 0.
+void LaunchQuantizeF8(const half_t* x, uint8_t* y, long long n, float mul, hipStream_t stream);
+
 // Same contract in float: C = act(scale * A.W^T + bias) with float A, W, C.
 // K % 4 == 0, lda % 4 == 0, ldw % 4 == 0.
 struct GemmArgsF32 {
@@ -78,14 +102,19 @@ void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_s
 
 // rows x C layer norm: y = beta + gamma * (t - mean) / sqrt(var + eps) with
 // t = x * alpha + skip (skip may be null). x, skip, y may alias. C % 8 == 0, C <= 8192.
+// y_f8 (optional): also receives e4m3(y * f8_mul), saturating, the operand of a following fp8 GEMM.
 void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
-                     int rows, int C, float alpha, float eps, hipStream_t stream);
+                     int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8 = nullptr,
+                     float f8_mul = 1.0f);
 
 // Fused multi-head attention over 64 tokens, head depth 32.
 // qkv: [B*64][3*d_model] (q | k | v column blocks), bias: smolgen logits in the
 // tile-native layout produced by SmolgenBiasIndex (may be null), out: [B*64][d_model].
 void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int batch, int heads,
                      float scale, hipStream_t stream);
+// Same with e4m3 output: out[...] = e4m3(result * out_mul), saturating.
+void LaunchAttentionF8Out(const half_t* qkv, const half_t* bias, uint8_t* out, float out_mul, int batch, int heads,
+                          float scale, hipStream_t stream);
 // Position inside one head's 4096-entry bias block of logit (query q, key k).
 int SmolgenBiasIndex(int q, int k);
 

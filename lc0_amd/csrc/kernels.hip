@@ -11,12 +11,18 @@
 //   attn_policy_gather    promotion offsets + kAttnPolicyMap gather  blas/network_blas.cc:873-914
 #include "kernels.h"
 
+#include <algorithm>
+#include <type_traits>
+#include <utility>
+
 namespace lc0mi {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx8 __attribute__((ext_vector_type(8)));
 
 namespace {
 
@@ -252,55 +258,84 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 // 16 bytes per lane from global memory into LDS at lds_base + lane * 16
 // (lds_base must be wave-uniform). Completion is visible through vmcnt only:
 // callers wait with s_waitcnt vmcnt(0) plus a barrier before reading the data.
-__device__ __forceinline__ void DmaToLds16(const half_t* gptr, half_t* lds_base) {
+__device__ __forceinline__ void DmaToLds16(const void* gptr, void* lds_base) {
   unsigned lds_addr = (unsigned)(size_t)LC0MI_LDS_PTR(lds_base);
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory", "m0");
 }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(GemmArgs p) {
+template <int... Is, typename F>
+__device__ __forceinline__ void StaticFor(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+
+// 4 floats -> 4 e4m3 bytes (round to nearest even, saturating at +-448; the
+// hardware conversion alone would turn |v| > 464 into NaN).
+__device__ __forceinline__ unsigned PackFp8x4(float a, float b, float c, float d) {
+  a = __builtin_fminf(__builtin_fmaxf(a, -448.0f), 448.0f);
+  b = __builtin_fminf(__builtin_fmaxf(b, -448.0f), 448.0f);
+  c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
+  d = __builtin_fminf(__builtin_fmaxf(d, -448.0f), 448.0f);
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return (unsigned)v;
+}
+
+// The same kernel serves fp16 operands (Args = GemmArgs: BKB = 128 bytes = 64
+// halves per tile row, v_mfma_f32_32x32x16_f16) and e4m3 operands (Args =
+// GemmF8Args: 128 bytes = 128 values per row, v_mfma_f32_32x32x64_f8f6f4);
+// BKB is the k-tile in bytes. OutT is half_t or uint8_t (e4m3, fp8 operands only).
+template <int BM, int BN, int BKB, int WAVES_M, int WAVES_N, typename Args, typename OutT>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(Args p) {
+  constexpr bool F8 = std::is_same<Args, GemmF8Args>::value;
+  constexpr int ES = F8 ? 1 : 2;                  // bytes per operand element
   constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int CPR = BK / 8;                     // 16-byte chunks per tile row
+  constexpr int CPR = BKB / 16;                   // 16-byte chunks per tile row
   constexpr int ROWS_PER_CHUNK = 64 / CPR;        // tile rows per 1 KiB transfer
-  constexpr int SWZ_SHIFT = (BK == 64) ? 1 : 2;   // log2(rows per 256 bytes of LDS)
+  constexpr int SWZ_SHIFT = (BKB == 128) ? 1 : 2; // log2(rows per 256 bytes of LDS)
   constexpr int A_CPW = BM / ROWS_PER_CHUNK / NWAVES, W_CPW = BN / ROWS_PER_CHUNK / NWAVES;
-  static_assert(BK == 64 || BK == 32, "BK must be 32 or 64");
+  static_assert(BKB == 128 || BKB == 64, "k-tile must be 64 or 128 bytes");
+  static_assert(F8 || sizeof(OutT) == 2, "fp8 output needs fp8 operands");
   static_assert(A_CPW >= 1 && W_CPW >= 1, "tile too small for the wave count");
-  constexpr int STAGE = (BM + BN) * BK;
-  constexpr int EPI_STRIDE = WN + 8;
-  constexpr int EPI_HALVES = NWAVES * 32 * EPI_STRIDE;
-  constexpr int SMEM = (2 * STAGE > EPI_HALVES) ? 2 * STAGE : EPI_HALVES;
-  __shared__ __attribute__((aligned(1024))) half_t smem[SMEM];
+  constexpr int STAGE = (BM + BN) * BKB;          // bytes
+  constexpr int OV = 16 / sizeof(OutT);           // output elements per 16-byte vector
+  constexpr int EPI_STRIDE = WN + OV;             // elements
+  constexpr int EPI_BYTES = NWAVES * 32 * EPI_STRIDE * (int)sizeof(OutT);
+  constexpr int SMEM = (2 * STAGE > EPI_BYTES) ? 2 * STAGE : EPI_BYTES;
+  __shared__ __attribute__((aligned(1024))) char smem[SMEM];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
-  const half_t* A = p.A + (long long)blockIdx.z * p.strideA;
-  const half_t* W = p.W + (long long)blockIdx.z * p.strideW;
   const int M = p.M, N = p.N, K = p.K;
+  const char* A = reinterpret_cast<const char*>(p.A);
+  const char* W = reinterpret_cast<const char*>(p.W);
+  if constexpr (!F8) {
+    A += (long long)blockIdx.z * p.strideA * ES;
+    W += (long long)blockIdx.z * p.strideW * ES;
+  }
 
-  const half_t* a_ptr[A_CPW];
-  const half_t* w_ptr[W_CPW];
+  const char* a_ptr[A_CPW];
+  const char* w_ptr[W_CPW];
 #pragma unroll
   for (int i = 0; i < A_CPW; i++) {
     const int row = (wave * A_CPW + i) * ROWS_PER_CHUNK + lane / CPR;
     const int c = (lane % CPR) ^ ((row >> SWZ_SHIFT) % CPR);
-    a_ptr[i] = A + (long long)min(m0 + row, M - 1) * p.lda + c * 8;
+    a_ptr[i] = A + (long long)min(m0 + row, M - 1) * p.lda * ES + c * 16;
   }
 #pragma unroll
   for (int i = 0; i < W_CPW; i++) {
     const int row = (wave * W_CPW + i) * ROWS_PER_CHUNK + lane / CPR;
     const int c = (lane % CPR) ^ ((row >> SWZ_SHIFT) % CPR);
-    w_ptr[i] = W + (long long)min(n0 + row, N - 1) * p.ldw + c * 8;
+    w_ptr[i] = W + (long long)min(n0 + row, N - 1) * p.ldw * ES + c * 16;
   }
-  auto issue = [&](half_t* As, half_t* Ws, int k0) {
+  auto issue = [&](char* As, char* Ws, int kbyte) {
 #pragma unroll
-    for (int i = 0; i < A_CPW; i++) DmaToLds16(a_ptr[i] + k0, As + (wave * A_CPW + i) * 512);
+    for (int i = 0; i < A_CPW; i++) DmaToLds16(a_ptr[i] + kbyte, As + (wave * A_CPW + i) * 1024);
 #pragma unroll
-    for (int i = 0; i < W_CPW; i++) DmaToLds16(w_ptr[i] + k0, Ws + (wave * W_CPW + i) * 512);
+    for (int i = 0; i < W_CPW; i++) DmaToLds16(w_ptr[i] + kbyte, Ws + (wave * W_CPW + i) * 1024);
   };
 
   floatx16 acc[TM][TN];
@@ -313,40 +348,67 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(GemmArg
 
   const int r = lane & 31, g = lane >> 5;
   const int swz = (r >> SWZ_SHIFT) % CPR;
-  const int a_row = (wm * WM + r) * BK, w_row = (wn * WN + r) * BK;
+  const int a_row = (wm * WM + r) * BKB, w_row = (wn * WN + r) * BKB;
 
-  const int nk = K / BK;
-  issue(smem, smem + BM * BK, 0);
+  const int nk = K * ES / BKB;
+  issue(smem, smem + BM * BKB, 0);
   for (int kt = 0; kt < nk; kt++) {
-    const half_t* As = smem + (kt & 1) * STAGE;
-    const half_t* Ws = As + BM * BK;
-    half_t* nxt = smem + ((kt + 1) & 1) * STAGE;
+    const char* As = smem + (kt & 1) * STAGE;
+    const char* Ws = As + BM * BKB;
+    char* nxt = smem + ((kt + 1) & 1) * STAGE;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of k-tile kt have landed
     __syncthreads();                     // ... and everybody's; everybody is done reading the other stage
-    if (kt + 1 < nk) issue(nxt, nxt + BM * BK, (kt + 1) * BK);
+    if (kt + 1 < nk) issue(nxt, nxt + BM * BKB, (kt + 1) * BKB);
+    if constexpr (F8) {
+      // One MFMA consumes 64 k-values: lane half g holds 32 consecutive bytes = 2 chunks.
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ks++) {
-      const int coff = ((2 * ks + g) ^ swz) * 8;
-      half8 af[TM], wf[TN];
+      for (int ks = 0; ks < BKB / 64; ks++) {
+        const int c0 = ((4 * ks + 2 * g) ^ swz) * 16, c1 = ((4 * ks + 2 * g + 1) ^ swz) * 16;
+        intx8 af[TM], wf[TN];
 #pragma unroll
-      for (int i = 0; i < TM; i++) af[i] = *reinterpret_cast<const half8*>(As + a_row + i * 32 * BK + coff);
+        for (int i = 0; i < TM; i++) {
+          const intx4 lo = *reinterpret_cast<const intx4*>(As + a_row + i * 32 * BKB + c0);
+          const intx4 hi = *reinterpret_cast<const intx4*>(As + a_row + i * 32 * BKB + c1);
+          af[i] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
 #pragma unroll
-      for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const half8*>(Ws + w_row + j * 32 * BK + coff);
+        for (int j = 0; j < TN; j++) {
+          const intx4 lo = *reinterpret_cast<const intx4*>(Ws + w_row + j * 32 * BKB + c0);
+          const intx4 hi = *reinterpret_cast<const intx4*>(Ws + w_row + j * 32 * BKB + c1);
+          wf[j] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
 #pragma unroll
-      for (int i = 0; i < TM; i++)
+        for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < TN; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j], af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < BKB / 32; ks++) {
+        const int coff = ((2 * ks + g) ^ swz) * 16;
+        half8 af[TM], wf[TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++) af[i] = *reinterpret_cast<const half8*>(As + a_row + i * 32 * BKB + coff);
+#pragma unroll
+        for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const half8*>(Ws + w_row + j * 32 * BKB + coff);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[i][j], 0, 0, 0);
+      }
     }
   }
 
   // Epilogue through LDS (the stage buffers are free after the barrier).
   __syncthreads();
-  half_t* C = reinterpret_cast<half_t*>(p.C) + (long long)blockIdx.z * p.strideC;
-  half_t* strip = smem + wave * 32 * EPI_STRIDE;
-  constexpr int CHUNKS_PER_ROW = WN / 8;
+  OutT* C = reinterpret_cast<OutT*>(p.C);
+  if constexpr (!F8) C += (long long)blockIdx.z * p.strideC;
+  OutT* strip = reinterpret_cast<OutT*>(smem) + wave * 32 * EPI_STRIDE;
+  constexpr int CHUNKS_PER_ROW = WN / OV;
   constexpr int STRIP_CHUNKS = 32 * CHUNKS_PER_ROW;
-  const bool vec_ok = (p.ldc % 8 == 0);
+  const bool vec_ok = (p.ldc % OV == 0);
   float bias_v[TN][4][4];
 #pragma unroll
   for (int j = 0; j < TN; j++)
@@ -359,10 +421,27 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(GemmArg
       for (int j = 0; j < TN; j++) {
 #pragma unroll
         for (int blk = 0; blk < 4; blk++) {
-          half4 h;
+          float v[4];
+          if constexpr (F8) {
+            // Per-column dequantisation factor (activation scale x weight-row scale).
+            float cs[4];
+            LoadBias4(p.col_scale, n0 + wn * WN + j * 32 + blk * 8 + g * 4, N, cs);
 #pragma unroll
-          for (int rr = 0; rr < 4; rr++) h[rr] = (half_t)act_fn(acc[i][j][blk * 4 + rr] * p.scale + bias_v[j][blk][rr]);
-          *reinterpret_cast<half4*>(&strip[r * EPI_STRIDE + j * 32 + blk * 8 + g * 4]) = h;
+            for (int rr = 0; rr < 4; rr++) v[rr] = act_fn(acc[i][j][blk * 4 + rr] * cs[rr] + bias_v[j][blk][rr]);
+          } else {
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) v[rr] = act_fn(acc[i][j][blk * 4 + rr] * p.scale + bias_v[j][blk][rr]);
+          }
+          OutT* dst = &strip[r * EPI_STRIDE + j * 32 + blk * 8 + g * 4];
+          if constexpr (sizeof(OutT) == 1) {
+            *reinterpret_cast<unsigned*>(dst) =
+                PackFp8x4(v[0] * p.out_mul, v[1] * p.out_mul, v[2] * p.out_mul, v[3] * p.out_mul);
+          } else {
+            half4 h;
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) h[rr] = (half_t)v[rr];
+            *reinterpret_cast<half4*>(dst) = h;
+          }
         }
       }
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0); the strip is private to this wave
@@ -373,13 +452,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(GemmArg
         const int row = idx / CHUNKS_PER_ROW;
         const int ch = idx - row * CHUNKS_PER_ROW;
         const int m = m0 + wm * WM + i * 32 + row;
-        const int n = n0 + wn * WN + ch * 8;
+        const int n = n0 + wn * WN + ch * OV;
         if (idx < STRIP_CHUNKS && m < M && n < N) {
-          half_t* dst = C + (long long)m * p.ldc + n;
-          if (vec_ok && n + 7 < N) {
-            *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&strip[row * EPI_STRIDE + ch * 8]);
+          OutT* dst = C + (long long)m * p.ldc + n;
+          if (vec_ok && n + OV - 1 < N) {
+            *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&strip[row * EPI_STRIDE + ch * OV]);
           } else {
-            for (int e = 0; e < 8 && n + e < N; e++) dst[e] = strip[row * EPI_STRIDE + ch * 8 + e];
+            for (int e = 0; e < OV && n + e < N; e++) dst[e] = strip[row * EPI_STRIDE + ch * OV + e];
           }
         }
       }
@@ -392,7 +471,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(GemmArg
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
   dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch);
-  hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK, WAVES_M, WAVES_N>), grid, dim3(WAVES_M * WAVES_N * 64), 0, stream, a);
+  hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t>), grid,
+                     dim3(WAVES_M * WAVES_N * 64), 0, stream, a);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKB = 128>
+void LaunchGemmDmaF8(const GemmF8Args& a, hipStream_t stream) {
+  dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, 1);
+  if (a.out_f8) {
+    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, uint8_t>), grid,
+                       dim3(WAVES_M * WAVES_N * 64), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, half_t>), grid,
+                       dim3(WAVES_M * WAVES_N * 64), 0, stream, a);
+  }
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
@@ -455,6 +547,38 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
     case kDma256x128: LaunchGemmDma<256, 128, 32, 4, 2>(a, stream); break;
     case kTile128: LaunchGemmTile<128, 128, 64, 2, 2>(a, stream); break;
     default: LaunchGemmTile<64, 64, 64, 2, 2>(a, stream); break;
+  }
+}
+
+namespace {
+// 0: 256x256, 1: 256x192, 2: 256x128 (fewest rounds over the 256 CUs, as for fp16).
+int PickGemmF8Variant(const GemmF8Args& a) {
+  if (g_variant_override >= 0 && g_variant_override <= 2) return g_variant_override;
+  const long long m_tiles = (a.M + 255) / 256;
+  auto cost = [&](int bn, double penalty) {
+    const long long tiles = m_tiles * ((a.N + bn - 1) / bn);
+    return (double)((tiles + 255) / 256) * bn * penalty;
+  };
+  const double c256 = cost(256, 1.0), c192 = cost(192, 1.04), c128 = cost(128, 1.15);
+  if (c256 <= c192 && c256 <= c128) return 0;
+  return c192 <= c128 ? 1 : 2;
+}
+}  // namespace
+
+const char* GemmF8VariantName(const GemmF8Args& a) {
+  switch (PickGemmF8Variant(a)) {
+    case 0: return "gemm_f8_256x256x128";
+    case 1: return "gemm_f8_256x192x128";
+    default: return "gemm_f8_256x128x128";
+  }
+}
+
+void LaunchGemmF8(const GemmF8Args& a, hipStream_t stream) {
+  if (a.M <= 0 || a.N <= 0) return;
+  switch (PickGemmF8Variant(a)) {
+    case 0: LaunchGemmDmaF8<256, 256, 2, 4>(a, stream); break;
+    case 1: LaunchGemmDmaF8<256, 192, 4, 2>(a, stream); break;
+    default: LaunchGemmDmaF8<256, 128, 4, 2>(a, stream); break;
   }
 }
 
@@ -588,7 +712,8 @@ template void LaunchExpandPlanesNchw<float>(const uint64_t*, const float*, float
 namespace {
 template <int NV>  // 16-byte vectors per lane; covers C <= 512 * NV
 __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restrict__ x, const half_t* skip,
-                                                         half_t* y, const float* __restrict__ gamma,
+                                                         half_t* y, uint8_t* yq, float q_mul,
+                                                         const float* __restrict__ gamma,
                                                          const float* __restrict__ beta, int rows, int C,
                                                          float alpha, float eps) {
   const int lane = threadIdx.x & 63;
@@ -636,11 +761,32 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restric
     int v = lane + i * 64;
     if (v < nvec) {
       half8 o;
+      float f[8];
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = (half_t)(beta[v * 8 + e] + gamma[v * 8 + e] * (t[i][e] - mean) * den);
+      for (int e = 0; e < 8; e++) {
+        f[e] = beta[v * 8 + e] + gamma[v * 8 + e] * (t[i][e] - mean) * den;
+        o[e] = (half_t)f[e];
+      }
       *reinterpret_cast<half8*>(yr + v * 8) = o;
+      if (yq) {  // e4m3 copy of the same row for the next fp8 GEMM
+        uint2 q;
+        q.x = PackFp8x4(f[0] * q_mul, f[1] * q_mul, f[2] * q_mul, f[3] * q_mul);
+        q.y = PackFp8x4(f[4] * q_mul, f[5] * q_mul, f[6] * q_mul, f[7] * q_mul);
+        *reinterpret_cast<uint2*>(yq + (long long)row * C + v * 8) = q;
+      }
     }
   }
+}
+
+__global__ __launch_bounds__(256) void quantize_f8_kernel(const half_t* __restrict__ x, uint8_t* __restrict__ y,
+                                                          long long nvec, float mul) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const half8 h = *reinterpret_cast<const half8*>(x + i * 8);
+  uint2 q;
+  q.x = PackFp8x4((float)h[0] * mul, (float)h[1] * mul, (float)h[2] * mul, (float)h[3] * mul);
+  q.y = PackFp8x4((float)h[4] * mul, (float)h[5] * mul, (float)h[6] * mul, (float)h[7] * mul);
+  *reinterpret_cast<uint2*>(y + i * 8) = q;
 }
 }  // namespace
 
@@ -748,19 +894,50 @@ void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_s
 }
 
 void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
-                     int rows, int C, float alpha, float eps, hipStream_t stream) {
+                     int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8, float f8_mul) {
   if (rows <= 0) return;
   dim3 grid((rows + 3) / 4), block(256);
   if (C <= 512) {
-    hipLaunchKernelGGL(layer_norm_kernel<1>, grid, block, 0, stream, x, skip, y, gamma, beta, rows, C, alpha, eps);
+    hipLaunchKernelGGL(layer_norm_kernel<1>, grid, block, 0, stream, x, skip, y, y_f8, f8_mul, gamma, beta, rows, C,
+                       alpha, eps);
   } else if (C <= 1024) {
-    hipLaunchKernelGGL(layer_norm_kernel<2>, grid, block, 0, stream, x, skip, y, gamma, beta, rows, C, alpha, eps);
+    hipLaunchKernelGGL(layer_norm_kernel<2>, grid, block, 0, stream, x, skip, y, y_f8, f8_mul, gamma, beta, rows, C,
+                       alpha, eps);
   } else if (C <= 2048) {
-    hipLaunchKernelGGL(layer_norm_kernel<4>, grid, block, 0, stream, x, skip, y, gamma, beta, rows, C, alpha, eps);
+    hipLaunchKernelGGL(layer_norm_kernel<4>, grid, block, 0, stream, x, skip, y, y_f8, f8_mul, gamma, beta, rows, C,
+                       alpha, eps);
   } else {  // callers guarantee C <= 8192
-    hipLaunchKernelGGL(layer_norm_kernel<16>, grid, block, 0, stream, x, skip, y, gamma, beta, rows, C, alpha,
-                       eps);
+    hipLaunchKernelGGL(layer_norm_kernel<16>, grid, block, 0, stream, x, skip, y, y_f8, f8_mul, gamma, beta, rows, C,
+                       alpha, eps);
   }
+}
+
+namespace {
+// out = max(out, max |x|), as float bits (non-negative floats order like unsigned integers).
+__global__ __launch_bounds__(256) void absmax_kernel(const half_t* __restrict__ x, long long nvec, unsigned* out) {
+  float m = 0.0f;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (long long)gridDim.x * 256) {
+    const half8 h = *reinterpret_cast<const half8*>(x + i * 8);
+#pragma unroll
+    for (int e = 0; e < 8; e++) m = fmaxf(m, fabsf((float)h[e]));
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  if ((threadIdx.x & 63) == 0) atomicMax(out, __float_as_uint(m));
+}
+}  // namespace
+
+void LaunchAbsMax(const half_t* x, long long n, float* out, hipStream_t stream) {
+  const long long nvec = n / 8;
+  if (nvec <= 0) return;
+  const unsigned blocks = (unsigned)std::min<long long>((nvec + 255) / 256, 2048);
+  hipLaunchKernelGGL(absmax_kernel, dim3(blocks), dim3(256), 0, stream, x, nvec, reinterpret_cast<unsigned*>(out));
+}
+
+void LaunchQuantizeF8(const half_t* x, uint8_t* y, long long n, float mul, hipStream_t stream) {
+  if (n <= 0) return;
+  const long long nvec = n / 8;
+  hipLaunchKernelGGL(quantize_f8_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, stream, x, y, nvec, mul);
 }
 
 // ---------------------------------------------------------------------------
@@ -776,10 +953,11 @@ void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float
 namespace {
 constexpr int kVStride = 40;  // halves per key row of V in LDS
 
+template <typename OutT>  // half_t, or uint8_t for e4m3 output scaled by out_mul
 __global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict__ qkv,
                                                         const half_t* __restrict__ bias,
-                                                        half_t* __restrict__ out, int total_heads, int heads,
-                                                        float scale) {
+                                                        OutT* __restrict__ out, int total_heads, int heads,
+                                                        float scale, float out_mul) {
   __shared__ __attribute__((aligned(16))) half_t Vs[4][64 * kVStride];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int gh_raw = blockIdx.x * 4 + wave;
@@ -882,13 +1060,17 @@ __global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict
     }
   }
   if (!live) return;
-  half_t* O = out + (long long)b * 64 * d_model + h * 32;
+  OutT* O = out + (long long)b * 64 * d_model + h * 32;
 #pragma unroll
   for (int nt = 0; nt < 2; nt++)
 #pragma unroll
     for (int e = 0; e < 16; e++) {
       int q = 32 * nt + 8 * (e / 4) + 4 * g + (e % 4);
-      O[(long long)q * d_model + r] = (half_t)o[nt][e];
+      if constexpr (sizeof(OutT) == 1) {
+        O[(long long)q * d_model + r] = (uint8_t)(PackFp8x4(o[nt][e] * out_mul, 0.0f, 0.0f, 0.0f) & 0xffu);
+      } else {
+        O[(long long)q * d_model + r] = (half_t)o[nt][e];
+      }
     }
 }
 }  // namespace
@@ -904,8 +1086,16 @@ void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int bat
                      hipStream_t stream) {
   int total = batch * heads;
   if (total <= 0) return;
-  hipLaunchKernelGGL(attention_kernel, dim3((total + 3) / 4), dim3(256), 0, stream, qkv, bias, out, total, heads,
-                     scale);
+  hipLaunchKernelGGL(attention_kernel<half_t>, dim3((total + 3) / 4), dim3(256), 0, stream, qkv, bias, out, total,
+                     heads, scale, 1.0f);
+}
+
+void LaunchAttentionF8Out(const half_t* qkv, const half_t* bias, uint8_t* out, float out_mul, int batch, int heads,
+                          float scale, hipStream_t stream) {
+  int total = batch * heads;
+  if (total <= 0) return;
+  hipLaunchKernelGGL(attention_kernel<uint8_t>, dim3((total + 3) / 4), dim3(256), 0, stream, qkv, bias, out, total,
+                     heads, scale, out_mul);
 }
 
 // ---------------------------------------------------------------------------

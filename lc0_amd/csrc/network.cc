@@ -140,8 +140,18 @@ struct LinearT {
   int out = 0, in = 0, ld = 0;
 };
 
+// e4m3 copy of a dense layer: one scale per output row (absmax / 448).
+struct LinearF8 {
+  uint8_t* w = nullptr;        // [out][in] e4m3 codes
+  std::vector<float> wscale;   // [out], host copy
+  float* col_scale = nullptr;  // [out] device: activation scale x wscale (set by calibration)
+};
+
 struct EncoderDev {
   Linear qkv, dense, ffn1, ffn2;
+  LinearF8 qkv8, dense8, ffn18, ffn28;
+  // Per-tensor activation scales (value = code x scale) of the four fp8 operands.
+  float s_x = 1.0f, s_att = 1.0f, s_x1 = 1.0f, s_ffn = 1.0f;
   float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
   bool has_smolgen = false;
   Linear sg_compress, sg_dense1, sg_dense2;
@@ -226,6 +236,7 @@ class Mi355xNetwork : public Network {
   }
   std::vector<KernelTime> TakeProfile() override;
   double TimeResidentForward(int batch, int iters) override;
+  void CalibrateFp8(int n, const uint64_t* masks, const float* values) override;
 
   // Used by the computation.
   std::unique_ptr<HostSlot> GetSlot();
@@ -252,6 +263,12 @@ class Mi355xNetwork : public Network {
   template <typename T>
   struct LinearT MakeLinearT(const Vec& w, const Vec& b, int out, int in);
   Linear MakeLinear(const Vec& w, const Vec& b, int out, int in);
+  LinearF8 MakeLinearF8(const Vec& w, int out, int in);
+  void GemmF8(const char* name, const uint8_t* A, const Linear& lin, const LinearF8& q, void* C, int M, int act,
+              bool out_f8, float out_mul);
+  void RecordAbsMax(const half_t* x, size_t n, int slot);
+  void ApplyCalibration(const std::vector<float>& absmax);
+  void DefaultCalibration();
   float* UploadF(const Vec& v) { return arena_.Upload(v); }
   half_t* AllocH(size_t n) { return static_cast<half_t*>(arena_.Alloc(n * sizeof(half_t))); }
   float* AllocF(size_t n) { return static_cast<float*>(arena_.Alloc(n * sizeof(float))); }
@@ -298,6 +315,13 @@ class Mi355xNetwork : public Network {
   float* sg2f_ = nullptr;  // split-K accumulator of smolgen dense1
   half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
   float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
+
+  // fp8 configuration: the four large GEMMs of every encoder layer run on e4m3 operands.
+  bool fp8_ = false;
+  bool q_qkv_ = true, q_dense_ = true, q_ffn1_ = true, q_ffn2_ = true;   // option fp8_gemms
+  bool calibrating_ = false;
+  float* d_absmax_ = nullptr;   // [4 * layers + 1] calibration maxima (float bits, non-negative)
+  uint8_t *xq_ = nullptr, *attq_ = nullptr, *ffnq_ = nullptr;
 
   // Residual tower.
   bool fp32_ = false;
@@ -411,6 +435,187 @@ void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linea
   Timed(label.c_str(), flops, bytes, [&] { LaunchGemm(g, st); }, st);
 }
 
+// ------------------------------------------------------------------- fp8 --
+namespace {
+// float -> e4m3 code: round to nearest even, saturating at +-448 (the rule of
+// FP32toFP8E4M3FN, src/utils/fp8_utils.h:111-138).
+uint8_t EncodeE4M3(float v) {
+  const uint8_t sign = std::signbit(v) ? 0x80 : 0;
+  float a = std::fabs(v);
+  if (std::isnan(a)) return 0x7f;
+  if (a >= 448.0f) return sign | 0x7e;
+  int ex;
+  std::frexp(a, &ex);               // a = f * 2^ex, f in [0.5, 1)
+  ex = std::max(ex - 1, -6);        // binade of a; subnormals share the spacing of the first one
+  const float step = std::ldexp(1.0f, ex - 3);
+  const float q = std::nearbyint(a / step);   // default rounding mode: ties to even
+  const float mag = q * step;
+  if (mag < std::ldexp(1.0f, -6)) return sign | static_cast<uint8_t>(q);
+  int e2;
+  const float f = std::frexp(mag, &e2);       // mag = f * 2^e2
+  const int mant = static_cast<int>((f * 2.0f - 1.0f) * 8.0f);
+  return sign | static_cast<uint8_t>(((e2 - 1 + 7) << 3) | mant);
+}
+}  // namespace
+
+LinearF8 Mi355xNetwork::MakeLinearF8(const Vec& w, int out, int in) {
+  if (static_cast<size_t>(out) * in != w.size()) throw Error("Weight tensor has an unexpected size.");
+  LinearF8 q;
+  q.wscale.resize(out);
+  std::vector<uint8_t> codes(w.size());
+  for (int o = 0; o < out; o++) {
+    const float* row = &w[static_cast<size_t>(o) * in];
+    float amax = 0.0f;
+    for (int i = 0; i < in; i++) amax = std::max(amax, std::fabs(row[i]));
+    const float scale = amax > 0.0f ? amax / 448.0f : 1.0f;
+    q.wscale[o] = scale;
+    for (int i = 0; i < in; i++) codes[static_cast<size_t>(o) * in + i] = EncodeE4M3(row[i] / scale);
+  }
+  q.w = arena_.Upload(codes);
+  q.col_scale = AllocF(out);
+  return q;
+}
+
+void Mi355xNetwork::GemmF8(const char* name, const uint8_t* A, const Linear& lin, const LinearF8& q, void* C, int M,
+                           int act, bool out_f8, float out_mul) {
+  GemmF8Args g;
+  g.A = A; g.lda = lin.in;
+  g.W = q.w; g.ldw = lin.in;
+  g.C = C; g.ldc = lin.out;
+  g.col_scale = q.col_scale;
+  g.bias = lin.b;
+  g.M = M; g.N = lin.out; g.K = lin.in;
+  g.act = act;
+  g.out_f8 = out_f8;
+  g.out_mul = out_mul;
+  const double flops = 2.0 * M * lin.out * lin.in;
+  const double bytes = static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in +
+                       static_cast<double>(M) * lin.out * (out_f8 ? 1 : 2);
+  const std::string label = std::string(name) + "|" + GemmF8VariantName(g);
+  Timed(label.c_str(), flops, bytes, [&] { LaunchGemmF8(g, stream_); });
+}
+
+void Mi355xNetwork::RecordAbsMax(const half_t* x, size_t n, int slot) {
+  LaunchAbsMax(x, static_cast<long long>(n), d_absmax_ + slot, stream_);
+}
+
+// Activation scales from the maxima seen during calibration: the largest value maps to
+// 224, half of the e4m3 range (headroom for unseen positions costs no precision in a
+// floating-point format; anything beyond saturates).
+void Mi355xNetwork::ApplyCalibration(const std::vector<float>& absmax) {
+  auto scale_of = [](float amax) { return amax > 0.0f ? amax / 224.0f : 1.0f; };
+  auto upload = [&](LinearF8& q, float s_act) {
+    std::vector<float> cs(q.wscale.size());
+    for (size_t i = 0; i < cs.size(); i++) cs[i] = s_act * q.wscale[i];
+    HIP_CHECK(hipMemcpy(q.col_scale, cs.data(), cs.size() * sizeof(float), hipMemcpyHostToDevice));
+  };
+  for (size_t li = 0; li < encoders_.size(); li++) {
+    EncoderDev& e = encoders_[li];
+    e.s_x = scale_of(absmax[4 * li + 0]);
+    e.s_att = scale_of(absmax[4 * li + 1]);
+    e.s_x1 = scale_of(absmax[4 * li + 2]);
+    e.s_ffn = scale_of(absmax[4 * li + 3]);
+    upload(e.qkv8, e.s_x);
+    upload(e.dense8, e.s_att);
+    upload(e.ffn18, e.s_x1);
+    upload(e.ffn28, e.s_ffn);
+  }
+}
+
+void Mi355xNetwork::CalibrateFp8(int n, const uint64_t* masks, const float* values) {
+  if (!fp8_) throw Error("CalibrateFp8 needs a network created with precision=fp8.");
+  if (n < 1 || !masks || !values) throw Error("CalibrateFp8 needs at least one position.");
+  std::lock_guard<std::mutex> lock(eval_mutex_);
+  HIP_CHECK(hipSetDevice(device_));
+  const size_t slots = 4 * encoders_.size() + 1;
+  std::vector<float> absmax(slots, 0.0f), part(slots);
+  for (int done = 0; done < n; done += max_batch_) {
+    const int b = std::min(max_batch_, n - done);
+    HIP_CHECK(hipMemcpy(d_masks_, masks + static_cast<size_t>(done) * kInputPlanes, sizeof(uint64_t) * kInputPlanes * b,
+                        hipMemcpyHostToDevice));
+    HIP_CHECK(hipMemcpy(d_values_, values + static_cast<size_t>(done) * kInputPlanes, sizeof(float) * kInputPlanes * b,
+                        hipMemcpyHostToDevice));
+    LaunchZero(d_absmax_, static_cast<long long>(slots), stream_);
+    calibrating_ = true;
+    const bool was_profiling = profiling_;
+    profiling_ = false;
+    try {
+      ForwardAttentionBody(b);   // fp16 pass that records the maxima
+    } catch (...) {
+      calibrating_ = false;
+      profiling_ = was_profiling;
+      throw;
+    }
+    calibrating_ = false;
+    profiling_ = was_profiling;
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    HIP_CHECK(hipMemcpy(part.data(), d_absmax_, slots * sizeof(float), hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < slots; i++) absmax[i] = std::max(absmax[i], part[i]);
+  }
+  ApplyCalibration(absmax);
+}
+
+// Built-in calibration set used at load, so that precision=fp8 works without any caller
+// support: 64 seeded pseudo-positions (two kings, a random subset of other pieces, eight
+// history steps that differ by one moved piece, plausible auxiliary planes). Callers that
+// own real positions replace it through CalibrateFp8.
+void Mi355xNetwork::DefaultCalibration() {
+  const int n = std::min(64, max_batch_);
+  std::vector<uint64_t> masks(static_cast<size_t>(n) * kInputPlanes, 0);
+  std::vector<float> values(static_cast<size_t>(n) * kInputPlanes, 1.0f);
+  uint64_t state = 0x9e3779b97f4a7c15ULL;
+  auto next = [&state]() {   // splitmix64
+    uint64_t z = (state += 0x9e3779b97f4a7c15ULL);
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+    return z ^ (z >> 31);
+  };
+  for (int p = 0; p < n; p++) {
+    uint64_t* m = &masks[static_cast<size_t>(p) * kInputPlanes];
+    float* v = &values[static_cast<size_t>(p) * kInputPlanes];
+    // piece planes of the newest history step: 0-5 ours (P N B R Q K), 6-11 theirs
+    int square_of[32], plane_of[32], count = 0;
+    uint64_t used = 0;
+    auto place = [&](int plane, int lo_rank, int hi_rank) {
+      for (int tries = 0; tries < 64; tries++) {
+        const int sq = static_cast<int>(next() % 64);
+        if (sq / 8 < lo_rank || sq / 8 > hi_rank || (used >> sq) & 1) continue;
+        used |= 1ULL << sq;
+        square_of[count] = sq; plane_of[count] = plane; count++;
+        return;
+      }
+    };
+    place(5, 0, 7); place(11, 0, 7);
+    static const int kMaxCount[5] = {8, 2, 2, 2, 1};
+    for (int side = 0; side < 2; side++)
+      for (int piece = 0; piece < 5; piece++) {
+        const int k = static_cast<int>(next() % (kMaxCount[piece] + 1));
+        for (int i = 0; i < k; i++) place(side * 6 + piece, piece == 0 ? 1 : 0, piece == 0 ? 6 : 7);
+      }
+    const int history = 1 + static_cast<int>(next() % 8);
+    for (int h = 0; h < history; h++) {
+      for (int i = 0; i < count; i++) m[h * 13 + plane_of[i]] |= 1ULL << square_of[i];
+      if (next() % 16 == 0) m[h * 13 + 12] = ~0ULL;   // repetition marker
+      // step back in time: move one piece to a free square
+      const int i = static_cast<int>(next() % count);
+      for (int tries = 0; tries < 64; tries++) {
+        const int sq = static_cast<int>(next() % 64);
+        if ((used >> sq) & 1) continue;
+        used &= ~(1ULL << square_of[i]);
+        used |= 1ULL << sq;
+        square_of[i] = sq;
+        break;
+      }
+    }
+    for (int c = 104; c < 108; c++) m[c] = (next() & 1) ? ~0ULL : 0;   // castling rights
+    m[108] = (next() & 1) ? ~0ULL : 0;                                  // side to move
+    m[109] = ~0ULL; v[109] = static_cast<float>(next() % 100);          // rule-50 counter
+    m[110] = 0;
+    m[111] = ~0ULL;                                                     // all ones
+  }
+  CalibrateFp8(n, masks.data(), values.data());
+}
+
 // ------------------------------------------------------------- construction --
 Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   const NetworkFormat& nf = file.format;
@@ -422,10 +627,27 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   max_batch_ = options.GetInt("max_batch", 1024);
   if (max_batch_ < 1 || max_batch_ > 4096) throw Error("max_batch must be in 1..4096.");
   const std::string precision = options.GetString("precision", "fp16");
-  if (precision != "fp16" && precision != "fp32") {
-    throw Error("Precision '" + precision + "' is not supported (fp16 or fp32).");
+  if (precision != "fp16" && precision != "fp32" && precision != "fp8") {
+    throw Error("Precision '" + precision + "' is not supported (fp16, fp32 or fp8).");
   }
   fp32_ = precision == "fp32";
+  fp8_ = precision == "fp8";
+  {
+    // Which of the four encoder GEMMs use e4m3 operands: names joined by '+'.
+    const std::string which = options.GetString("fp8_gemms", "qkv+dense+ffn1+ffn2");
+    q_qkv_ = q_dense_ = q_ffn1_ = q_ffn2_ = false;
+    size_t pos = 0;
+    while (pos <= which.size()) {
+      const size_t end = std::min(which.find('+', pos), which.size());
+      const std::string name = which.substr(pos, end - pos);
+      if (name == "qkv") q_qkv_ = true;
+      else if (name == "dense") q_dense_ = true;
+      else if (name == "ffn1") q_ffn1_ = true;
+      else if (name == "ffn2") q_ffn2_ = true;
+      else if (!name.empty()) throw Error("Unknown name '" + name + "' in fp8_gemms (qkv, dense, ffn1, ffn2).");
+      pos = end + 1;
+    }
+  }
   policy_head_ = options.GetString("policy_head", "vanilla");
   value_head_ = options.GetString("value_head", "winner");
   wdl_ = nf.value == kValueWdl;
@@ -465,6 +687,9 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   if (attn_body_) {
     if (fp32_) throw Error("precision=fp32 is available for residual-tower networks only.");
     BuildAttentionBody(file);
+    if (fp8_) DefaultCalibration();
+  } else if (fp8_) {
+    throw Error("precision=fp8 is available for attention-body networks only.");
   } else if (fp32_) {
     BuildResnet<float>(file);
   } else {
@@ -538,6 +763,15 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     e.dense = MakeLinear(l.mha.dense_w, l.mha.dense_b, emb_, d_model_);
     e.ffn1 = MakeLinear(l.ffn.dense1_w, l.ffn.dense1_b, dff_, emb_);
     e.ffn2 = MakeLinear(l.ffn.dense2_w, l.ffn.dense2_b, emb_, dff_);
+    if (fp8_) {
+      if (emb_ % 128 || d_model_ % 128 || dff_ % 128) {
+        throw Error("precision=fp8 needs embedding, attention and FFN widths that are multiples of 128.");
+      }
+      e.qkv8 = MakeLinearF8(qkv_w, 3 * d_model_, emb_);
+      e.dense8 = MakeLinearF8(l.mha.dense_w, emb_, d_model_);
+      e.ffn18 = MakeLinearF8(l.ffn.dense1_w, dff_, emb_);
+      e.ffn28 = MakeLinearF8(l.ffn.dense2_w, emb_, dff_);
+    }
     e.ln1_g = UploadF(l.ln1_gammas); e.ln1_b = UploadF(l.ln1_betas);
     e.ln2_g = UploadF(l.ln2_gammas); e.ln2_b = UploadF(l.ln2_betas);
     if (static_cast<int>(l.ln1_gammas.size()) != emb_ || static_cast<int>(l.ln2_gammas.size()) != emb_) {
@@ -631,6 +865,12 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     }
     sg3_ = AllocH(static_cast<size_t>(max_batch_) * sg_gen_);
     sbias_ = AllocH(static_cast<size_t>(max_batch_) * heads_ * 4096);
+  }
+  if (fp8_) {
+    xq_ = static_cast<uint8_t*>(arena_.Alloc(T * emb_));
+    attq_ = static_cast<uint8_t*>(arena_.Alloc(T * d_model_));
+    ffnq_ = static_cast<uint8_t*>(arena_.Alloc(T * dff_));
+    d_absmax_ = AllocF(4 * encoders_.size() + 1);
   }
   pol_e_ = AllocH(T * pol_emb_);
   pol_qk_ = AllocH(T * 2 * pol_d_);
@@ -856,9 +1096,18 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
   Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * 2),
         [&] { LaunchExpandPlanesAttn<half_t>(d_masks_, d_values_, pos_enc_, in0_, in_ld_, B, stream_); });
   Gemm("gemm_embedding", in0_, in_ld_, emb_lin_, x_, emb_, T, default_act_);
+  // fp8: the large GEMMs read e4m3 operands written by the kernel that produces each tensor.
+  const bool f8 = fp8_ && !calibrating_;
+  const size_t nx = static_cast<size_t>(T) * emb_;
+  if (calibrating_) RecordAbsMax(x_, nx, 0);
+  if (f8 && q_qkv_) {
+    Timed("quantize_f8", 0.0, 3.0 * nx,
+          [&] { LaunchQuantizeF8(x_, xq_, static_cast<long long>(nx), 1.0f / encoders_[0].s_x, stream_); });
+  }
 
   for (size_t li = 0; li < encoders_.size(); li++) {
     const EncoderDev& e = encoders_[li];
+    const bool last = li + 1 == encoders_.size();
     const half_t* bias = nullptr;
     // The smolgen chain depends only on x: it runs on the side stream next to the
     // QKV projection (on the main stream when profiling, for clean per-kernel times).
@@ -887,20 +1136,57 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       if (ss != stream_) HIP_CHECK(hipEventRecord(join_events_[li], ss));
       bias = sbias_;
     }
-    Gemm("gemm_qkv", x_, emb_, e.qkv, qkv_, 3 * d_model_, T, kActNone);
+    if (f8 && q_qkv_) {
+      GemmF8("gemm_qkv", xq_, e.qkv, e.qkv8, qkv_, T, kActNone, false, 1.0f);
+    } else {
+      Gemm("gemm_qkv", x_, emb_, e.qkv, qkv_, 3 * d_model_, T, kActNone);
+    }
     if (e.has_smolgen && ss != stream_) HIP_CHECK(hipStreamWaitEvent(stream_, join_events_[li], 0));
-    Timed("attention", 4.0 * 2 * 64 * 64 * 32 * B * heads_ / 2.0,
-          B * heads_ * (2.0 * (3 * 64 * 32 + 64 * 32) + (bias ? 2.0 * 4096 : 0.0)),
-          [&] { LaunchAttention(qkv_, bias, att_, B, heads_, 1.0f / std::sqrt(32.0f), stream_); });
-    Gemm("gemm_mha_dense", att_, d_model_, e.dense, t_, emb_, T, kActNone);
-    Timed("layer_norm_skip", 0.0, 6.0 * T * emb_, [&] {
-      LaunchLayerNorm(t_, x_, x_, e.ln1_g, e.ln1_b, T, emb_, alpha_, eps_, stream_);
+    const double att_flops = 4.0 * 2 * 64 * 64 * 32 * B * heads_ / 2.0;
+    const bool att_f8 = f8 && q_dense_;
+    const double att_bytes =
+        B * heads_ * (2.0 * 3 * 64 * 32 + (att_f8 ? 1.0 : 2.0) * 64 * 32 + (bias ? 2.0 * 4096 : 0.0));
+    const float att_scale = 1.0f / std::sqrt(32.0f);
+    if (att_f8) {
+      Timed("attention", att_flops, att_bytes,
+            [&] { LaunchAttentionF8Out(qkv_, bias, attq_, 1.0f / e.s_att, B, heads_, att_scale, stream_); });
+      GemmF8("gemm_mha_dense", attq_, e.dense, e.dense8, t_, T, kActNone, false, 1.0f);
+    } else {
+      Timed("attention", att_flops, att_bytes,
+            [&] { LaunchAttention(qkv_, bias, att_, B, heads_, att_scale, stream_); });
+      if (calibrating_) RecordAbsMax(att_, static_cast<size_t>(T) * d_model_, static_cast<int>(4 * li + 1));
+      Gemm("gemm_mha_dense", att_, d_model_, e.dense, t_, emb_, T, kActNone);
+    }
+    const bool ln1_f8 = f8 && q_ffn1_;
+    Timed("layer_norm_skip", 0.0, (ln1_f8 ? 7.0 : 6.0) * T * emb_, [&] {
+      LaunchLayerNorm(t_, x_, x_, e.ln1_g, e.ln1_b, T, emb_, alpha_, eps_, stream_, ln1_f8 ? xq_ : nullptr,
+                      1.0f / e.s_x1);
     });
-    Gemm("gemm_ffn1", x_, emb_, e.ffn1, ffn_, dff_, T, ffn_act_);
-    Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, t_, emb_, T, kActNone);
-    Timed("layer_norm_skip", 0.0, 6.0 * T * emb_, [&] {
-      LaunchLayerNorm(t_, x_, x_, e.ln2_g, e.ln2_b, T, emb_, alpha_, eps_, stream_);
+    if (calibrating_) RecordAbsMax(x_, nx, static_cast<int>(4 * li + 2));
+    const bool ffn_f8 = f8 && q_ffn2_;   // FFN2 reads an e4m3 operand
+    if (f8 && q_ffn1_) {
+      GemmF8("gemm_ffn1", xq_, e.ffn1, e.ffn18, ffn_f8 ? static_cast<void*>(ffnq_) : ffn_, T, ffn_act_, ffn_f8,
+             1.0f / e.s_ffn);
+    } else {
+      Gemm("gemm_ffn1", x_, emb_, e.ffn1, ffn_, dff_, T, ffn_act_);
+      if (calibrating_) RecordAbsMax(ffn_, static_cast<size_t>(T) * dff_, static_cast<int>(4 * li + 3));
+      if (ffn_f8) {
+        const size_t nf = static_cast<size_t>(T) * dff_;
+        Timed("quantize_f8", 0.0, 3.0 * nf,
+              [&] { LaunchQuantizeF8(ffn_, ffnq_, static_cast<long long>(nf), 1.0f / e.s_ffn, stream_); });
+      }
+    }
+    if (ffn_f8) {
+      GemmF8("gemm_ffn2", ffnq_, e.ffn2, e.ffn28, t_, T, kActNone, false, 1.0f);
+    } else {
+      Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, t_, emb_, T, kActNone);
+    }
+    const bool ln2_f8 = f8 && q_qkv_ && !last;
+    Timed("layer_norm_skip", 0.0, (ln2_f8 ? 7.0 : 6.0) * T * emb_, [&] {
+      LaunchLayerNorm(t_, x_, x_, e.ln2_g, e.ln2_b, T, emb_, alpha_, eps_, stream_, ln2_f8 ? xq_ : nullptr,
+                      last ? 1.0f : 1.0f / encoders_[li + 1].s_x);
     });
+    if (calibrating_) RecordAbsMax(x_, nx, static_cast<int>(4 * li + 4));
   }
 
   // Value head.

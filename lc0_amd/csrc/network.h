@@ -93,6 +93,9 @@ class Network {
   // resident in HBM) and returns the mean milliseconds per pass measured with
   // HIP events on the compute stream.
   virtual double TimeResidentForward(int batch, int iters) = 0;
+  // precision=fp8 only: re-derives the per-tensor activation scales from the maxima
+  // that these n positions (packed planes as for AddInputs) produce in an fp16 pass.
+  virtual void CalibrateFp8(int n, const uint64_t* masks, const float* values) = 0;
 };
 
 // Factory: the counterpart of MakeBlasNetwork (src/neural/backends/blas/network_blas.cc:1115-1182).

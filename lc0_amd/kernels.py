@@ -27,6 +27,10 @@ def _lib():
         lib.lc0mi_k_expand_planes_attn.argtypes = [vp, vp, ci, ci, vp, ci, cd]
         lib.lc0mi_k_expand_planes_nchw.argtypes = [vp, vp, ci, vp]
         lib.lc0mi_k_attn_policy_gather.argtypes = [vp, vp, vp, ci, ci, vp]
+        lib.lc0mi_k_gemm_f8.argtypes = [vp, ci, vp, ci, vp, vp, ci, ci, ci, ci, ci, cf, vp, ci, ci, cd]
+        lib.lc0mi_k_quantize_f8.argtypes = [vp, ll, cf, vp]
+        lib.lc0mi_k_layer_norm_f8.argtypes = [vp, vp, vp, vp, ci, ci, cf, cf, cf, vp, vp]
+        lib.lc0mi_k_attention_f8.argtypes = [vp, vp, ci, ci, cf, cf, vp]
         lib._k_ready = True
     return lib
 
@@ -123,6 +127,49 @@ def attention(qkv, bias, batch, heads, scale, time_iters=0):
     ms = C.c_double(0)
     _check(_lib().lc0mi_k_attention(_ptr(qkv), _ptr(b), batch, heads, scale, _ptr(out), time_iters, C.byref(ms)))
     return (out, ms.value) if time_iters else out
+
+
+def gemm_f8(a, w, col_scale, bias=None, act=ACT_NONE, out_f8=False, out_mul=1.0, time_iters=0):
+    """a [M,K], w [N,K] uint8 e4m3 -> act(col_scale * a.w^T + bias) as half (or e4m3 bytes of it * out_mul)."""
+    a = np.ascontiguousarray(a, np.uint8)
+    w = np.ascontiguousarray(w, np.uint8)
+    cs = np.ascontiguousarray(col_scale, np.float32)
+    b = np.ascontiguousarray(bias, np.float32) if bias is not None else None
+    m, k = a.shape
+    n = w.shape[0]
+    out = np.zeros((m, n), np.uint8 if out_f8 else np.float16)
+    ms = C.c_double(0)
+    _check(_lib().lc0mi_k_gemm_f8(_ptr(a), k, _ptr(w), k, _ptr(cs), _ptr(b), m, n, k, act, int(out_f8),
+                                  C.c_float(out_mul), _ptr(out), n, time_iters, C.byref(ms)))
+    return (out, ms.value) if time_iters else out
+
+
+def quantize_f8(x, mul=1.0):
+    x = _h(x)
+    y = np.zeros(x.shape, np.uint8)
+    _check(_lib().lc0mi_k_quantize_f8(_ptr(x), C.c_longlong(x.size), C.c_float(mul), _ptr(y)))
+    return y
+
+
+def layer_norm_f8(x, skip, gamma, beta, alpha, eps, f8_mul):
+    x = _h(x)
+    s = _h(skip) if skip is not None else None
+    g = np.ascontiguousarray(gamma, np.float32)
+    b = np.ascontiguousarray(beta, np.float32)
+    y = np.zeros_like(x)
+    yq = np.zeros(x.shape, np.uint8)
+    _check(_lib().lc0mi_k_layer_norm_f8(_ptr(x), _ptr(s), _ptr(g), _ptr(b), x.shape[0], x.shape[1], C.c_float(alpha),
+                                        C.c_float(eps), C.c_float(f8_mul), _ptr(y), _ptr(yq)))
+    return y, yq
+
+
+def attention_f8(qkv, bias, batch, heads, scale, out_mul):
+    qkv = _h(qkv)
+    b = _h(bias) if bias is not None else None
+    out = np.zeros((batch * 64, heads * 32), np.uint8)
+    _check(_lib().lc0mi_k_attention_f8(_ptr(qkv), _ptr(b), batch, heads, C.c_float(scale), C.c_float(out_mul),
+                                       _ptr(out)))
+    return out
 
 
 def expand_planes_attn(masks, values, ld=176, time_iters=0):

@@ -162,6 +162,8 @@ CONFIGS = {
     "tiny_resnet_convpolicy": lambda: se_resnet(32, 2, 8, seed=2003, conv_policy=True),
     "tiny_resnet_nose": lambda: se_resnet(24, 3, 0, seed=2004, moves_left=True),
     "tiny_attn": lambda: attention_body(64, 2, 2, 96, seed=2001, smolgen=(8, 32, 32), perturb_ln=True),
+    # smallest shape the fp8 configuration accepts (all widths multiples of 128)
+    "tiny_attn_f8": lambda: attention_body(128, 3, 4, 256, seed=2005, smolgen=(8, 32, 32), perturb_ln=True),
     "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True),
 }
 

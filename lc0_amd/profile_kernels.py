@@ -3,6 +3,7 @@ counters to it. Meant to be launched under the profiler:
 
   rocprofv3 --pmc FETCH_SIZE -- python3 -m lc0_amd.profile_kernels copy --mib 256
   rocprofv3 --pmc WRITE_SIZE -- python3 -m lc0_amd.profile_kernels gemm --m 16384 --n 3072 --k 1024
+  rocprofv3 --kernel-trace --stats -- python3 -m lc0_amd.profile_kernels gemm_f8 --m 16384 --n 3072 --k 1024
   rocprofv3 --kernel-trace --stats -- python3 -m lc0_amd.profile_kernels attention --batch 256 --heads 32
 
 `copy` moves a known number of bytes (reads N, writes N) and calibrates the HBM byte counters.
@@ -18,7 +19,7 @@ from .backend import load_library
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("kernel", choices=["copy", "gemm", "attention", "layer_norm", "expand"])
+    ap.add_argument("kernel", choices=["copy", "gemm", "gemm_f8", "attention", "layer_norm", "expand"])
     ap.add_argument("--mib", type=int, default=256)
     ap.add_argument("--m", type=int, default=16384)
     ap.add_argument("--n", type=int, default=3072)
@@ -26,7 +27,10 @@ def main():
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--heads", type=int, default=32)
     ap.add_argument("--iters", type=int, default=5)
+    ap.add_argument("--variant", type=int, default=-1, help="force a GEMM tile variant (see kernels.set_gemm_variant)")
     args = ap.parse_args()
+    if args.variant >= 0:
+        K.set_gemm_variant(args.variant)
     rng = np.random.default_rng(0)
     if args.kernel == "copy":
         lib = load_library()
@@ -42,6 +46,12 @@ def main():
         _, ms = K.gemm(a, w, np.zeros(args.n, np.float32), time_iters=args.iters)
         print("gemm %dx%dx%d: %.1f us, %.0f TFLOP/s" % (args.m, args.n, args.k, ms * 1e3,
                                                        2.0 * args.m * args.n * args.k / (ms * 1e-3) / 1e12))
+    elif args.kernel == "gemm_f8":
+        a = rng.integers(0, 120, (args.m, args.k), dtype=np.uint8) | (rng.integers(0, 2, (args.m, args.k), dtype=np.uint8) << 7)
+        w = rng.integers(0, 127, (args.n, args.k), dtype=np.uint8) | (rng.integers(0, 2, (args.n, args.k), dtype=np.uint8) << 7)
+        _, ms = K.gemm_f8(a, w, np.full(args.n, 1e-3, np.float32), np.zeros(args.n, np.float32), time_iters=args.iters)
+        print("gemm_f8 %dx%dx%d: %.1f us, %.0f TFLOP/s" % (args.m, args.n, args.k, ms * 1e3,
+                                                          2.0 * args.m * args.n * args.k / (ms * 1e-3) / 1e12))
     elif args.kernel == "attention":
         d = args.heads * 32
         qkv = rng.standard_normal((args.batch * 64, 3 * d), dtype=np.float32).astype(np.float16)

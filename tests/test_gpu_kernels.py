@@ -210,3 +210,82 @@ def test_expand_planes_nhwc_bit_exact():
     pos = oc.random_positions(9, seed=6)
     want = onn.encode_planes(pos["masks"], pos["values"]).transpose(0, 2, 1)
     assert np.array_equal(K.expand_planes_nhwc(pos["masks"], pos["values"]), want)
+
+
+# ---- e4m3 (fp8) kernels -----------------------------------------------------
+def _f8_close(got_codes, want_values, mul, tol=2e-3):
+    """Quantised outputs: the kernel quantises its own fp32 value, which differs from the oracle's by
+    up to tol (absolute and relative, the bound of the unquantised tests); so the decoded code must
+    lie within half an e4m3 step plus that of the oracle value, and nearly all codes must be equal."""
+    from oracle import fp8
+    got = fp8.e4m3_decode(got_codes).astype(np.float64)
+    want = np.clip(np.asarray(want_values, np.float64) * mul, -448, 448)
+    step = np.maximum(2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -6))) - 3), 2.0 ** -9)
+    excess = np.abs(got - want) - (0.5 * step + tol * mul + tol * np.abs(want))
+    assert excess.max() <= 0, excess.max()
+    exact = fp8.e4m3_encode(want.astype(f32))
+    assert (exact == got_codes).mean() > 0.97
+
+
+def test_quantize_f8_bit_exact():
+    """Every fp16 value (x scale) -> e4m3: bit-exact against the oracle codec (NaN inputs excluded:
+    the reference maps them to 0x7f, the kernel's clamp to +-448)."""
+    from lc0_amd import kernels as K
+    from oracle import fp8
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16)
+    halves = halves[~np.isnan(halves)]
+    halves = np.concatenate([halves, np.zeros((-len(halves)) % 8, np.float16)])
+    for mul in (1.0, 0.37, 16.0):
+        got = K.quantize_f8(halves, mul)
+        want = fp8.e4m3_encode(halves.astype(f32) * f32(mul))
+        np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2])
+@pytest.mark.parametrize("m,n,k", [(512, 512, 128), (300, 200, 256), (2048, 1536, 1024), (64, 3072, 1024), (1, 17, 128)])
+def test_gemm_f8_vs_exact_product(variant, m, n, k):
+    """e4m3 operands are exact inputs, so the product is pinned by float64 arithmetic on the decoded
+    values; tolerance covers fp32 accumulation and the fp16 output rounding."""
+    from lc0_amd import kernels as K
+    from oracle import fp8
+    rng = np.random.default_rng(m + n + k)
+    a = fp8.e4m3_encode(rng.standard_normal((m, k)) * 2)
+    w, wscale = fp8.quantize_rows(rng.standard_normal((n, k)) * 0.05)
+    b = rng.standard_normal(n).astype(f32)
+    sa = f32(0.031)
+    exact = (fp8.e4m3_decode(a).astype(np.float64) @ fp8.e4m3_decode(w).astype(np.float64).T) * (sa * wscale) + b
+    K.set_gemm_variant(variant)
+    try:
+        got = K.gemm_f8(a, w, sa * wscale, b).astype(np.float64)
+        np.testing.assert_allclose(got, exact, rtol=2e-3, atol=2e-3)
+        want_act = onn.activate(exact.astype(f32), nr.ACT_MISH)
+        got8 = K.gemm_f8(a, w, sa * wscale, b, act=nr.ACT_MISH, out_f8=True, out_mul=20.0)
+        _f8_close(got8, want_act, 20.0)
+    finally:
+        K.set_gemm_variant(-1)
+
+
+def test_layer_norm_f8_output():
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(77)
+    x = _h(rng.standard_normal((200, 1024)))
+    s = _h(rng.standard_normal((200, 1024)))
+    g = (1 + 0.1 * rng.standard_normal(1024)).astype(f32)
+    b = (0.1 * rng.standard_normal(1024)).astype(f32)
+    want = onn.layer_norm_skip(x, 0.427, s, g, b, 1e-6)
+    y, yq = K.layer_norm_f8(x, s, g, b, 0.427, 1e-6, 50.0)
+    np.testing.assert_allclose(y.astype(f32), want, rtol=2e-3, atol=2e-3)
+    _f8_close(yq, want, 50.0)
+    np.testing.assert_array_equal(y, K.layer_norm(x, s, g, b, 0.427, 1e-6))   # the fp16 output is unchanged
+
+
+def test_attention_f8_output_matches_half_output():
+    from lc0_amd import kernels as K
+    from oracle import fp8
+    rng = np.random.default_rng(78)
+    batch, heads = 3, 4
+    qkv = _h(rng.standard_normal((batch * 64, 3 * heads * 32)))
+    bias = _h(rng.standard_normal((batch, heads, 64, 64)))
+    half_out = K.attention(qkv, bias, batch, heads, 32 ** -0.5).astype(f32)
+    got = K.attention_f8(qkv, bias, batch, heads, 32 ** -0.5, 100.0)
+    _f8_close(got, half_out, 100.0)   # same fp32 result, rounded to e4m3 instead of fp16 (fp16 error << e4m3 step)

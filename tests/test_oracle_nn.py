@@ -360,3 +360,45 @@ def test_fast_exp_and_legal_softmax(ref):
     legal = np.array([3, 77, 500, 1857])
     p = onn.softmax_policy_legal(logits, legal)
     assert abs(p.sum() - 1) < 1e-5 and p.argmax() == logits[legal].argmax()
+
+
+def test_e4m3_codec_vs_compiled_reference(ref):
+    """oracle/fp8.py against FP32toFP8E4M3FN / FP8E4M3FNtoFP32 (fp8_utils.h:111-155): all 256 codes,
+    every fp16 value and random floats including exact ties and the saturation edge."""
+    from oracle import fp8
+    ref.ref_fp32_to_fp8e4m3.argtypes = [ctypes.c_float]
+    ref.ref_fp32_to_fp8e4m3.restype = ctypes.c_uint8
+    ref.ref_fp8e4m3_to_fp32.argtypes = [ctypes.c_uint8]
+    ref.ref_fp8e4m3_to_fp32.restype = ctypes.c_float
+    table = fp8.e4m3_table()
+    for code in range(256):
+        want = ref.ref_fp8e4m3_to_fp32(code)
+        assert (np.isnan(want) and np.isnan(table[code])) or want == table[code]
+    rng = np.random.default_rng(8)
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    mids = (table[:126] + table[1:127]) / 2                       # exact ties between neighbours
+    xs = np.concatenate([halves[~np.isnan(halves)], mids, -mids, [448, 463.9, 464, 465, 1e9, -1e9, np.inf, -np.inf],
+                         rng.standard_normal(20000) * np.exp(rng.uniform(-8, 7, 20000))]).astype(np.float32)
+    got = fp8.e4m3_encode(xs)
+    want = np.array([ref.ref_fp32_to_fp8e4m3(float(v)) for v in xs], np.uint8)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_e4m3_codec_is_nearest_even_by_brute_force():
+    """Textbook definition: the nearest of the 254 finite codes, ties to the even mantissa, saturating."""
+    from oracle import fp8
+    table = fp8.e4m3_table().astype(np.float64)
+    pos = table[:127]                                             # 0 .. 448, increasing
+    rng = np.random.default_rng(9)
+    xs = np.abs(rng.standard_normal(5000) * np.exp(rng.uniform(-8, 6.5, 5000))).astype(np.float32)
+    xs = np.concatenate([xs, ((pos[:-1] + pos[1:]) / 2).astype(np.float32)])
+    got = fp8.e4m3_encode(xs)
+    for x, g in zip(xs.astype(np.float64), got):
+        d = np.abs(pos - min(x, 448.0))
+        best = np.flatnonzero(d == d.min())
+        want = best[0] if len(best) == 1 else [c for c in best if c % 2 == 0][0]
+        assert g == want, (x, g, want)
+    np.testing.assert_array_equal(fp8.e4m3_encode(-xs), got | 0x80)
+    codes, scale = fp8.quantize_rows(np.array([[1.0, -2.0, 0.5], [0, 0, 0]], np.float32))
+    assert scale[0] == np.float32(2.0 / 448) and scale[1] == 1.0
+    np.testing.assert_array_equal(fp8.e4m3_decode(codes[0]) * scale[0], [1.0, -2.0, 0.5])
