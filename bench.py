@@ -40,6 +40,8 @@ WORKLOADS = {
     "c4_bt4_fp8": dict(batch=1024, net="c2_bt4_15x1024", options="precision=fp8", dtype="fp8_e4m3",
                        desc="BT4-shape attention body with e4m3 operands (fp32 accumulation) in the QKV, attention-output "
                             "and FFN GEMMs; weights scaled per output row, activations per tensor; the rest fp16"),
+    "bt4_dense_15x1024": dict(batch=256, desc="BT4 as published: PE_DENSE embedding (64 channels, embedding FFN 1536), "
+                                              "15 layers, d=1024, 32 heads, dff 1536, smolgen, multi-head format, fp16"),
     "tiny_attn": dict(batch=64, desc="tiny smolgen attention body (test net)"),
 }
 
@@ -74,6 +76,8 @@ def main():
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-sample", type=int, default=16)
+    ap.add_argument("--sweep", default="", help="comma-separated batch sizes: adds their resident-batch evals/s "
+                                                "as \"batch_sweep\" to the JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend evaluates on one GPU (batch rows are independent; more GPUs means "
@@ -87,10 +91,14 @@ def main():
     wl = WORKLOADS[args.config]
     batch = args.batch or wl["batch"]
     path = netgen.cached_config(wl.get("net", args.config))
-    pos = oc.random_positions(max(batch, args.cpu_sample), seed=20240)
+    sweep = [int(b) for b in args.sweep.split(",") if b]
+    pos = oc.random_positions(min(max([batch, args.cpu_sample] + sweep), 1024), seed=20240)
     masks, values = pos["masks"], pos["values"]
 
-    net = Network(path, "gpu=0,max_batch=%d" % max(batch, 16) + ("," + wl["options"] if wl.get("options") else ""))
+    if max([batch] + sweep) > masks.shape[0]:
+        reps = -(-max([batch] + sweep) // masks.shape[0])
+        masks, values = np.tile(masks, (reps, 1)), np.tile(values, (reps, 1))
+    net = Network(path, "gpu=0,max_batch=%d" % max([batch, 16] + sweep) + ("," + wl["options"] if wl.get("options") else ""))
     comp = net.NewComputation()
     comp.AddInputs(masks[:batch], values[:batch])
     comp.ComputeBlocking()          # stages the batch into HBM and warms everything up
@@ -166,6 +174,19 @@ def main():
         "sum_kernel_ms_per_step": total_kernel_ms,
         "policy_checksum": checksum,
     }
+    if sweep:
+        result["batch_sweep"] = {}
+        for b in sweep:
+            c = net.NewComputation()
+            c.AddInputs(masks[:b], values[:b])
+            c.ComputeBlocking()
+            iters = max(5, min(200, int(2000 / max(b, 8))))
+            net.TimeResidentForward(b, 3)
+            t0 = time.perf_counter()
+            net.TimeResidentForward(b, iters)
+            ms = (time.perf_counter() - t0) * 1e3 / iters
+            result["batch_sweep"][str(b)] = {"evals_per_s": b / (ms * 1e-3), "ms_per_step": ms}
+            c.close()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(path, masks, values, args.cpu_sample)
     print(json.dumps(result))

@@ -79,6 +79,14 @@ void LaunchGemmF32(const GemmArgsF32& args, hipStream_t stream);
 template <typename T>
 void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T* pos_enc /*[64][64]*/,
                             T* out, int ld, int batch, hipStream_t stream);
+// Same with per-sample extra channels (the dense position encoding): out[b*64+sq][112 + c] =
+// extra[b][sq][c], c < n_extra.
+void LaunchExpandPlanesDense(const uint64_t* masks, const float* values, const half_t* extra, int n_extra,
+                             half_t* out, int ld, int batch, hipStream_t stream);
+// First 12 input planes, square-major: out[b][sq * 12 + j] (input of the dense position-encoding layer).
+void LaunchPiecePlanes(const uint64_t* masks, const float* values, half_t* out, int batch, hipStream_t stream);
+// Input gating: x[b][i] = x[b][i] * mult[i] + add[i], i < per_sample (= 64 * channels, square-major).
+void LaunchInputGating(half_t* x, const float* mult, const float* add, int batch, int per_sample, hipStream_t stream);
 // Input planes -> NCHW dense planes out[b][c][sq] (T = half_t or float).
 template <typename T>
 void LaunchExpandPlanesNchw(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream);

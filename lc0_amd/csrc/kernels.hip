@@ -649,9 +649,11 @@ namespace {
 template <typename T>
 __global__ __launch_bounds__(256) void expand_planes_attn_kernel(const uint64_t* __restrict__ masks,
                                                                  const float* __restrict__ values,
-                                                                 const T* __restrict__ pos_enc, T* __restrict__ out,
-                                                                 int ld) {
+                                                                 const T* __restrict__ extra, int n_extra,
+                                                                 long long extra_batch_stride,
+                                                                 T* __restrict__ out, int ld) {
   const int b = blockIdx.x;
+  const T* ex = extra + (long long)b * extra_batch_stride;
   __shared__ uint64_t smask[112];
   __shared__ float sval[112];
   if (threadIdx.x < 112) {
@@ -665,11 +667,33 @@ __global__ __launch_bounds__(256) void expand_planes_attn_kernel(const uint64_t*
     T v = (T)0.0f;
     if (c < 112) {
       if ((smask[c] >> sq) & 1ull) v = (T)sval[c];
-    } else if (c < 176) {
-      v = pos_enc[sq * 64 + (c - 112)];
+    } else if (c < 112 + n_extra) {
+      v = ex[sq * n_extra + (c - 112)];
     }
     o[i] = v;
   }
+}
+
+// First 12 planes (the current position's pieces) square-major: out[b][sq * 12 + j].
+__global__ __launch_bounds__(256) void piece_planes_kernel(const uint64_t* __restrict__ masks,
+                                                           const float* __restrict__ values,
+                                                           half_t* __restrict__ out) {
+  const int b = blockIdx.x;
+  for (int i = threadIdx.x; i < 64 * 12; i += 256) {
+    const int sq = i / 12, j = i - sq * 12;
+    const bool bit = (masks[(long long)b * 112 + j] >> sq) & 1ull;
+    out[(long long)b * 768 + i] = bit ? (half_t)values[(long long)b * 112 + j] : (half_t)0.0f;
+  }
+}
+
+// x[b][sq][c] = x * mult[sq][c] + add[sq][c]
+__global__ __launch_bounds__(256) void input_gating_kernel(half_t* __restrict__ x, const float* __restrict__ mult,
+                                                           const float* __restrict__ add, int per_sample,
+                                                           long long total) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int j = (int)(i % per_sample);
+  x[i] = (half_t)((float)x[i] * mult[j] + add[j]);
 }
 
 template <typename T>
@@ -688,8 +712,27 @@ template <typename T>
 void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T* pos_enc, T* out, int ld,
                             int batch, hipStream_t stream) {
   if (batch <= 0) return;
-  hipLaunchKernelGGL(expand_planes_attn_kernel<T>, dim3(batch), dim3(256), 0, stream, masks, values, pos_enc, out,
-                     ld);
+  hipLaunchKernelGGL(expand_planes_attn_kernel<T>, dim3(batch), dim3(256), 0, stream, masks, values, pos_enc, 64, 0LL,
+                     out, ld);
+}
+
+void LaunchExpandPlanesDense(const uint64_t* masks, const float* values, const half_t* extra, int n_extra,
+                             half_t* out, int ld, int batch, hipStream_t stream) {
+  if (batch <= 0) return;
+  hipLaunchKernelGGL(expand_planes_attn_kernel<half_t>, dim3(batch), dim3(256), 0, stream, masks, values, extra,
+                     n_extra, 64LL * n_extra, out, ld);
+}
+
+void LaunchPiecePlanes(const uint64_t* masks, const float* values, half_t* out, int batch, hipStream_t stream) {
+  if (batch <= 0) return;
+  hipLaunchKernelGGL(piece_planes_kernel, dim3(batch), dim3(256), 0, stream, masks, values, out);
+}
+
+void LaunchInputGating(half_t* x, const float* mult, const float* add, int batch, int per_sample, hipStream_t stream) {
+  const long long total = (long long)batch * per_sample;
+  if (total <= 0) return;
+  hipLaunchKernelGGL(input_gating_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, mult, add,
+                     per_sample, total);
 }
 template void LaunchExpandPlanesAttn<half_t>(const uint64_t*, const float*, const half_t*, half_t*, int, int,
                                              hipStream_t);

@@ -298,6 +298,14 @@ class Mi355xNetwork : public Network {
   int pol_emb_ = 0, pol_d_ = 0, val_ch_ = 0, val_fc_ = 0, val_out_ = 0, mov_ch_ = 0, mov_fc_ = 0;
   float alpha_ = 1.0f, eps_ = 1e-6f;
   bool any_smolgen_ = false;
+  // Dense position encoding (PE_DENSE nets): preprocessing layer, embedding layer norm and
+  // embedding FFN; optional input gating.
+  bool pe_dense_ = false, gating_ = false;
+  int enc_ch_ = 0, emb_dff_ = 0;
+  Linear preproc_lin_, emb_ffn1_, emb_ffn2_;
+  float *emb_ln_g_ = nullptr, *emb_ln_b_ = nullptr, *emb_ffn_ln_g_ = nullptr, *emb_ffn_ln_b_ = nullptr;
+  float *gate_mult_ = nullptr, *gate_add_ = nullptr;   // [64][emb]
+  half_t *pre_in_ = nullptr, *pre_out_ = nullptr;
 
   // Device weights.
   Linear emb_lin_, smolgen_w_, pol_emb_lin_, pol_qk_lin_, val_emb_lin_, val_fc1_, val_fc2_, mov_emb_lin_, mov_fc1_,
@@ -721,10 +729,11 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   const NetWeights& w = file.weights;
   const NetworkFormat& nf = file.format;
   if (!w.residual.empty()) throw Error("Attention body on top of a residual tower is not supported.");
-  if (nf.input_embedding != kInputEmbeddingPeMap) {
-    throw Error("Only the PE_MAP input embedding is supported by the mi355x backend.");
+  pe_dense_ = nf.input_embedding == kInputEmbeddingPeDense;
+  if (!pe_dense_ && nf.input_embedding != kInputEmbeddingPeMap) {
+    throw Error("The attention body needs the PE_MAP or PE_DENSE input embedding.");
   }
-  if (!w.ip_mult_gate.empty() || !w.ip_add_gate.empty()) throw Error("Input gating is not supported.");
+  gating_ = !w.ip_mult_gate.empty() && !w.ip_add_gate.empty();
   if (!attn_policy_) throw Error("Attention-body networks need the attention policy head.");
   const PolicyHead& ph = w.policy_heads.at(policy_head_);
   const ValueHead& vh = w.value_heads.at(value_head_);
@@ -739,10 +748,41 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   if (d_model_ != heads_ * 32) throw Error("Only attention heads of depth 32 are supported.");
   if (dff_ % 8 != 0) throw Error("FFN width must be a multiple of 8.");
   alpha_ = static_cast<float>(std::pow(2.0 * w.encoder.size(), -0.25));
-  eps_ = 1e-6f;
+  eps_ = pe_dense_ ? 1e-3f : 1e-6f;   // src/neural/backends/blas/network_blas.cc:719
 
-  emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + 64);
+  if (pe_dense_) {
+    // src/neural/backends/blas/network_blas.cc:612-628, 662-712
+    if (w.ip_emb_preproc_b.empty() || w.ip_emb_preproc_b.size() % 64) throw Error("Bad dense position-encoding weights.");
+    enc_ch_ = static_cast<int>(w.ip_emb_preproc_b.size() / 64);
+    preproc_lin_ = MakeLinear(w.ip_emb_preproc_w, w.ip_emb_preproc_b, 64 * enc_ch_, 64 * 12);
+    emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + enc_ch_);
+    if (static_cast<int>(w.ip_emb_ln_gammas.size()) != emb_ || static_cast<int>(w.ip_emb_ln_betas.size()) != emb_) {
+      throw Error("Embedding layer norm parameters do not match the embedding size.");
+    }
+    emb_ln_g_ = UploadF(w.ip_emb_ln_gammas); emb_ln_b_ = UploadF(w.ip_emb_ln_betas);
+    emb_dff_ = static_cast<int>(w.ip_emb_ffn.dense1_b.size());
+    if (emb_dff_ <= 0 || emb_dff_ % 8) throw Error("Embedding FFN width must be a positive multiple of 8.");
+    emb_ffn1_ = MakeLinear(w.ip_emb_ffn.dense1_w, w.ip_emb_ffn.dense1_b, emb_dff_, emb_);
+    emb_ffn2_ = MakeLinear(w.ip_emb_ffn.dense2_w, w.ip_emb_ffn.dense2_b, emb_, emb_dff_);
+    if (static_cast<int>(w.ip_emb_ffn_ln_gammas.size()) != emb_) throw Error("Embedding FFN layer norm has a wrong size.");
+    emb_ffn_ln_g_ = UploadF(w.ip_emb_ffn_ln_gammas); emb_ffn_ln_b_ = UploadF(w.ip_emb_ffn_ln_betas);
+  } else {
+    emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + 64);
+  }
   in_ld_ = emb_lin_.ld;
+  if (gating_) {
+    // Stored [channel][square] (network_blas.cc:670-682); kept [square][channel] like the activations.
+    if (w.ip_mult_gate.size() != static_cast<size_t>(64) * emb_ || w.ip_add_gate.size() != w.ip_mult_gate.size()) {
+      throw Error("Input gating weights have a wrong size.");
+    }
+    Vec mult(w.ip_mult_gate.size()), add(w.ip_add_gate.size());
+    for (int c = 0; c < emb_; c++)
+      for (int sq = 0; sq < 64; sq++) {
+        mult[static_cast<size_t>(sq) * emb_ + c] = w.ip_mult_gate[static_cast<size_t>(c) * 64 + sq];
+        add[static_cast<size_t>(sq) * emb_ + c] = w.ip_add_gate[static_cast<size_t>(c) * 64 + sq];
+      }
+    gate_mult_ = UploadF(mult); gate_add_ = UploadF(add);
+  }
   {
     const std::vector<float>& pe = PosEncoding();
     std::vector<half_t> h(pe.size());
@@ -851,7 +891,11 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   t_ = AllocH(T * emb_);
   qkv_ = AllocH(T * 3 * d_model_);
   att_ = AllocH(T * d_model_);
-  ffn_ = AllocH(T * dff_);
+  ffn_ = AllocH(T * std::max(dff_, emb_dff_));
+  if (pe_dense_) {
+    pre_in_ = AllocH(static_cast<size_t>(max_batch_) * 768);
+    pre_out_ = AllocH(T * enc_ch_);
+  }
   if (any_smolgen_) {
     sg1_ = AllocH(T * sg_hc_);
     sg2_ = AllocH(static_cast<size_t>(max_batch_) * sg_hs_);
@@ -1093,9 +1137,32 @@ void Mi355xNetwork::ForwardResnet(int B) {
 // ------------------------------------------------------------------ forward --
 void Mi355xNetwork::ForwardAttentionBody(int B) {
   const int T = B * 64;
-  Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * 2),
-        [&] { LaunchExpandPlanesAttn<half_t>(d_masks_, d_values_, pos_enc_, in0_, in_ld_, B, stream_); });
+  if (pe_dense_) {
+    Timed("piece_planes", 0.0, B * (12.0 * 12 + 768.0 * 2), [&] { LaunchPiecePlanes(d_masks_, d_values_, pre_in_, B, stream_); });
+    Gemm("gemm_pos_encoding", pre_in_, 768, preproc_lin_, pre_out_, 64 * enc_ch_, B, kActNone);
+    Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * 2 + 64.0 * enc_ch_ * 2), [&] {
+      LaunchExpandPlanesDense(d_masks_, d_values_, pre_out_, enc_ch_, in0_, in_ld_, B, stream_);
+    });
+  } else {
+    Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * 2),
+          [&] { LaunchExpandPlanesAttn<half_t>(d_masks_, d_values_, pos_enc_, in0_, in_ld_, B, stream_); });
+  }
   Gemm("gemm_embedding", in0_, in_ld_, emb_lin_, x_, emb_, T, default_act_);
+  if (pe_dense_) {
+    Timed("layer_norm_skip", 0.0, 4.0 * T * emb_, [&] {
+      LaunchLayerNorm(x_, nullptr, x_, emb_ln_g_, emb_ln_b_, T, emb_, 1.0f, 1e-3f, stream_);
+    });
+  }
+  if (gating_) {
+    Timed("input_gating", 0.0, 4.0 * T * emb_, [&] { LaunchInputGating(x_, gate_mult_, gate_add_, B, 64 * emb_, stream_); });
+  }
+  if (pe_dense_) {
+    Gemm("gemm_emb_ffn1", x_, emb_, emb_ffn1_, ffn_, emb_dff_, T, ffn_act_);
+    Gemm("gemm_emb_ffn2", ffn_, emb_dff_, emb_ffn2_, t_, emb_, T, kActNone);
+    Timed("layer_norm_skip", 0.0, 6.0 * T * emb_, [&] {
+      LaunchLayerNorm(t_, x_, x_, emb_ffn_ln_g_, emb_ffn_ln_b_, T, emb_, alpha_, 1e-3f, stream_);
+    });
+  }
   // fp8: the large GEMMs read e4m3 operands written by the kernel that produces each tensor.
   const bool f8 = fp8_ && !calibrating_;
   const size_t nx = static_cast<size_t>(T) * emb_;

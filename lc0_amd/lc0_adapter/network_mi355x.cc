@@ -10,9 +10,13 @@
 // It is not compiled as part of liblc0mi.so: it needs lc0's headers.
 #include <memory>
 #include <optional>
+#include <random>
 #include <string>
+#include <vector>
 
+#include "chess/position.h"
 #include "lc0mi.h"
+#include "neural/encoder.h"
 #include "neural/factory.h"
 #include "neural/network.h"
 #include "utils/exception.h"
@@ -76,7 +80,11 @@ class Mi355xNetwork : public Network {
     };
     add("gpu", std::to_string(options.GetOrDefault<int>("gpu", 0)));
     add("max_batch", std::to_string(options.GetOrDefault<int>("max_batch", 1024)));
-    add("precision", options.GetOrDefault<std::string>("precision", "fp16"));
+    const std::string precision = options.GetOrDefault<std::string>("precision", "fp16");
+    add("precision", precision);
+    if (precision == "fp8") {
+      add("fp8_gemms", options.GetOrDefault<std::string>("fp8_gemms", "qkv+dense+ffn1+ffn2"));
+    }
     add("policy_head", options.GetOrDefault<std::string>("policy_head", "vanilla"));
     add("value_head", options.GetOrDefault<std::string>("value_head", "winner"));
     add("mlh", options.GetOrDefault<bool>("mlh", true) ? "true" : "false");
@@ -88,8 +96,38 @@ class Mi355xNetwork : public Network {
                      static_cast<pblczero::NetworkFormat::OutputFormat>(out),
                      static_cast<pblczero::NetworkFormat::MovesLeftFormat>(mlh)};
     Check(lc0mi_net_hints(net_, &minibatch_, &batch_step_, nullptr, &threads_, nullptr));
+    if (precision == "fp8") CalibrateFp8(capabilities_.input_format);
   }
   ~Mi355xNetwork() override { lc0mi_net_destroy(net_); }
+
+  // The library calibrates its fp8 activation scales on built-in pseudo-positions; here
+  // lc0's own move generator and encoder are at hand, so it gets real ones instead:
+  // positions reached by seeded uniform-random legal playouts from the start position.
+  void CalibrateFp8(pblczero::NetworkFormat::InputFormat input_format) {
+    constexpr int kPositions = 256;
+    std::vector<uint64_t> masks(static_cast<size_t>(kPositions) * kInputPlanes);
+    std::vector<float> values(masks.size());
+    std::mt19937 rng(20240);
+    int filled = 0;
+    while (filled < kPositions) {
+      PositionHistory history;
+      history.Reset(ChessBoard::kStartposBoard, 0, 1);
+      const int plies = 10 + static_cast<int>(rng() % 71);
+      for (int ply = 0; ply < plies; ++ply) {
+        const MoveList moves = history.Last().GetBoard().GenerateLegalMoves();
+        if (moves.empty() || history.ComputeGameResult() != GameResult::UNDECIDED) break;
+        history.Append(moves[rng() % moves.size()]);
+      }
+      const InputPlanes planes =
+          EncodePositionForNN(input_format, history, 8, FillEmptyHistory::FEN_ONLY, nullptr);
+      for (int i = 0; i < kInputPlanes; ++i) {
+        masks[static_cast<size_t>(filled) * kInputPlanes + i] = planes[i].mask;
+        values[static_cast<size_t>(filled) * kInputPlanes + i] = planes[i].value;
+      }
+      ++filled;
+    }
+    Check(lc0mi_net_calibrate_fp8(net_, kPositions, masks.data(), values.data()));
+  }
 
   const NetworkCapabilities& GetCapabilities() const override { return capabilities_; }
   std::unique_ptr<NetworkComputation> NewComputation() override {

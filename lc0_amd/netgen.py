@@ -19,12 +19,13 @@ INPUT_CLASSICAL_112_PLANE = 1
 OUTPUT_WDL = 2
 NETWORK_SE_WITH_HEADFORMAT = 4
 NETWORK_ATTENTIONBODY_WITH_HEADFORMAT = 6
+NETWORK_ATTENTIONBODY_WITH_MULTIHEADFORMAT = 7
 POLICY_CLASSICAL, POLICY_CONVOLUTION, POLICY_ATTENTION = 1, 2, 3
 VALUE_WDL = 2
 MOVES_LEFT_NONE, MOVES_LEFT_V1 = 0, 1
 DEFAULT_ACTIVATION_RELU, DEFAULT_ACTIVATION_MISH = 0, 1
 ACTIVATION_DEFAULT, ACTIVATION_SWISH = 0, 7
-INPUT_EMBEDDING_PE_MAP = 1
+INPUT_EMBEDDING_PE_MAP, INPUT_EMBEDDING_PE_DENSE = 1, 2
 
 
 class _Gen:
@@ -80,11 +81,15 @@ def se_resnet(filters, blocks, se_channels, seed, policy_channels=32, value_chan
 
 def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_std=0.02,
                    policy_d=None, value_channels=32, value_fc=128, mlh_channels=32, mlh_fc=128,
-                   perturb_ln=False):
-    """Attention-body net (PE_MAP embedding, attention policy, WDL, MLH).
+                   perturb_ln=False, pe_dense=None, gating=False, multihead=False):
+    """Attention-body net (attention policy, WDL, MLH).
 
     smolgen = (hidden_channels, hidden_sz, gen_sz) or None. Weights N(0, std),
     LayerNorm gamma=1 / beta=0 unless perturb_ln (tests).
+    pe_dense = (enc_channels, emb_ffn_width): PE_DENSE input embedding with its layer norm and
+    embedding FFN (src/neural/backends/blas/network_blas.cc:612-712) instead of PE_MAP.
+    gating: ip_mult_gate / ip_add_gate. multihead: network format 7 with policy heads
+    vanilla / optimistic_st / soft (shared embedding) and value heads winner / q / st.
     """
     g = _Gen(seed)
     d_model = emb
@@ -100,7 +105,20 @@ def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_s
         return np.ones(n, np.float32), np.zeros(n, np.float32)
 
     w = {}
-    w["ip_emb_w"], w["ip_emb_b"] = fc(emb, 112 + 64)
+    if pe_dense:
+        enc_ch, emb_dff = pe_dense
+        w["ip_emb_preproc_w"], w["ip_emb_preproc_b"] = fc(64 * enc_ch, 64 * 12)
+        w["ip_emb_w"], w["ip_emb_b"] = fc(emb, 112 + enc_ch)
+        w["ip_emb_ln_gammas"], w["ip_emb_ln_betas"] = ln(emb)
+        w["ip_emb_ffn"] = {}
+        w["ip_emb_ffn"]["dense1_w"], w["ip_emb_ffn"]["dense1_b"] = fc(emb_dff, emb)
+        w["ip_emb_ffn"]["dense2_w"], w["ip_emb_ffn"]["dense2_b"] = fc(emb, emb_dff)
+        w["ip_emb_ffn_ln_gammas"], w["ip_emb_ffn_ln_betas"] = ln(emb)
+    else:
+        w["ip_emb_w"], w["ip_emb_b"] = fc(emb, 112 + 64)
+    if gating:
+        w["ip_mult_gate"] = 1.0 + g.normal((emb * 64,), 0.1)
+        w["ip_add_gate"] = g.normal((emb * 64,), 0.1)
     w["encoder"] = []
     for _ in range(layers):
         mha = {}
@@ -125,25 +143,45 @@ def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_s
         layer["ln2_gammas"], layer["ln2_betas"] = ln(emb)
         w["encoder"].append(layer)
     w["headcount"] = heads
-    w["ip_pol_w"], w["ip_pol_b"] = fc(policy_d, emb)
-    w["ip2_pol_w"], w["ip2_pol_b"] = fc(policy_d, policy_d)
-    w["ip3_pol_w"], w["ip3_pol_b"] = fc(policy_d, policy_d)
-    w["ip4_pol_w"] = fc(4, policy_d, bias=False)
-    w["ip_val_w"], w["ip_val_b"] = fc(value_channels, emb)
-    w["ip1_val_w"], w["ip1_val_b"] = fc(value_fc, 64 * value_channels)
-    w["ip2_val_w"], w["ip2_val_b"] = fc(3, value_fc)
+
+    def policy_head():
+        h = {}
+        h["ip2_pol_w"], h["ip2_pol_b"] = fc(policy_d, policy_d)
+        h["ip3_pol_w"], h["ip3_pol_b"] = fc(policy_d, policy_d)
+        h["ip4_pol_w"] = fc(4, policy_d, bias=False)
+        return h
+
+    def value_head():
+        h = {}
+        h["ip_val_w"], h["ip_val_b"] = fc(value_channels, emb)
+        h["ip1_val_w"], h["ip1_val_b"] = fc(value_fc, 64 * value_channels)
+        h["ip2_val_w"], h["ip2_val_b"] = fc(3, value_fc)
+        return h
+
+    if multihead:
+        ph = {}
+        ph["ip_pol_w"], ph["ip_pol_b"] = fc(policy_d, emb)
+        for name in ("vanilla", "optimistic_st", "soft"):
+            ph[name] = policy_head()
+        w["policy_heads"] = ph
+        w["value_heads"] = {name: value_head() for name in ("winner", "q", "st")}
+    else:
+        w["ip_pol_w"], w["ip_pol_b"] = fc(policy_d, emb)
+        w.update(policy_head())
+        w.update(value_head())
     w["ip_mov_w"], w["ip_mov_b"] = fc(mlh_channels, emb)
     w["ip1_mov_w"], w["ip1_mov_b"] = fc(mlh_fc, 64 * mlh_channels)
     w["ip2_mov_w"], w["ip2_mov_b"] = fc(1, mlh_fc)
     if smolgen:
         w["smolgen_w"] = fc(64 * 64, smolgen[2], bias=False)
     nf = {"input": INPUT_CLASSICAL_112_PLANE, "output": OUTPUT_WDL,
-          "network": NETWORK_ATTENTIONBODY_WITH_HEADFORMAT, "policy": POLICY_ATTENTION,
+          "network": NETWORK_ATTENTIONBODY_WITH_MULTIHEADFORMAT if multihead else NETWORK_ATTENTIONBODY_WITH_HEADFORMAT,
+          "policy": POLICY_ATTENTION,
           "value": VALUE_WDL, "moves_left": MOVES_LEFT_V1,
           "default_activation": DEFAULT_ACTIVATION_MISH,
           "smolgen_activation": ACTIVATION_SWISH if smolgen else ACTIVATION_DEFAULT,
           "ffn_activation": ACTIVATION_DEFAULT,
-          "input_embedding": INPUT_EMBEDDING_PE_MAP}
+          "input_embedding": INPUT_EMBEDDING_PE_DENSE if pe_dense else INPUT_EMBEDDING_PE_MAP}
     return {"format": {"weights_encoding": netproto.LINEAR16, "network_format": nf}, "weights": w}
 
 
@@ -161,11 +199,23 @@ CONFIGS = {
     "tiny_resnet": lambda: se_resnet(32, 2, 8, seed=2000, moves_left=True),
     "tiny_resnet_convpolicy": lambda: se_resnet(32, 2, 8, seed=2003, conv_policy=True),
     "tiny_resnet_nose": lambda: se_resnet(24, 3, 0, seed=2004, moves_left=True),
-    "tiny_attn": lambda: attention_body(64, 2, 2, 96, seed=2001, smolgen=(8, 32, 32), perturb_ln=True),
+    # (std 0.1 instead of 0.02: at width 64 that gives policy logits of order 0.1-1, so absolute
+    # tolerances in the parity tests mean something)
+    "tiny_attn": lambda: attention_body(64, 2, 2, 96, seed=2001, smolgen=(8, 32, 32), perturb_ln=True, std=0.1),
     # smallest shape the fp8 configuration accepts (all widths multiples of 128)
-    "tiny_attn_f8": lambda: attention_body(128, 3, 4, 256, seed=2005, smolgen=(8, 32, 32), perturb_ln=True),
-    "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True),
+    "tiny_attn_f8": lambda: attention_body(128, 3, 4, 256, seed=2005, smolgen=(8, 32, 32), perturb_ln=True, std=0.07),
+    # modern format: dense position encoding + embedding FFN, input gating, multi-head format
+    "tiny_attn_dense": lambda: attention_body(64, 2, 2, 96, seed=2006, smolgen=(8, 32, 32), perturb_ln=True,
+                                              pe_dense=(16, 128), gating=True, multihead=True, std=0.1),
+    # BT4 as published: 15 layers, d=1024, 32 heads, dff 1536, smolgen, PE_DENSE (64 channels, FFN 1536), multi-head
+    "bt4_dense_15x1024": lambda: attention_body(1024, 15, 32, 1536, seed=1004, smolgen=(32, 256, 256),
+                                                pe_dense=(64, 1536), multihead=True),
+    "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True, std=0.1),
 }
+
+
+# Part of the cache file name: bump when a generator or a configuration changes.
+CACHE_VERSION = "-g2"
 
 
 def write_config(name, path):
@@ -179,7 +229,7 @@ def cached_config(name, cache_dir=None):
     """Path of the generated file for `name`, generating it on first use."""
     cache_dir = cache_dir or os.environ.get("LC0MI_NET_CACHE", "/tmp/lc0mi_nets")
     os.makedirs(cache_dir, exist_ok=True)
-    path = os.path.join(cache_dir, name + ".pb.gz")
+    path = os.path.join(cache_dir, name + CACHE_VERSION + ".pb.gz")
     if not os.path.exists(path):
         tmp = path + ".tmp%d" % os.getpid()
         write_config(name, tmp)

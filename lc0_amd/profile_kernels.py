@@ -27,6 +27,9 @@ def main():
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--heads", type=int, default=32)
     ap.add_argument("--iters", type=int, default=5)
+    ap.add_argument("--data", choices=["random", "zeros", "const"], default="random",
+                    help="operand values for gemm / gemm_f8: the same instruction stream runs faster on "
+                         "constant operands (less switching power, higher sustained clock)")
     ap.add_argument("--variant", type=int, default=-1, help="force a GEMM tile variant (see kernels.set_gemm_variant)")
     args = ap.parse_args()
     if args.variant >= 0:
@@ -43,14 +46,20 @@ def main():
     elif args.kernel == "gemm":
         a = rng.standard_normal((args.m, args.k), dtype=np.float32).astype(np.float16)
         w = (rng.standard_normal((args.n, args.k), dtype=np.float32) * 0.02).astype(np.float16)
+        if args.data != "random":
+            a[:] = 0.0 if args.data == "zeros" else 1.0
+            w[:] = 0.0 if args.data == "zeros" else 0.125
         _, ms = K.gemm(a, w, np.zeros(args.n, np.float32), time_iters=args.iters)
-        print("gemm %dx%dx%d: %.1f us, %.0f TFLOP/s" % (args.m, args.n, args.k, ms * 1e3,
+        print("gemm (%s data) %dx%dx%d: %.1f us, %.0f TFLOP/s" % (args.data, args.m, args.n, args.k, ms * 1e3,
                                                        2.0 * args.m * args.n * args.k / (ms * 1e-3) / 1e12))
     elif args.kernel == "gemm_f8":
         a = rng.integers(0, 120, (args.m, args.k), dtype=np.uint8) | (rng.integers(0, 2, (args.m, args.k), dtype=np.uint8) << 7)
         w = rng.integers(0, 127, (args.n, args.k), dtype=np.uint8) | (rng.integers(0, 2, (args.n, args.k), dtype=np.uint8) << 7)
+        if args.data != "random":
+            a[:] = 0 if args.data == "zeros" else 0x38
+            w[:] = 0 if args.data == "zeros" else 0x30
         _, ms = K.gemm_f8(a, w, np.full(args.n, 1e-3, np.float32), np.zeros(args.n, np.float32), time_iters=args.iters)
-        print("gemm_f8 %dx%dx%d: %.1f us, %.0f TFLOP/s" % (args.m, args.n, args.k, ms * 1e3,
+        print("gemm_f8 (%s data) %dx%dx%d: %.1f us, %.0f TFLOP/s" % (args.data, args.m, args.n, args.k, ms * 1e3,
                                                           2.0 * args.m * args.n * args.k / (ms * 1e-3) / 1e12))
     elif args.kernel == "attention":
         d = args.heads * 32
