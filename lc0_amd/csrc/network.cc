@@ -14,6 +14,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <sstream>
 
@@ -343,6 +344,13 @@ class Mi355xNetwork : public Network {
   void *r_in_ = nullptr, *r_x_ = nullptr, *r_y_ = nullptr, *r_v_ = nullptr, *r_m_ = nullptr, *r_h1_ = nullptr,
        *r_h2_ = nullptr;
 
+  // Captured device passes, one per batch size (option graphs=true): replaying a graph
+  // costs one launch instead of several hundred, which is what bounds small batches.
+  bool use_graphs_ = true;
+  std::map<int, hipGraphExec_t> graphs_;
+  void DropGraphs();
+  void LaunchEager(int batch);
+
   // Profiling.
   bool profiling_ = false;
   struct Pending { std::string name; hipEvent_t start, stop; double flops, bytes; };
@@ -561,6 +569,7 @@ void Mi355xNetwork::CalibrateFp8(int n, const uint64_t* masks, const float* valu
     for (size_t i = 0; i < slots; i++) absmax[i] = std::max(absmax[i], part[i]);
   }
   ApplyCalibration(absmax);
+  DropGraphs();   // recorded kernel arguments hold the old scales
 }
 
 // Built-in calibration set used at load, so that precision=fp8 works without any caller
@@ -656,6 +665,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
       pos = end + 1;
     }
   }
+  use_graphs_ = options.GetBool("graphs", true);
   policy_head_ = options.GetString("policy_head", "vanilla");
   value_head_ = options.GetString("value_head", "winner");
   wdl_ = nf.value == kValueWdl;
@@ -714,6 +724,7 @@ Mi355xNetwork::~Mi355xNetwork() {
   }
   if (stream_) {
     (void)hipStreamSynchronize(stream_);
+    DropGraphs();
     for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
     for (hipEvent_t e : fork_events_) (void)hipEventDestroy(e);
     for (hipEvent_t e : join_events_) (void)hipEventDestroy(e);
@@ -1287,7 +1298,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
   });
 }
 
-void Mi355xNetwork::ForwardDevice(int batch) {
+void Mi355xNetwork::LaunchEager(int batch) {
   if (attn_body_) {
     ForwardAttentionBody(batch);
   } else if (fp32_) {
@@ -1295,6 +1306,49 @@ void Mi355xNetwork::ForwardDevice(int batch) {
   } else {
     ForwardResnet<half_t>(batch);
   }
+}
+
+void Mi355xNetwork::DropGraphs() {
+  for (auto& g : graphs_) (void)hipGraphExecDestroy(g.second);
+  graphs_.clear();
+}
+
+void Mi355xNetwork::ForwardDevice(int batch) {
+  constexpr size_t kMaxGraphs = 96;
+  if (!use_graphs_ || profiling_ || calibrating_) {
+    LaunchEager(batch);
+    return;
+  }
+  auto it = graphs_.find(batch);
+  if (it == graphs_.end()) {
+    if (graphs_.size() >= kMaxGraphs) {
+      LaunchEager(batch);
+      return;
+    }
+    // Record the launch sequence of this batch size once. All buffers are allocated at
+    // construction and kernel arguments depend only on the batch size, so the recorded
+    // graph stays valid (calibration, which changes fp8 scales, drops the graphs).
+    hipGraph_t graph = nullptr;
+    HIP_CHECK(hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal));
+    try {
+      LaunchEager(batch);
+    } catch (...) {
+      (void)hipStreamEndCapture(stream_, &graph);
+      if (graph) (void)hipGraphDestroy(graph);
+      use_graphs_ = false;
+      throw;
+    }
+    HIP_CHECK(hipStreamEndCapture(stream_, &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t err = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (err != hipSuccess) {
+      use_graphs_ = false;
+      throw Error(std::string("HIP error: ") + hipGetErrorString(err) + " (hipGraphInstantiate)");
+    }
+    it = graphs_.emplace(batch, exec).first;
+  }
+  HIP_CHECK(hipGraphLaunch(it->second, stream_));
 }
 
 void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {

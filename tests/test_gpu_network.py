@@ -326,3 +326,36 @@ def test_bt4_dense_multihead_batch_256(positions):
     full = comp.results()
     assert np.isfinite(full["policy"]).all()
     np.testing.assert_allclose(full["policy"][:32], res32["policy"], rtol=0, atol=5e-3)
+
+
+@pytest.mark.parametrize("name,options", [("tiny_attn", ""), ("tiny_attn_f8", "precision=fp8"), ("tiny_resnet", "")])
+def test_graph_replays_equal_eager_launches(name, options, positions):
+    """The device pass is recorded once per batch size and replayed; every replay, with other
+    batch sizes and eager work of a second network in between, must give exactly what plain
+    launches give (same kernels, same arguments: bitwise)."""
+    from lc0_amd import Network
+    path = netgen.cached_config(name)
+    sep = "," if options else ""
+    replay = Network(path, options + sep + "graphs=true")
+    eager = Network(path, options + sep + "graphs=false")
+    rng = np.random.default_rng(5)
+    for n in (5, 17, 5, 40, 17, 5, 1, 40, 1):
+        idx = rng.permutation(320)[:n]
+        outs = []
+        for net in (replay, eager):
+            comp = net.NewComputation()
+            comp.AddInputs(positions["masks"][idx], positions["values"][idx])
+            comp.ComputeBlocking()
+            outs.append(comp.results())
+        for key in ("policy", "q", "d", "m"):
+            np.testing.assert_array_equal(outs[0][key], outs[1][key])
+    if options:   # re-calibration drops the recorded graphs: the next replay must use the new scales
+        for net in (replay, eager):
+            net.CalibrateFp8(positions["masks"][100:164], positions["values"][100:164])
+        outs = []
+        for net in (replay, eager):
+            comp = net.NewComputation()
+            comp.AddInputs(positions["masks"][:5], positions["values"][:5])
+            comp.ComputeBlocking()
+            outs.append(comp.results())
+        np.testing.assert_array_equal(outs[0]["policy"], outs[1]["policy"])
