@@ -322,12 +322,15 @@ void WinogradConvHost(const float* x, const float* filter, const float* bias, co
   float *w1 = nullptr, *b1 = nullptr, *w2 = nullptr, *b2 = nullptr;
   if (se_k > 0) {
     w1 = dev.Put(se_w1, (size_t)se_k * cout); b1 = dev.Put(se_b1, (size_t)se_k);
-    w2 = dev.Put(se_w2, (size_t)2 * cout * se_k); b2 = dev.Put(se_b2, (size_t)2 * cout);
+    std::vector<float> w2t((size_t)2 * cout * se_k);   // [2C][K] -> [K][2C], the layout the kernels read
+    for (int o = 0; o < 2 * cout; o++)
+      for (int k = 0; k < se_k; k++) w2t[(size_t)k * 2 * cout + o] = se_w2[(size_t)o * se_k + k];
+    w2 = dev.Put(w2t.data(), w2t.size()); b2 = dev.Put(se_b2, (size_t)2 * cout);
   }
   const int tiles = batch * 4;
   T* dv = static_cast<T*>(dev.Alloc(sizeof(T) * 36 * tiles * ld));
   K_CHECK(hipMemset(dv, 0, sizeof(T) * 36 * tiles * ld));
-  float* dm = static_cast<float*>(dev.Alloc(sizeof(float) * 36 * tiles * cout));
+  T* dm = static_cast<T*>(dev.Alloc(sizeof(T) * 36 * tiles * cout));   // winograd-domain products, in the tower's type
   T* dout = static_cast<T*>(dev.Alloc(sizeof(T) * no));
   lc0mi::LaunchWinogradInputTransform<T>(dx, dv, batch, cin, ld, nullptr);
   if constexpr (sizeof(T) == 2) {
@@ -335,7 +338,7 @@ void WinogradConvHost(const float* x, const float* filter, const float* bias, co
     g.A = dv; g.lda = ld; g.strideA = (long long)tiles * ld;
     g.W = du; g.ldw = ld; g.strideW = (long long)cout * ld;
     g.C = dm; g.ldc = cout; g.strideC = (long long)tiles * cout;
-    g.M = tiles; g.N = cout; g.K = ld; g.batch = 36; g.out_f32 = true;
+    g.M = tiles; g.N = cout; g.K = ld; g.batch = 36; g.out_f32 = false;
     lc0mi::LaunchGemm(g, nullptr);
   } else {
     lc0mi::GemmArgsF32 g;
@@ -345,7 +348,7 @@ void WinogradConvHost(const float* x, const float* filter, const float* bias, co
     g.M = tiles; g.N = cout; g.K = ld; g.batch = 36;
     lc0mi::LaunchGemmF32(g, nullptr);
   }
-  lc0mi::LaunchWinogradOutputTransform<T, float>(dm, dbias, dskip, w1, b1, w2, b2, se_k, dout, batch, cout, act, nullptr);
+  lc0mi::LaunchWinogradOutputTransform<T, T>(dm, dbias, dskip, w1, b1, w2, b2, se_k, dout, batch, cout, act, nullptr);
   K_CHECK(hipDeviceSynchronize());
   K_CHECK(hipGetLastError());
   std::vector<T> ho(no);

@@ -162,7 +162,7 @@ void LaunchWinogradInputTransform(const T* x, T* v, int batch, int C, int ldv, h
 //           gamma = sigmoid(s[0:C]); beta = s[C:2C] + gamma * bias;
 //           out = act(gamma * y + skip + beta)
 // m: [36][B*4][C] (M_IS_F32 selects float m for T = half_t), out/skip: [B][64][C].
-// se_w1: [K][C], se_w2: [2C][K] floats. C <= 1024, K <= 256.
+// se_w1: [K][C], se_w2: [K][2C] floats (the transpose of lc0's [2C][K]). C <= 1024, K <= 256.
 template <typename T, typename MT>
 void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip, const float* se_w1,
                                    const float* se_b1, const float* se_w2, const float* se_b2, int se_k, T* out,

@@ -285,7 +285,13 @@ __device__ __forceinline__ unsigned PackFp8x4(float a, float b, float c, float d
 // GemmF8Args: 128 bytes = 128 values per row, v_mfma_f32_32x32x64_f8f6f4);
 // BKB is the k-tile in bytes. OutT is half_t or uint8_t (e4m3, fp8 operands only).
 template <int BM, int BN, int BKB, int WAVES_M, int WAVES_N, typename Args, typename OutT>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(Args p) {
+// Second launch bound = waves per SIMD: with small wave tiles two workgroups share a CU
+// (4 waves per SIMD, at most 128 VGPRs) and overlap each other's prologue and epilogue.
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
+                             ((BM / WAVES_M / 32) * (BN / WAVES_N / 32) <= 4 && 4 * (BM + BN) * BKB <= 160 * 1024)
+                                 ? WAVES_M * WAVES_N / 2
+                                 : WAVES_M * WAVES_N / 4)
+void gemm_dma_kernel(Args p) {
   constexpr bool F8 = std::is_same<Args, GemmF8Args>::value;
   constexpr int ES = F8 ? 1 : 2;                  // bytes per operand element
   constexpr int NWAVES = WAVES_M * WAVES_N;

@@ -1020,7 +1020,14 @@ void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
         throw Error("SE unit weights have an unexpected size.");
       }
       b.se.w1 = arena_.Upload(r.se.w1); b.se.b1 = arena_.Upload(r.se.b1);
-      b.se.w2 = arena_.Upload(r.se.w2); b.se.b2 = arena_.Upload(r.se.b2);
+      {
+        // [2C][K] -> [K][2C], so that threads of neighbouring channels read neighbouring addresses.
+        Vec w2t(r.se.w2.size());
+        for (int o = 0; o < 2 * filters_; o++)
+          for (int k = 0; k < b.se.k; k++) w2t[static_cast<size_t>(k) * 2 * filters_ + o] = r.se.w2[static_cast<size_t>(o) * b.se.k + k];
+        b.se.w2 = arena_.Upload(w2t);
+      }
+      b.se.b2 = arena_.Upload(r.se.b2);
     }
     res_blocks_.push_back(b);
   }
@@ -1094,17 +1101,17 @@ void Mi355xNetwork::WinogradConv(const char* name, const ConvDev& conv, const vo
   Timed("winograd_input_transform", 0.0, sizeof(T) * B * (64.0 + 144.0) * conv.cin, [&] {
     LaunchWinogradInputTransform<T>(static_cast<const T*>(x), static_cast<T*>(r_v_), B, conv.cin, conv.ld, stream_);
   });
-  // Winograd-domain products are kept in float when the tower runs in fp16: the output
-  // transform sums 36 of them with weights up to 64.
-  constexpr bool kHalf = sizeof(T) == 2;
+  // Winograd-domain products M in the tower's own type (half products are accurate enough
+  // because the transform matrices are row-balanced; float M would double the traffic of
+  // both the GEMM epilogue and the output transform).
   GemmT<T>(name, r_v_, conv.ld, static_cast<long long>(tiles) * conv.ld, conv.u, conv.ld,
            static_cast<long long>(conv.cout) * conv.ld, r_m_, conv.cout, static_cast<long long>(tiles) * conv.cout,
-           nullptr, tiles, conv.cout, conv.ld, 36, kActNone, /*out_f32=*/kHalf);
-  Timed("winograd_output_transform", 0.0, B * conv.cout * (144.0 * 4 + sizeof(T) * 64.0 * (skip ? 2 : 1)), [&] {
-    LaunchWinogradOutputTransform<T, float>(static_cast<const float*>(r_m_), conv.bias, static_cast<const T*>(skip),
-                                            se ? se->w1 : nullptr, se ? se->b1 : nullptr, se ? se->w2 : nullptr,
-                                            se ? se->b2 : nullptr, se ? se->k : 0, static_cast<T*>(out), B, conv.cout,
-                                            act, stream_);
+           nullptr, tiles, conv.cout, conv.ld, 36, kActNone, /*out_f32=*/false);
+  Timed("winograd_output_transform", 0.0, B * conv.cout * sizeof(T) * (144.0 + 64.0 * (skip ? 2 : 1)), [&] {
+    LaunchWinogradOutputTransform<T, T>(static_cast<const T*>(r_m_), conv.bias, static_cast<const T*>(skip),
+                                        se ? se->w1 : nullptr, se ? se->b1 : nullptr, se ? se->w2 : nullptr,
+                                        se ? se->b2 : nullptr, se ? se->k : 0, static_cast<T*>(out), B, conv.cout,
+                                        act, stream_);
   });
 }
 

@@ -160,11 +160,9 @@ __global__ void winograd_output_transform_kernel(const MT* __restrict__ m, const
     }
     __syncthreads();
     float sg = se_b2[c], sb = se_b2[C + c];
-    const float* wg = se_w2 + (long long)c * se_k;
-    const float* wb = se_w2 + (long long)(C + c) * se_k;
-    for (int k = 0; k < se_k; k++) {
-      sg += wg[k] * hidden[k];
-      sb += wb[k] * hidden[k];
+    for (int k = 0; k < se_k; k++) {   // se_w2 is stored [K][2C]: neighbouring channels, neighbouring addresses
+      sg += se_w2[(long long)k * 2 * C + c] * hidden[k];
+      sb += se_w2[(long long)k * 2 * C + C + c] * hidden[k];
     }
     gamma = 1.0f / (1.0f + __expf(-sg));
     beta = sb + gamma * bc;
@@ -177,6 +175,90 @@ __global__ void winograd_output_transform_kernel(const MT* __restrict__ m, const
     if (sk) v += (float)sk[(long long)sq * C];
     o[(long long)sq * C] = (T)RActivate(v, act);
   }
+}
+
+// Same for C <= 256 with four times the parallelism: one thread per (tile, channel),
+// blockDim.x == 4 * C. Shared memory: part[4][C] | hidden[K] | gate[2][C] floats.
+template <typename T, typename MT>
+__global__ __launch_bounds__(1024) void winograd_output_transform_tiles_kernel(
+    const MT* __restrict__ m, const float* __restrict__ bias, const T* skip, const float* __restrict__ se_w1,
+    const float* __restrict__ se_b1, const float* __restrict__ se_w2, const float* __restrict__ se_b2, int se_k,
+    T* out, int batch, int C, int act) {
+  extern __shared__ float shm[];
+  float* part = shm;               // [4][C], then pool[C] in its first row
+  float* hidden = shm + 4 * C;     // [K]
+  float* gate = hidden + se_k;     // gamma[C] | beta[C]
+  const int b = blockIdx.x;
+  const int tile = threadIdx.x / C, c = threadIdx.x - tile * C;
+  const long long kstride = (long long)batch * 4 * C;
+  const MT* mp = m + (long long)(b * 4 + tile) * C + c;
+  float mm[36];
+#pragma unroll
+  for (int k = 0; k < 36; k++) mm[k] = (float)mp[(long long)k * kstride];
+  float s[4][6];
+#pragma unroll
+  for (int j = 0; j < 6; j++) {
+    const float m0 = mm[j], m1 = mm[6 + j], m2 = mm[12 + j], m3 = mm[18 + j], m4 = mm[24 + j], m5 = mm[30 + j];
+    s[0][j] = m0 + m1 + m2 + m3 + m4;
+    s[1][j] = m1 - m2 + 2.0f * (m3 - m4);
+    s[2][j] = m1 + m2 + 4.0f * (m3 + m4);
+    s[3][j] = m1 - m2 + 8.0f * (m3 - m4) + m5;
+  }
+  float y[4][4];
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const float s0 = s[i][0], s1 = s[i][1], s2 = s[i][2], s3 = s[i][3], s4 = s[i][4], s5 = s[i][5];
+    y[i][0] = s0 + s1 + s2 + s3 + s4;
+    y[i][1] = s1 - s2 + 2.0f * (s3 - s4);
+    y[i][2] = s1 + s2 + 4.0f * (s3 + s4);
+    y[i][3] = s1 - s2 + 8.0f * (s3 - s4) + s5;
+    sum += y[i][0] + y[i][1] + y[i][2] + y[i][3];
+  }
+  const float bc = bias[c];
+  float gamma = 1.0f, beta = bc;
+  if (se_k > 0) {
+    part[tile * C + c] = sum;
+    __syncthreads();
+    if (tile == 0) part[c] = (part[c] + part[C + c] + part[2 * C + c] + part[3 * C + c]) * (1.0f / 64.0f) + bc;
+    __syncthreads();
+    // hidden[k] = act(w1[k] . pool + b1[k]): one wave per k, lanes stride over the channels.
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    for (int k = wave; k < se_k; k += nwaves) {
+      const float* w = se_w1 + (long long)k * C;
+      float h = 0.0f;
+      for (int i = lane; i < C; i += 64) h += w[i] * part[i];
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) h += __shfl_xor(h, off, 64);
+      if (lane == 0) hidden[k] = RActivate(h + se_b1[k], act);
+    }
+    __syncthreads();
+    if (tile == 0) {
+      float sg = se_b2[c], sb = se_b2[C + c];
+      for (int k = 0; k < se_k; k++) {
+        sg += se_w2[(long long)k * 2 * C + c] * hidden[k];
+        sb += se_w2[(long long)k * 2 * C + C + c] * hidden[k];
+      }
+      const float gm = 1.0f / (1.0f + __expf(-sg));
+      gate[c] = gm;
+      gate[C + c] = sb + gm * bc;
+    }
+    __syncthreads();
+    gamma = gate[c];
+    beta = gate[C + c];
+  }
+  const int ty = (tile >> 1) * 4, tx = (tile & 1) * 4;
+  const T* sk = skip ? skip + (long long)b * 64 * C + c : nullptr;
+  T* o = out + (long long)b * 64 * C + c;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int sq = (ty + i) * 8 + tx + j;
+      float v = gamma * y[i][j] + beta;
+      if (sk) v += (float)sk[(long long)sq * C];
+      o[(long long)sq * C] = (T)RActivate(v, act);
+    }
 }
 
 template <typename T>
@@ -232,7 +314,14 @@ void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip
                                    const float* se_b1, const float* se_w2, const float* se_b2, int se_k, T* out,
                                    int batch, int C, int act, hipStream_t stream) {
   if (batch <= 0) return;
-  const size_t shm = sizeof(float) * (size_t)(C + (se_k > 0 ? se_k : 0));
+  const int k = se_k > 0 ? se_k : 0;
+  if (C <= 256) {
+    const size_t shm = sizeof(float) * (size_t)(6 * C + k);
+    hipLaunchKernelGGL((winograd_output_transform_tiles_kernel<T, MT>), dim3(batch), dim3(4 * C), shm, stream, m, bias,
+                       skip, se_w1, se_b1, se_w2, se_b2, se_k, out, batch, C, act);
+    return;
+  }
+  const size_t shm = sizeof(float) * (size_t)(C + k);
   hipLaunchKernelGGL((winograd_output_transform_kernel<T, MT>), dim3(batch), dim3(C), shm, stream, m, bias, skip,
                      se_w1, se_b1, se_w2, se_b2, se_k, out, batch, C, act);
 }

@@ -26,6 +26,7 @@ def main():
     ap.add_argument("--k", type=int, default=1024)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--heads", type=int, default=32)
+    ap.add_argument("--gemm-batch", type=int, default=1, help="independent GEMMs in one launch (gemm only)")
     ap.add_argument("--iters", type=int, default=5)
     ap.add_argument("--data", choices=["random", "zeros", "const"], default="random",
                     help="operand values for gemm / gemm_f8: the same instruction stream runs faster on "
@@ -44,14 +45,15 @@ def main():
         print("copy %d MiB: %.1f us per launch, %.0f GB/s (read+write)" % (args.mib, ms.value * 1e3,
                                                                           2 * nbytes / (ms.value * 1e-3) / 1e9))
     elif args.kernel == "gemm":
-        a = rng.standard_normal((args.m, args.k), dtype=np.float32).astype(np.float16)
-        w = (rng.standard_normal((args.n, args.k), dtype=np.float32) * 0.02).astype(np.float16)
+        nb = args.gemm_batch
+        a = rng.standard_normal((nb, args.m, args.k), dtype=np.float32).astype(np.float16)
+        w = (rng.standard_normal((nb, args.n, args.k), dtype=np.float32) * 0.02).astype(np.float16)
         if args.data != "random":
             a[:] = 0.0 if args.data == "zeros" else 1.0
             w[:] = 0.0 if args.data == "zeros" else 0.125
         _, ms = K.gemm(a, w, np.zeros(args.n, np.float32), time_iters=args.iters)
-        print("gemm (%s data) %dx%dx%d: %.1f us, %.0f TFLOP/s" % (args.data, args.m, args.n, args.k, ms * 1e3,
-                                                       2.0 * args.m * args.n * args.k / (ms * 1e-3) / 1e12))
+        print("gemm (%s data) %d x %dx%dx%d: %.1f us, %.0f TFLOP/s" % (
+            args.data, nb, args.m, args.n, args.k, ms * 1e3, 2.0 * nb * args.m * args.n * args.k / (ms * 1e-3) / 1e12))
     elif args.kernel == "gemm_f8":
         a = rng.integers(0, 120, (args.m, args.k), dtype=np.uint8) | (rng.integers(0, 2, (args.m, args.k), dtype=np.uint8) << 7)
         w = rng.integers(0, 127, (args.n, args.k), dtype=np.uint8) | (rng.integers(0, 2, (args.n, args.k), dtype=np.uint8) << 7)

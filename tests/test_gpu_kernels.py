@@ -200,8 +200,15 @@ def test_winograd_conv_vs_oracle(batch, cin, cout, se_k, with_skip, fp16):
         want = onn.activate(t, nr.ACT_RELU)
     got = K.winograd_conv(x.reshape(batch, cin, 64).transpose(0, 2, 1), filt, bias,
                           skip.transpose(0, 2, 1) if with_skip else None, se, act=nr.ACT_RELU, fp16=fp16)
-    tol = 2e-2 if fp16 else 2e-4   # fp16: transformed operands are rounded to 11 bits
-    np.testing.assert_allclose(got.transpose(0, 2, 1), want, rtol=tol, atol=tol)
+    got = got.transpose(0, 2, 1)
+    if fp16:
+        # Transformed inputs, filters and the winograd-domain products are all rounded to 11 bits, and
+        # the inverse transform A^T (entries up to 8, i.e. 64 in two dimensions) amplifies the rounding of
+        # the products: a few per cent of the output scale at the corner outputs of a tile, ~0.3 % rms.
+        np.testing.assert_allclose(got, want, rtol=5e-2, atol=5e-2)
+        assert np.sqrt(np.mean((got - want) ** 2)) <= 6e-3 * max(1.0, float(np.abs(want).max()))
+    else:
+        np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
 
 
 def test_expand_planes_nhwc_bit_exact():
