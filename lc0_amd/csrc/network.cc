@@ -12,7 +12,9 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
+#include <condition_variable>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -220,9 +222,60 @@ class Mi355xComputation : public NetworkComputation {
   bool computed_ = false;
 };
 
-class Mi355xNetwork : public Network {
+// Everything that describes the loaded network and is the same for every lane: options,
+// dimensions and device weights (pointers into the arena of the network that loaded them).
+struct ModelState {
+  NetworkCapabilities caps_;
+  int device_ = 0;
+  int max_batch_ = 1024;
+  bool wdl_ = false, moves_left_ = false, attn_body_ = false, attn_policy_ = false, conv_policy_ = false;
+  int default_act_ = kActRelu, smolgen_act_ = kActNone, ffn_act_ = kActNone;
+  std::string policy_head_, value_head_;
+  bool use_graphs_ = true;
+
+  // Attention body dimensions.
+  int emb_ = 0, d_model_ = 0, heads_ = 0, dff_ = 0, in_ld_ = 192;
+  int sg_hc_ = 0, sg_hs_ = 0, sg_gen_ = 0;
+  int pol_emb_ = 0, pol_d_ = 0, val_ch_ = 0, val_fc_ = 0, val_out_ = 0, mov_ch_ = 0, mov_fc_ = 0;
+  float alpha_ = 1.0f, eps_ = 1e-6f;
+  bool any_smolgen_ = false;
+  // Dense position encoding (PE_DENSE nets): preprocessing layer, embedding layer norm and
+  // embedding FFN; optional input gating.
+  bool pe_dense_ = false, gating_ = false;
+  int enc_ch_ = 0, emb_dff_ = 0;
+  Linear preproc_lin_, emb_ffn1_, emb_ffn2_;
+  float *emb_ln_g_ = nullptr, *emb_ln_b_ = nullptr, *emb_ffn_ln_g_ = nullptr, *emb_ffn_ln_b_ = nullptr;
+  float *gate_mult_ = nullptr, *gate_add_ = nullptr;   // [64][emb]
+
+  // Device weights.
+  Linear emb_lin_, smolgen_w_, pol_emb_lin_, pol_qk_lin_, val_emb_lin_, val_fc1_, val_fc2_, mov_emb_lin_, mov_fc1_,
+      mov_fc2_;
+  std::vector<EncoderDev> encoders_;
+  half_t* pos_enc_ = nullptr;
+  float* ppo_ = nullptr;
+  int16_t* inv_map_ = nullptr;
+
+  // fp8 configuration: the four large GEMMs of every encoder layer run on e4m3 operands.
+  bool fp8_ = false;
+  bool q_qkv_ = true, q_dense_ = true, q_ffn1_ = true, q_ffn2_ = true;   // option fp8_gemms
+
+  // Residual tower.
+  bool fp32_ = false;
+  int filters_ = 0;
+  bool classical_value_ = false;
+  ConvDev res_input_, res_policy1_, res_policy_conv_;
+  std::vector<ResBlockDev> res_blocks_;
+  LinearT res_pol_conv1x1_, res_pol_fc_, res_val_conv_, res_val_fc1_, res_val_fc2_, res_mov_conv_, res_mov_fc1_,
+      res_mov_fc2_;
+  int16_t* conv_inv_map_ = nullptr;
+  size_t res_max_fc_ = 0, res_cmax_ = 0;
+};
+
+class Mi355xNetwork : public Network, protected ModelState {
  public:
+  struct LaneTag {};
   Mi355xNetwork(const WeightsFile& file, Options& options);
+  Mi355xNetwork(const Mi355xNetwork& parent, LaneTag);   // one more lane on the parent's weights
   ~Mi355xNetwork() override;
 
   const NetworkCapabilities& GetCapabilities() const override { return caps_; }
@@ -269,6 +322,7 @@ class Mi355xNetwork : public Network {
               bool out_f8, float out_mul);
   void RecordAbsMax(const half_t* x, size_t n, int slot);
   void ApplyCalibration(const std::vector<float>& absmax);
+  void CalibrateExclusive(int n, const uint64_t* masks, const float* values);
   void DefaultCalibration();
   float* UploadF(const Vec& v) { return arena_.Upload(v); }
   half_t* AllocH(size_t n) { return static_cast<half_t*>(arena_.Alloc(n * sizeof(half_t))); }
@@ -280,41 +334,13 @@ class Mi355xNetwork : public Network {
   void Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act,
             bool out_f32 = false, hipStream_t st = nullptr, int split_k = 1);
 
-  NetworkCapabilities caps_;
-  int device_ = 0;
-  int max_batch_ = 1024;
-  bool wdl_ = false, moves_left_ = false, attn_body_ = false, attn_policy_ = false, conv_policy_ = false;
-  int default_act_ = kActRelu, smolgen_act_ = kActNone, ffn_act_ = kActNone;
-  std::string policy_head_, value_head_;
+  // ---- per-lane state: streams, activations, recorded graphs ----
   hipStream_t stream_ = nullptr;
   hipStream_t side_stream_ = nullptr;  // smolgen chain, overlapped with the QKV projection
   std::vector<hipEvent_t> fork_events_, join_events_;
   DeviceArena arena_;
   std::mutex eval_mutex_;
   std::shared_ptr<SlotPool> pool_ = std::make_shared<SlotPool>();
-
-  // Attention body dimensions.
-  int emb_ = 0, d_model_ = 0, heads_ = 0, dff_ = 0, in_ld_ = 192;
-  int sg_hc_ = 0, sg_hs_ = 0, sg_gen_ = 0;
-  int pol_emb_ = 0, pol_d_ = 0, val_ch_ = 0, val_fc_ = 0, val_out_ = 0, mov_ch_ = 0, mov_fc_ = 0;
-  float alpha_ = 1.0f, eps_ = 1e-6f;
-  bool any_smolgen_ = false;
-  // Dense position encoding (PE_DENSE nets): preprocessing layer, embedding layer norm and
-  // embedding FFN; optional input gating.
-  bool pe_dense_ = false, gating_ = false;
-  int enc_ch_ = 0, emb_dff_ = 0;
-  Linear preproc_lin_, emb_ffn1_, emb_ffn2_;
-  float *emb_ln_g_ = nullptr, *emb_ln_b_ = nullptr, *emb_ffn_ln_g_ = nullptr, *emb_ffn_ln_b_ = nullptr;
-  float *gate_mult_ = nullptr, *gate_add_ = nullptr;   // [64][emb]
-  half_t *pre_in_ = nullptr, *pre_out_ = nullptr;
-
-  // Device weights.
-  Linear emb_lin_, smolgen_w_, pol_emb_lin_, pol_qk_lin_, val_emb_lin_, val_fc1_, val_fc2_, mov_emb_lin_, mov_fc1_,
-      mov_fc2_;
-  std::vector<EncoderDev> encoders_;
-  half_t* pos_enc_ = nullptr;
-  float* ppo_ = nullptr;
-  int16_t* inv_map_ = nullptr;
 
   // Device activations (sized for max_batch_).
   uint64_t* d_masks_ = nullptr;
@@ -324,35 +350,38 @@ class Mi355xNetwork : public Network {
   float* sg2f_ = nullptr;  // split-K accumulator of smolgen dense1
   half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
   float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
-
-  // fp8 configuration: the four large GEMMs of every encoder layer run on e4m3 operands.
-  bool fp8_ = false;
-  bool q_qkv_ = true, q_dense_ = true, q_ffn1_ = true, q_ffn2_ = true;   // option fp8_gemms
+  half_t *pre_in_ = nullptr, *pre_out_ = nullptr;
   bool calibrating_ = false;
   float* d_absmax_ = nullptr;   // [4 * layers + 1] calibration maxima (float bits, non-negative)
   uint8_t *xq_ = nullptr, *attq_ = nullptr, *ffnq_ = nullptr;
-
-  // Residual tower.
-  bool fp32_ = false;
-  int filters_ = 0;
-  bool classical_value_ = false;
-  ConvDev res_input_, res_policy1_, res_policy_conv_;
-  std::vector<ResBlockDev> res_blocks_;
-  LinearT res_pol_conv1x1_, res_pol_fc_, res_val_conv_, res_val_fc1_, res_val_fc2_, res_mov_conv_, res_mov_fc1_,
-      res_mov_fc2_;
-  int16_t* conv_inv_map_ = nullptr;
   void *r_in_ = nullptr, *r_x_ = nullptr, *r_y_ = nullptr, *r_v_ = nullptr, *r_m_ = nullptr, *r_h1_ = nullptr,
        *r_h2_ = nullptr;
 
+  // Lanes: further instances that share this network's weights and own their streams and
+  // activations, so that computations of several search threads run concurrently on the GPU
+  // (option lanes=N; precedent: multi_stream in src/neural/backends/cuda/network_cuda.cc:634-706).
+  std::vector<std::unique_ptr<Mi355xNetwork>> extra_lanes_;
+  std::mutex lane_mutex_;
+  std::condition_variable lane_cv_;
+  std::vector<Mi355xNetwork*> free_lanes_;
+  int lane_count_ = 1;
+  bool is_lane_ = false;
+  Mi355xNetwork* AcquireLane();
+  void ReleaseLane(Mi355xNetwork* lane);
+  void AcquireAllLanes();
+  void ReleaseAllLanes();
+  void EvaluateOnLane(HostSlot* slot, int batch);
+  void CreateStreams();
+  void AllocActivations();
+
   // Captured device passes, one per batch size (option graphs=true): replaying a graph
   // costs one launch instead of several hundred, which is what bounds small batches.
-  bool use_graphs_ = true;
   std::map<int, hipGraphExec_t> graphs_;
   void DropGraphs();
   void LaunchEager(int batch);
 
   // Profiling.
-  bool profiling_ = false;
+  std::atomic<bool> profiling_{false};   // read without the lane's mutex when a computation picks its lane
   struct Pending { std::string name; hipEvent_t start, stop; double flops, bytes; };
   std::vector<Pending> pending_;
   std::vector<hipEvent_t> event_pool_;
@@ -541,6 +570,18 @@ void Mi355xNetwork::ApplyCalibration(const std::vector<float>& absmax) {
 void Mi355xNetwork::CalibrateFp8(int n, const uint64_t* masks, const float* values) {
   if (!fp8_) throw Error("CalibrateFp8 needs a network created with precision=fp8.");
   if (n < 1 || !masks || !values) throw Error("CalibrateFp8 needs at least one position.");
+  AcquireAllLanes();
+  try {
+    CalibrateExclusive(n, masks, values);
+  } catch (...) {
+    ReleaseAllLanes();
+    throw;
+  }
+  ReleaseAllLanes();
+}
+
+// Caller guarantees that no computation is in flight on any lane.
+void Mi355xNetwork::CalibrateExclusive(int n, const uint64_t* masks, const float* values) {
   std::lock_guard<std::mutex> lock(eval_mutex_);
   HIP_CHECK(hipSetDevice(device_));
   const size_t slots = 4 * encoders_.size() + 1;
@@ -553,7 +594,7 @@ void Mi355xNetwork::CalibrateFp8(int n, const uint64_t* masks, const float* valu
                         hipMemcpyHostToDevice));
     LaunchZero(d_absmax_, static_cast<long long>(slots), stream_);
     calibrating_ = true;
-    const bool was_profiling = profiling_;
+    const bool was_profiling = profiling_.load();
     profiling_ = false;
     try {
       ForwardAttentionBody(b);   // fp16 pass that records the maxima
@@ -570,6 +611,10 @@ void Mi355xNetwork::CalibrateFp8(int n, const uint64_t* masks, const float* valu
   }
   ApplyCalibration(absmax);
   DropGraphs();   // recorded kernel arguments hold the old scales
+  for (auto& lane : extra_lanes_) {
+    static_cast<ModelState&>(*lane) = static_cast<const ModelState&>(*this);
+    lane->DropGraphs();
+  }
 }
 
 // Built-in calibration set used at load, so that precision=fp8 works without any caller
@@ -630,7 +675,7 @@ void Mi355xNetwork::DefaultCalibration() {
     m[110] = 0;
     m[111] = ~0ULL;                                                     // all ones
   }
-  CalibrateFp8(n, masks.data(), values.data());
+  CalibrateExclusive(n, masks.data(), values.data());
 }
 
 // ------------------------------------------------------------- construction --
@@ -666,6 +711,8 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
     }
   }
   use_graphs_ = options.GetBool("graphs", true);
+  lane_count_ = options.GetInt("lanes", 4);
+  if (lane_count_ < 1 || lane_count_ > 8) throw Error("lanes must be in 1..8.");
   policy_head_ = options.GetString("policy_head", "vanilla");
   value_head_ = options.GetString("value_head", "winner");
   wdl_ = nf.value == kValueWdl;
@@ -692,20 +739,10 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
     throw Error("No HIP device is available: the mi355x backend needs a GPU (there is no CPU fallback).");
   }
   if (device_ < 0 || device_ >= count) throw Error("Invalid GPU id " + std::to_string(device_) + ".");
-  HIP_CHECK(hipSetDevice(device_));
-  HIP_CHECK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
-  HIP_CHECK(hipStreamCreateWithFlags(&side_stream_, hipStreamNonBlocking));
-
-  d_masks_ = static_cast<uint64_t*>(arena_.Alloc(sizeof(uint64_t) * kInputPlanes * max_batch_));
-  d_values_ = AllocF(static_cast<size_t>(kInputPlanes) * max_batch_);
-  d_policy_ = AllocF(static_cast<size_t>(kPolicyOutputs) * max_batch_);
-  d_wdl_ = AllocF(3 * static_cast<size_t>(max_batch_));
-  d_mlh_ = AllocF(max_batch_);
-
+  CreateStreams();
   if (attn_body_) {
     if (fp32_) throw Error("precision=fp32 is available for residual-tower networks only.");
     BuildAttentionBody(file);
-    if (fp8_) DefaultCalibration();
   } else if (fp8_) {
     throw Error("precision=fp8 is available for attention-body networks only.");
   } else if (fp32_) {
@@ -713,11 +750,23 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   } else {
     BuildResnet<half_t>(file);
   }
+  AllocActivations();
+  if (fp8_) DefaultCalibration();
   HIP_CHECK(hipStreamSynchronize(stream_));
+  for (int i = 1; i < lane_count_; i++) extra_lanes_.push_back(std::make_unique<Mi355xNetwork>(*this, LaneTag{}));
+  ReleaseAllLanes();
+}
+
+Mi355xNetwork::Mi355xNetwork(const Mi355xNetwork& parent, LaneTag) : ModelState(parent) {
+  pool_ = parent.pool_;
+  is_lane_ = true;
+  CreateStreams();
+  AllocActivations();
 }
 
 Mi355xNetwork::~Mi355xNetwork() {
-  {
+  if (!is_lane_) {   // the network that owns weights and lanes
+    extra_lanes_.clear();
     std::lock_guard<std::mutex> lock(pool_->mutex);
     pool_->network_alive = false;
     pool_->free_slots.clear();
@@ -734,6 +783,71 @@ Mi355xNetwork::~Mi355xNetwork() {
     }
     (void)hipStreamDestroy(stream_);
   }
+}
+
+// Streams and events of one lane.
+void Mi355xNetwork::CreateStreams() {
+  HIP_CHECK(hipSetDevice(device_));
+  HIP_CHECK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+  HIP_CHECK(hipStreamCreateWithFlags(&side_stream_, hipStreamNonBlocking));
+}
+
+// Device buffers of one lane (inputs, activations, outputs), sized for max_batch_.
+void Mi355xNetwork::AllocActivations() {
+  d_masks_ = static_cast<uint64_t*>(arena_.Alloc(sizeof(uint64_t) * kInputPlanes * max_batch_));
+  d_values_ = AllocF(static_cast<size_t>(kInputPlanes) * max_batch_);
+  d_policy_ = AllocF(static_cast<size_t>(kPolicyOutputs) * max_batch_);
+  d_wdl_ = AllocF(3 * static_cast<size_t>(max_batch_));
+  d_mlh_ = AllocF(max_batch_);
+  if (!attn_body_) {
+    const size_t ts = fp32_ ? sizeof(float) : sizeof(half_t);
+    const size_t B = static_cast<size_t>(max_batch_);
+    const size_t cmax = res_cmax_;
+    r_in_ = arena_.Alloc(ts * B * 64 * kInputPlanes);
+    r_x_ = arena_.Alloc(ts * B * 64 * cmax);
+    r_y_ = arena_.Alloc(ts * B * 64 * cmax);
+    r_v_ = arena_.Alloc(ts * 36 * B * 4 * std::max<size_t>(filters_, kInputPlanes));
+    r_m_ = arena_.Alloc(ts * 36 * B * 4 * cmax);
+    r_h1_ = arena_.Alloc(ts * B * 64 * cmax);
+    r_h2_ = arena_.Alloc(ts * B * res_max_fc_);
+    return;
+  }
+  const size_t T = static_cast<size_t>(max_batch_) * 64;
+  in0_ = AllocH(T * in_ld_);
+  x_ = AllocH(T * emb_);
+  t_ = AllocH(T * emb_);
+  qkv_ = AllocH(T * 3 * d_model_);
+  att_ = AllocH(T * d_model_);
+  ffn_ = AllocH(T * std::max(dff_, emb_dff_));
+  if (pe_dense_) {
+    pre_in_ = AllocH(static_cast<size_t>(max_batch_) * 768);
+    pre_out_ = AllocH(T * enc_ch_);
+  }
+  if (any_smolgen_) {
+    sg1_ = AllocH(T * sg_hc_);
+    sg2_ = AllocH(static_cast<size_t>(max_batch_) * sg_hs_);
+    sg2f_ = AllocF(static_cast<size_t>(max_batch_) * sg_hs_ * 16);  // up to 16 split-K slices
+    for (size_t i = 0; i < encoders_.size(); i++) {
+      hipEvent_t a, b;
+      HIP_CHECK(hipEventCreateWithFlags(&a, hipEventDisableTiming));
+      HIP_CHECK(hipEventCreateWithFlags(&b, hipEventDisableTiming));
+      fork_events_.push_back(a);
+      join_events_.push_back(b);
+    }
+    sg3_ = AllocH(static_cast<size_t>(max_batch_) * sg_gen_);
+    sbias_ = AllocH(static_cast<size_t>(max_batch_) * heads_ * 4096);
+  }
+  if (fp8_) {
+    xq_ = static_cast<uint8_t*>(arena_.Alloc(T * emb_));
+    attq_ = static_cast<uint8_t*>(arena_.Alloc(T * d_model_));
+    ffnq_ = static_cast<uint8_t*>(arena_.Alloc(T * dff_));
+    d_absmax_ = AllocF(4 * encoders_.size() + 1);
+  }
+  pol_e_ = AllocH(T * pol_emb_);
+  pol_qk_ = AllocH(T * 2 * pol_d_);
+  pol_logits_ = AllocF(static_cast<size_t>(max_batch_) * 4096);
+  head1_ = AllocH(T * std::max(val_ch_, mov_ch_));
+  head2_ = AllocH(static_cast<size_t>(max_batch_) * std::max(val_fc_, mov_fc_));
 }
 
 void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
@@ -895,43 +1009,6 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     mov_fc2_ = MakeLinear(w.ip2_mov_w, w.ip2_mov_b, 1, mov_fc_);
   }
 
-  // Activations.
-  const size_t T = static_cast<size_t>(max_batch_) * 64;
-  in0_ = AllocH(T * in_ld_);
-  x_ = AllocH(T * emb_);
-  t_ = AllocH(T * emb_);
-  qkv_ = AllocH(T * 3 * d_model_);
-  att_ = AllocH(T * d_model_);
-  ffn_ = AllocH(T * std::max(dff_, emb_dff_));
-  if (pe_dense_) {
-    pre_in_ = AllocH(static_cast<size_t>(max_batch_) * 768);
-    pre_out_ = AllocH(T * enc_ch_);
-  }
-  if (any_smolgen_) {
-    sg1_ = AllocH(T * sg_hc_);
-    sg2_ = AllocH(static_cast<size_t>(max_batch_) * sg_hs_);
-    sg2f_ = AllocF(static_cast<size_t>(max_batch_) * sg_hs_ * 16);  // up to 16 split-K slices
-    for (size_t i = 0; i < encoders_.size(); i++) {
-      hipEvent_t a, b;
-      HIP_CHECK(hipEventCreateWithFlags(&a, hipEventDisableTiming));
-      HIP_CHECK(hipEventCreateWithFlags(&b, hipEventDisableTiming));
-      fork_events_.push_back(a);
-      join_events_.push_back(b);
-    }
-    sg3_ = AllocH(static_cast<size_t>(max_batch_) * sg_gen_);
-    sbias_ = AllocH(static_cast<size_t>(max_batch_) * heads_ * 4096);
-  }
-  if (fp8_) {
-    xq_ = static_cast<uint8_t*>(arena_.Alloc(T * emb_));
-    attq_ = static_cast<uint8_t*>(arena_.Alloc(T * d_model_));
-    ffnq_ = static_cast<uint8_t*>(arena_.Alloc(T * dff_));
-    d_absmax_ = AllocF(4 * encoders_.size() + 1);
-  }
-  pol_e_ = AllocH(T * pol_emb_);
-  pol_qk_ = AllocH(T * 2 * pol_d_);
-  pol_logits_ = AllocF(static_cast<size_t>(max_batch_) * 4096);
-  head1_ = AllocH(T * std::max(val_ch_, mov_ch_));
-  head2_ = AllocH(static_cast<size_t>(max_batch_) * std::max(val_fc_, mov_fc_));
 }
 
 
@@ -1082,15 +1159,8 @@ void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
     max_fc = std::max(max_fc, mov_fc_);
   }
 
-  const size_t B = static_cast<size_t>(max_batch_);
-  const size_t cmax = static_cast<size_t>(std::max(filters_, max_head_ch));
-  r_in_ = arena_.Alloc(sizeof(T) * B * 64 * kInputPlanes);
-  r_x_ = arena_.Alloc(sizeof(T) * B * 64 * cmax);
-  r_y_ = arena_.Alloc(sizeof(T) * B * 64 * cmax);
-  r_v_ = arena_.Alloc(sizeof(T) * 36 * B * 4 * std::max<size_t>(filters_, kInputPlanes));
-  r_m_ = arena_.Alloc(sizeof(float) * 36 * B * 4 * cmax);
-  r_h1_ = arena_.Alloc(sizeof(T) * B * 64 * cmax);
-  r_h2_ = arena_.Alloc(sizeof(T) * B * static_cast<size_t>(max_fc));
+  res_max_fc_ = static_cast<size_t>(max_fc);
+  res_cmax_ = static_cast<size_t>(std::max(filters_, max_head_ch));
 }
 
 // One 3x3 convolution: input transform, 36 batched GEMMs, output transform with the fused tail.
@@ -1358,8 +1428,64 @@ void Mi355xNetwork::ForwardDevice(int batch) {
   HIP_CHECK(hipGraphLaunch(it->second, stream_));
 }
 
+Mi355xNetwork* Mi355xNetwork::AcquireLane() {
+  std::unique_lock<std::mutex> lock(lane_mutex_);
+  lane_cv_.wait(lock, [&] { return !free_lanes_.empty(); });
+  Mi355xNetwork* lane = free_lanes_.back();   // most recently used first
+  free_lanes_.pop_back();
+  return lane;
+}
+
+void Mi355xNetwork::ReleaseLane(Mi355xNetwork* lane) {
+  {
+    std::lock_guard<std::mutex> lock(lane_mutex_);
+    free_lanes_.push_back(lane);
+  }
+  lane_cv_.notify_all();
+}
+
+// Exclusive use of the network (profiling, timing, calibration): waits until no
+// computation is in flight on any lane.
+void Mi355xNetwork::AcquireAllLanes() {
+  std::unique_lock<std::mutex> lock(lane_mutex_);
+  lane_cv_.wait(lock, [&] { return static_cast<int>(free_lanes_.size()) == lane_count_; });
+  free_lanes_.clear();
+}
+
+void Mi355xNetwork::ReleaseAllLanes() {
+  {
+    std::lock_guard<std::mutex> lock(lane_mutex_);
+    free_lanes_.clear();
+    for (auto it = extra_lanes_.rbegin(); it != extra_lanes_.rend(); ++it) free_lanes_.push_back(it->get());
+    free_lanes_.push_back(this);
+  }
+  lane_cv_.notify_all();
+}
+
 void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {
   if (batch <= 0) return;
+  if (profiling_.load()) {   // per-kernel timing records live in this object: run alone, on this lane
+    AcquireAllLanes();
+    try {
+      EvaluateOnLane(slot, batch);
+    } catch (...) {
+      ReleaseAllLanes();
+      throw;
+    }
+    ReleaseAllLanes();
+    return;
+  }
+  Mi355xNetwork* lane = AcquireLane();
+  try {
+    lane->EvaluateOnLane(slot, batch);
+  } catch (...) {
+    ReleaseLane(lane);
+    throw;
+  }
+  ReleaseLane(lane);
+}
+
+void Mi355xNetwork::EvaluateOnLane(HostSlot* slot, int batch) {
   std::lock_guard<std::mutex> lock(eval_mutex_);
   HIP_CHECK(hipSetDevice(device_));
   HIP_CHECK(hipMemcpyAsync(d_masks_, slot->masks, sizeof(uint64_t) * kInputPlanes * batch, hipMemcpyHostToDevice,
@@ -1394,9 +1520,14 @@ void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {
 double Mi355xNetwork::TimeResidentForward(int batch, int iters) {
   if (batch < 1 || batch > max_batch_) throw Error("batch out of range");
   if (iters < 1) throw Error("iters must be positive");
+  AcquireAllLanes();
+  struct Release {
+    Mi355xNetwork* n;
+    ~Release() { n->ReleaseAllLanes(); }
+  } release{this};
   std::lock_guard<std::mutex> lock(eval_mutex_);
   HIP_CHECK(hipSetDevice(device_));
-  const bool was_profiling = profiling_;
+  const bool was_profiling = profiling_.load();
   profiling_ = false;
   hipEvent_t start = NewEvent(), stop = NewEvent();
   HIP_CHECK(hipEventRecord(start, stream_));

@@ -80,6 +80,8 @@ class Mi355xNetwork : public Network {
     };
     add("gpu", std::to_string(options.GetOrDefault<int>("gpu", 0)));
     add("max_batch", std::to_string(options.GetOrDefault<int>("max_batch", 1024)));
+    add("lanes", std::to_string(options.GetOrDefault<int>("lanes", 4)));
+    add("graphs", options.GetOrDefault<bool>("graphs", true) ? "true" : "false");
     const std::string precision = options.GetOrDefault<std::string>("precision", "fp16");
     add("precision", precision);
     if (precision == "fp8") {

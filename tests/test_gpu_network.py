@@ -359,3 +359,46 @@ def test_graph_replays_equal_eager_launches(name, options, positions):
             comp.ComputeBlocking()
             outs.append(comp.results())
         np.testing.assert_array_equal(outs[0]["policy"], outs[1]["policy"])
+
+
+@pytest.mark.parametrize("name,options", [("tiny_attn", "lanes=1"), ("tiny_attn", "lanes=3"), ("tiny_resnet", "lanes=2"),
+                                          ("tiny_attn_f8", "precision=fp8,lanes=2")])
+def test_concurrent_computations_from_several_threads(name, options, positions):
+    """Search threads share one network (backendbench.cc:177-184 does the same): computations
+    issued concurrently from 4 threads, spread over the network's lanes, must each return
+    what a lone computation returns for the same positions."""
+    import threading
+    from lc0_amd import Network
+    net = Network(netgen.cached_config(name), options)
+    jobs = [(t, i, 1 + (7 * t + 13 * i) % 60) for t in range(4) for i in range(6)]
+    want = {}
+    for t, i, n in jobs:                      # sequential reference results
+        idx = (np.arange(n) * 3 + 11 * t + i) % 320
+        comp = net.NewComputation()
+        comp.AddInputs(positions["masks"][idx], positions["values"][idx])
+        comp.ComputeBlocking()
+        want[(t, i)] = comp.results()
+    got, errors = {}, []
+
+    def worker(t):
+        try:
+            for tt, i, n in jobs:
+                if tt != t:
+                    continue
+                idx = (np.arange(n) * 3 + 11 * t + i) % 320
+                comp = net.NewComputation()
+                comp.AddInputs(positions["masks"][idx], positions["values"][idx])
+                comp.ComputeBlocking()
+                got[(t, i)] = comp.results()
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    for key, w in want.items():
+        for field in ("policy", "q", "d", "m"):
+            np.testing.assert_array_equal(got[key][field], w[field])
