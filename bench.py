@@ -62,9 +62,27 @@ def cpu_baseline(path, masks, values, sample, seconds_budget=25.0):
     times.sort()
     med = times[len(times) // 2]
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return {"value": sample / med, "unit": "evals/s", "cores": cores, "kind": "port",
-            "sample": "%d positions per pass, %d timed passes, median; numpy float32 + its bundled BLAS sgemm"
-                      % (sample, len(times))}
+    out = {"value": sample / med, "unit": "evals/s", "cores": cores, "kind": "port",
+           "sample": "%d positions per pass, %d timed passes, median; numpy float32 + its bundled BLAS sgemm"
+                     % (sample, len(times))}
+    # The reference blas backend defaults to one thread (network_blas.cc:994): same oracle, BLAS pinned to 1 thread.
+    try:
+        from threadpoolctl import threadpool_limits
+        small = max(1, min(4, sample))
+        with threadpool_limits(limits=1):
+            bn.forward(m[:1], v[:1])
+            t1 = []
+            t_end = time.time() + 8.0
+            while len(t1) < 2 or (time.time() < t_end and len(t1) < 5):
+                t0 = time.perf_counter()
+                bn.forward(m[:small], v[:small])
+                t1.append(time.perf_counter() - t0)
+        t1.sort()
+        out["one_thread"] = {"value": small / t1[len(t1) // 2], "unit": "evals/s", "cores": 1,
+                             "sample": "%d positions per pass, %d timed passes, median" % (small, len(t1))}
+    except ImportError:
+        pass
+    return out
 
 
 def main():

@@ -40,11 +40,11 @@ int lc0mi_k_layer_norm(const uint16_t* x, const uint16_t* skip, const float* gam
 int lc0mi_k_layer_norm_rows(const float* x_f32, const uint16_t* x_f16, int pre_act, const uint16_t* skip,
                             const float* gamma, const float* beta, int rows, int C, float alpha, float eps,
                             uint16_t* y);
-/* Fused attention: qkv [B*64][3*heads*32] halves, bias [B][heads][64 q][64 k]
- * halves in natural order (may be NULL), out [B*64][heads*32]
+/* Fused attention, head depth 32, 64 or 128: qkv [B*64][3*heads*depth] halves, bias [B][heads][64 q][64 k]
+ * halves in natural order (may be NULL), out [B*64][heads*depth]
  * (src/neural/backends/blas/network_blas.cc:352-439). */
-int lc0mi_k_attention(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, float scale, uint16_t* out,
-                      int time_iters, double* ms);
+int lc0mi_k_attention(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, int depth, float scale,
+                      uint16_t* out, int time_iters, double* ms);
 /* Input planes -> [B*64][ld] halves with position encoding appended
  * (src/neural/backends/blas/network_blas.cc:973-981, 630-652). */
 int lc0mi_k_expand_planes_attn(const uint64_t* masks, const float* values, int batch, int ld, uint16_t* out,

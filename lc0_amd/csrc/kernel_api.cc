@@ -209,13 +209,13 @@ int lc0mi_k_layer_norm(const uint16_t* x, const uint16_t* skip, const float* gam
   });
 }
 
-int lc0mi_k_attention(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, float scale, uint16_t* out,
-                      int time_iters, double* ms) {
+int lc0mi_k_attention(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, int depth, float scale,
+                      uint16_t* out, int time_iters, double* ms) {
   return Guard([&] {
     RequireDevice();
-    if (batch < 1 || heads < 1) throw Error("bad attention shape");
+    if (batch < 1 || heads < 1 || !lc0mi::AttentionDepthSupported(depth)) throw Error("bad attention shape");
     Dev dev;
-    const int d = heads * 32;
+    const int d = heads * depth;
     auto* dq = reinterpret_cast<half_t*>(dev.Put(qkv, (size_t)batch * 64 * 3 * d));
     half_t* db = nullptr;
     if (bias) {
@@ -226,12 +226,12 @@ int lc0mi_k_attention(const uint16_t* qkv, const uint16_t* bias, int batch, int 
       db = reinterpret_cast<half_t*>(dev.Put(perm.data(), perm.size()));
     }
     auto* dout = reinterpret_cast<half_t*>(dev.Alloc((size_t)batch * 64 * d * 2));
-    lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr);
+    lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr, depth);
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());
     K_CHECK(hipMemcpy(out, dout, (size_t)batch * 64 * d * 2, hipMemcpyDeviceToHost));
     if (time_iters > 0 && ms) {
-      *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr); });
+      *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr, depth); });
     }
   });
 }

@@ -115,14 +115,15 @@ void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float
                      int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8 = nullptr,
                      float f8_mul = 1.0f);
 
-// Fused multi-head attention over 64 tokens, head depth 32.
+// Fused multi-head attention over 64 tokens, head depth 32, 64 or 128 (d_model = heads * depth).
 // qkv: [B*64][3*d_model] (q | k | v column blocks), bias: smolgen logits in the
 // tile-native layout produced by SmolgenBiasIndex (may be null), out: [B*64][d_model].
 void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int batch, int heads,
-                     float scale, hipStream_t stream);
+                     float scale, hipStream_t stream, int depth = 32);
+bool AttentionDepthSupported(int depth);
 // Same with e4m3 output: out[...] = e4m3(result * out_mul), saturating.
 void LaunchAttentionF8Out(const half_t* qkv, const half_t* bias, uint8_t* out, float out_mul, int batch, int heads,
-                          float scale, hipStream_t stream);
+                          float scale, hipStream_t stream, int depth = 32);
 // Position inside one head's 4096-entry bias block of logit (query q, key k).
 int SmolgenBiasIndex(int q, int k);
 

@@ -1000,31 +1000,33 @@ void LaunchQuantizeF8(const half_t* x, uint8_t* y, long long n, float mul, hipSt
 //   key = 16 s + 8 (e / 4) + 4 g + e % 4.
 // ---------------------------------------------------------------------------
 namespace {
-constexpr int kVStride = 40;  // halves per key row of V in LDS
-
-template <typename OutT>  // half_t, or uint8_t for e4m3 output scaled by out_mul
+// DEPTH = head depth (32, 64 or 128); OutT = half_t, or uint8_t for e4m3 output scaled by out_mul.
+template <int DEPTH, typename OutT>
 __global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict__ qkv,
                                                         const half_t* __restrict__ bias,
                                                         OutT* __restrict__ out, int total_heads, int heads,
                                                         float scale, float out_mul) {
+  constexpr int kVStride = DEPTH + 8;  // halves per key row of V in LDS
+  constexpr int DT = DEPTH / 32;       // 32-wide depth tiles of the output
   __shared__ __attribute__((aligned(16))) half_t Vs[4][64 * kVStride];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int gh_raw = blockIdx.x * 4 + wave;
   const bool live = gh_raw < total_heads;
   const int gh = live ? gh_raw : total_heads - 1;
   const int b = gh / heads, h = gh - b * heads;
-  const int d_model = heads * 32, ld = 3 * d_model;
-  const half_t* Q = qkv + (long long)b * 64 * ld + h * 32;
+  const int d_model = heads * DEPTH, ld = 3 * d_model;
+  const half_t* Q = qkv + (long long)b * 64 * ld + h * DEPTH;
   const half_t* Kp = Q + d_model;
   const half_t* V = Q + 2 * d_model;
   const int r = lane & 31, g = lane >> 5;
 
-  // Stage V (64 keys x 32 depth) into this wave's LDS region.
+  // Stage V (64 keys x DEPTH) into this wave's LDS region.
   half_t* vs = Vs[wave];
+  constexpr int VCH = DEPTH / 8;  // 16-byte chunks per key row
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
+  for (int i = 0; i < VCH; i++) {
     int v = lane + 64 * i;
-    int row = v >> 2, cv = v & 3;
+    int row = v / VCH, cv = v - row * VCH;
     *reinterpret_cast<uint4*>(&vs[row * kVStride + cv * 8]) =
         *reinterpret_cast<const uint4*>(V + (long long)row * ld + cv * 8);
   }
@@ -1037,7 +1039,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict
 #pragma unroll
       for (int e = 0; e < 16; e++) st[mt][nt][e] = 0.0f;
 #pragma unroll
-  for (int ks = 0; ks < 2; ks++) {
+  for (int ks = 0; ks < DEPTH / 16; ks++) {
     half8 kf[2], qf[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
@@ -1090,37 +1092,44 @@ __global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict
 
   __syncthreads();  // V tile visible (each wave reads only its own region)
 
-  floatx16 o[2];
+  floatx16 o[2][DT];
 #pragma unroll
   for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-    for (int e = 0; e < 16; e++) o[nt][e] = 0.0f;
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) o[nt][dt][e] = 0.0f;
 #pragma unroll
   for (int s = 0; s < 4; s++) {
-    half8 vf;
+    half8 pf[2];
 #pragma unroll
-    for (int e = 0; e < 8; e++) vf[e] = vs[(16 * s + 8 * (e / 4) + 4 * g + (e % 4)) * kVStride + r];
+    for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-    for (int nt = 0; nt < 2; nt++) {
-      half8 pf;
+      for (int e = 0; e < 8; e++) pf[nt][e] = (half_t)st[s / 2][nt][8 * (s % 2) + e];
 #pragma unroll
-      for (int e = 0; e < 8; e++) pf[e] = (half_t)st[s / 2][nt][8 * (s % 2) + e];
-      o[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(pf, vf, o[nt], 0, 0, 0);
+    for (int dt = 0; dt < DT; dt++) {
+      half8 vf;
+#pragma unroll
+      for (int e = 0; e < 8; e++) vf[e] = vs[(16 * s + 8 * (e / 4) + 4 * g + (e % 4)) * kVStride + dt * 32 + r];
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++) o[nt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(pf[nt], vf, o[nt][dt], 0, 0, 0);
     }
   }
   if (!live) return;
-  OutT* O = out + (long long)b * 64 * d_model + h * 32;
+  OutT* O = out + (long long)b * 64 * d_model + h * DEPTH;
 #pragma unroll
   for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-    for (int e = 0; e < 16; e++) {
-      int q = 32 * nt + 8 * (e / 4) + 4 * g + (e % 4);
-      if constexpr (sizeof(OutT) == 1) {
-        O[(long long)q * d_model + r] = (uint8_t)(PackFp8x4(o[nt][e] * out_mul, 0.0f, 0.0f, 0.0f) & 0xffu);
-      } else {
-        O[(long long)q * d_model + r] = (half_t)o[nt][e];
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        int q = 32 * nt + 8 * (e / 4) + 4 * g + (e % 4);
+        if constexpr (sizeof(OutT) == 1) {
+          O[(long long)q * d_model + dt * 32 + r] = (uint8_t)(PackFp8x4(o[nt][dt][e] * out_mul, 0.0f, 0.0f, 0.0f) & 0xffu);
+        } else {
+          O[(long long)q * d_model + dt * 32 + r] = (half_t)o[nt][dt][e];
+        }
       }
-    }
 }
 }  // namespace
 
@@ -1131,20 +1140,37 @@ int SmolgenBiasIndex(int q, int k) {
   return ((nt * 2 + mt) * 2 + blk / 2) * 512 + lane * 8 + (blk % 2) * 4 + j;
 }
 
-void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int batch, int heads, float scale,
-                     hipStream_t stream) {
-  int total = batch * heads;
+namespace {
+template <typename OutT>
+void LaunchAttentionT(const half_t* qkv, const half_t* bias, OutT* out, float out_mul, int batch, int heads, int depth,
+                      float scale, hipStream_t stream) {
+  const int total = batch * heads;
   if (total <= 0) return;
-  hipLaunchKernelGGL(attention_kernel<half_t>, dim3((total + 3) / 4), dim3(256), 0, stream, qkv, bias, out, total,
-                     heads, scale, 1.0f);
+  const dim3 grid((total + 3) / 4), block(256);
+  switch (depth) {
+    case 32:
+      hipLaunchKernelGGL((attention_kernel<32, OutT>), grid, block, 0, stream, qkv, bias, out, total, heads, scale, out_mul);
+      break;
+    case 64:
+      hipLaunchKernelGGL((attention_kernel<64, OutT>), grid, block, 0, stream, qkv, bias, out, total, heads, scale, out_mul);
+      break;
+    default:  // 128; callers check the depth
+      hipLaunchKernelGGL((attention_kernel<128, OutT>), grid, block, 0, stream, qkv, bias, out, total, heads, scale, out_mul);
+      break;
+  }
+}
+}  // namespace
+
+bool AttentionDepthSupported(int depth) { return depth == 32 || depth == 64 || depth == 128; }
+
+void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int batch, int heads, float scale,
+                     hipStream_t stream, int depth) {
+  LaunchAttentionT<half_t>(qkv, bias, out, 1.0f, batch, heads, depth, scale, stream);
 }
 
 void LaunchAttentionF8Out(const half_t* qkv, const half_t* bias, uint8_t* out, float out_mul, int batch, int heads,
-                          float scale, hipStream_t stream) {
-  int total = batch * heads;
-  if (total <= 0) return;
-  hipLaunchKernelGGL(attention_kernel<uint8_t>, dim3((total + 3) / 4), dim3(256), 0, stream, qkv, bias, out, total,
-                     heads, scale, out_mul);
+                          float scale, hipStream_t stream, int depth) {
+  LaunchAttentionT<uint8_t>(qkv, bias, out, out_mul, batch, heads, depth, scale, stream);
 }
 
 // ---------------------------------------------------------------------------

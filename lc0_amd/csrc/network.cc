@@ -251,6 +251,10 @@ struct ModelState {
   Linear emb_lin_, smolgen_w_, pol_emb_lin_, pol_qk_lin_, val_emb_lin_, val_fc1_, val_fc2_, mov_emb_lin_, mov_fc1_,
       mov_fc2_;
   std::vector<EncoderDev> encoders_;
+  int depth_ = 32;   // attention head depth of the body
+  // Policy-head encoder layers (network_blas.cc:836-842): post-LN layers without smolgen on the policy embedding.
+  std::vector<EncoderDev> pol_encoders_;
+  int pe_heads_ = 0, pe_dmodel_ = 0, pe_dff_ = 0, pe_depth_ = 32, pe_ffn_act_ = kActNone, pol_emb_act_ = kActNone;
   half_t* pos_enc_ = nullptr;
   float* ppo_ = nullptr;
   int16_t* inv_map_ = nullptr;
@@ -305,6 +309,9 @@ class Mi355xNetwork : public Network, protected ModelState {
   void BuildResnet(const WeightsFile& file);
   void ForwardDevice(int batch);
   void ForwardAttentionBody(int B);
+  void BuildAttentionPolicy(const PolicyHead& ph, int in_channels);
+  void ForwardAttentionPolicy(const half_t* x, int ld_x, int B);
+  EncoderDev MakeEncoderLayer(const EncoderLayer& l, int emb, int d_model, int dff);
   template <typename T>
   void ForwardResnet(int B);
   template <typename T>
@@ -349,6 +356,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   half_t *sg1_ = nullptr, *sg2_ = nullptr, *sg3_ = nullptr, *sbias_ = nullptr;
   float* sg2f_ = nullptr;  // split-K accumulator of smolgen dense1
   half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
+  half_t *pe_qkv_ = nullptr, *pe_att_ = nullptr, *pe_t_ = nullptr, *pe_ffn_ = nullptr;   // policy encoder scratch
   float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
   half_t *pre_in_ = nullptr, *pre_out_ = nullptr;
   bool calibrating_ = false;
@@ -799,6 +807,18 @@ void Mi355xNetwork::AllocActivations() {
   d_policy_ = AllocF(static_cast<size_t>(kPolicyOutputs) * max_batch_);
   d_wdl_ = AllocF(3 * static_cast<size_t>(max_batch_));
   d_mlh_ = AllocF(max_batch_);
+  if (attn_policy_) {
+    const size_t T = static_cast<size_t>(max_batch_) * 64;
+    pol_e_ = AllocH(T * pol_emb_);
+    pol_qk_ = AllocH(T * 2 * pol_d_);
+    pol_logits_ = AllocF(static_cast<size_t>(max_batch_) * 4096);
+    if (!pol_encoders_.empty()) {
+      pe_qkv_ = AllocH(T * 3 * pe_dmodel_);
+      pe_att_ = AllocH(T * pe_dmodel_);
+      pe_t_ = AllocH(T * pol_emb_);
+      pe_ffn_ = AllocH(T * pe_dff_);
+    }
+  }
   if (!attn_body_) {
     const size_t ts = fp32_ ? sizeof(float) : sizeof(half_t);
     const size_t B = static_cast<size_t>(max_batch_);
@@ -843,11 +863,101 @@ void Mi355xNetwork::AllocActivations() {
     ffnq_ = static_cast<uint8_t*>(arena_.Alloc(T * dff_));
     d_absmax_ = AllocF(4 * encoders_.size() + 1);
   }
-  pol_e_ = AllocH(T * pol_emb_);
-  pol_qk_ = AllocH(T * 2 * pol_d_);
-  pol_logits_ = AllocF(static_cast<size_t>(max_batch_) * 4096);
   head1_ = AllocH(T * std::max(val_ch_, mov_ch_));
   head2_ = AllocH(static_cast<size_t>(max_batch_) * std::max(val_fc_, mov_fc_));
+}
+
+// Weights of one post-LN encoder layer without smolgen (q, k and v stacked into one matrix).
+EncoderDev Mi355xNetwork::MakeEncoderLayer(const EncoderLayer& l, int emb, int d_model, int dff) {
+  EncoderDev e;
+  if (static_cast<int>(l.mha.q_b.size()) != d_model || static_cast<int>(l.ffn.dense1_b.size()) != dff) {
+    throw Error("Encoder layers of different sizes are not supported.");
+  }
+  Vec qkv_w, qkv_b;
+  qkv_w.reserve(3 * l.mha.q_w.size());
+  for (const Vec* v : {&l.mha.q_w, &l.mha.k_w, &l.mha.v_w}) qkv_w.insert(qkv_w.end(), v->begin(), v->end());
+  for (const Vec* v : {&l.mha.q_b, &l.mha.k_b, &l.mha.v_b}) qkv_b.insert(qkv_b.end(), v->begin(), v->end());
+  e.qkv = MakeLinear(qkv_w, qkv_b, 3 * d_model, emb);
+  e.dense = MakeLinear(l.mha.dense_w, l.mha.dense_b, emb, d_model);
+  e.ffn1 = MakeLinear(l.ffn.dense1_w, l.ffn.dense1_b, dff, emb);
+  e.ffn2 = MakeLinear(l.ffn.dense2_w, l.ffn.dense2_b, emb, dff);
+  if (static_cast<int>(l.ln1_gammas.size()) != emb || static_cast<int>(l.ln2_gammas.size()) != emb) {
+    throw Error("Layer norm parameters do not match the embedding size.");
+  }
+  e.ln1_g = UploadF(l.ln1_gammas); e.ln1_b = UploadF(l.ln1_betas);
+  e.ln2_g = UploadF(l.ln2_gammas); e.ln2_b = UploadF(l.ln2_betas);
+  return e;
+}
+
+// Attention policy head (network_blas.cc:806-914) on token-major input of in_channels channels.
+void Mi355xNetwork::BuildAttentionPolicy(const PolicyHead& ph, int in_channels) {
+  pol_emb_ = static_cast<int>(ph.ip_pol_b.size());
+  pol_d_ = static_cast<int>(ph.ip2_pol_b.size());
+  if (pol_emb_ <= 0 || pol_emb_ % 8 || pol_d_ % 8 || pol_d_ <= 0 || in_channels % 8) {
+    throw Error("Unsupported policy head sizes.");
+  }
+  pol_emb_lin_ = MakeLinear(ph.ip_pol_w, ph.ip_pol_b, pol_emb_, in_channels);
+  if (!ph.pol_encoder.empty()) {
+    pe_heads_ = ph.pol_encoder_head_count;
+    pe_dmodel_ = static_cast<int>(ph.pol_encoder[0].mha.q_b.size());
+    pe_dff_ = static_cast<int>(ph.pol_encoder[0].ffn.dense1_b.size());
+    if (pe_heads_ <= 0 || pe_dmodel_ <= 0 || pe_dmodel_ % pe_heads_ || pe_dff_ <= 0 || pe_dff_ % 8) {
+      throw Error("Unsupported policy encoder sizes.");
+    }
+    pe_depth_ = pe_dmodel_ / pe_heads_;
+    if (!AttentionDepthSupported(pe_depth_)) throw Error("Policy encoder head depth must be 32, 64 or 128.");
+    for (const EncoderLayer& l : ph.pol_encoder) {
+      if (l.mha.has_smolgen) throw Error("Smolgen in policy encoder layers is not supported.");
+      pol_encoders_.push_back(MakeEncoderLayer(l, pol_emb_, pe_dmodel_, pe_dff_));
+    }
+  }
+  {
+    Vec qk_w(ph.ip2_pol_w), qk_b(ph.ip2_pol_b);
+    qk_w.insert(qk_w.end(), ph.ip3_pol_w.begin(), ph.ip3_pol_w.end());
+    qk_b.insert(qk_b.end(), ph.ip3_pol_b.begin(), ph.ip3_pol_b.end());
+    pol_qk_lin_ = MakeLinear(qk_w, qk_b, 2 * pol_d_, pol_emb_);
+  }
+  if (ph.ip4_pol_w.size() != static_cast<size_t>(4) * pol_d_) throw Error("Promotion weights have a wrong size.");
+  ppo_ = UploadF(ph.ip4_pol_w);
+  inv_map_ = arena_.Upload(AttnPolicyInverseMap());
+}
+
+void Mi355xNetwork::ForwardAttentionPolicy(const half_t* x, int ld_x, int B) {
+  const int T = B * 64;
+  Gemm("gemm_policy_embed", x, ld_x, pol_emb_lin_, pol_e_, pol_emb_, T, pol_emb_act_);
+  for (const EncoderDev& e : pol_encoders_) {   // alpha 1, eps 1e-6 (network_blas.cc:836-842)
+    Gemm("gemm_pol_qkv", pol_e_, pol_emb_, e.qkv, pe_qkv_, 3 * pe_dmodel_, T, kActNone);
+    Timed("attention", 4.0 * 64 * 64 * pe_depth_ * B * pe_heads_, B * pe_heads_ * 2.0 * 4 * 64 * pe_depth_, [&] {
+      LaunchAttention(pe_qkv_, nullptr, pe_att_, B, pe_heads_, 1.0f / std::sqrt(static_cast<float>(pe_depth_)), stream_,
+                      pe_depth_);
+    });
+    Gemm("gemm_pol_dense", pe_att_, pe_dmodel_, e.dense, pe_t_, pol_emb_, T, kActNone);
+    Timed("layer_norm_skip", 0.0, 6.0 * T * pol_emb_, [&] {
+      LaunchLayerNorm(pe_t_, pol_e_, pol_e_, e.ln1_g, e.ln1_b, T, pol_emb_, 1.0f, 1e-6f, stream_);
+    });
+    Gemm("gemm_pol_ffn1", pol_e_, pol_emb_, e.ffn1, pe_ffn_, pe_dff_, T, pe_ffn_act_);
+    Gemm("gemm_pol_ffn2", pe_ffn_, pe_dff_, e.ffn2, pe_t_, pol_emb_, T, kActNone);
+    Timed("layer_norm_skip", 0.0, 6.0 * T * pol_emb_, [&] {
+      LaunchLayerNorm(pe_t_, pol_e_, pol_e_, e.ln2_g, e.ln2_b, T, pol_emb_, 1.0f, 1e-6f, stream_);
+    });
+  }
+  Gemm("gemm_policy_qk", pol_e_, pol_emb_, pol_qk_lin_, pol_qk_, 2 * pol_d_, T, kActNone);
+  {
+    GemmArgs g;
+    g.A = pol_qk_; g.lda = 2 * pol_d_; g.strideA = 64LL * 2 * pol_d_;
+    g.W = pol_qk_ + pol_d_; g.ldw = 2 * pol_d_; g.strideW = 64LL * 2 * pol_d_;
+    g.C = pol_logits_; g.ldc = 64; g.strideC = 4096;
+    g.M = 64; g.N = 64; g.K = pol_d_; g.batch = B;
+    g.scale = 1.0f / std::sqrt(static_cast<float>(pol_d_));
+    g.act = kActNone;
+    g.out_f32 = true;
+    const std::string label = std::string("gemm_policy_logits|") + GemmVariantName(g);
+    Timed(label.c_str(), 2.0 * 64 * 64 * pol_d_ * B, B * (2.0 * 2 * 64 * pol_d_ + 4.0 * 4096),
+          [&] { LaunchGemm(g, stream_); });
+  }
+  Timed("policy_gather", 0.0, B * (4.0 * 4288 + 4.0 * 1858), [&] {
+    LaunchAttnPolicyGather(pol_logits_, pol_qk_, 2 * pol_d_, pol_d_, ppo_, pol_d_, inv_map_, d_policy_, B, stream_);
+  });
 }
 
 void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
@@ -862,7 +972,6 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   if (!attn_policy_) throw Error("Attention-body networks need the attention policy head.");
   const PolicyHead& ph = w.policy_heads.at(policy_head_);
   const ValueHead& vh = w.value_heads.at(value_head_);
-  if (!ph.pol_encoder.empty()) throw Error("Policy encoder layers are not supported.");
 
   emb_ = static_cast<int>(w.ip_emb_b.size());
   heads_ = w.encoder_head_count;
@@ -870,7 +979,11 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   if (w.encoder.empty() || heads_ <= 0) throw Error("Attention body without encoder layers.");
   d_model_ = static_cast<int>(w.encoder[0].mha.q_b.size());
   dff_ = static_cast<int>(w.encoder[0].ffn.dense1_b.size());
-  if (d_model_ != heads_ * 32) throw Error("Only attention heads of depth 32 are supported.");
+  depth_ = d_model_ / heads_;
+  if (d_model_ != heads_ * depth_ || !AttentionDepthSupported(depth_)) {
+    throw Error("Attention head depth must be 32, 64 or 128 (got " + std::to_string(d_model_) + " / " +
+                std::to_string(heads_) + ").");
+  }
   if (dff_ % 8 != 0) throw Error("FFN width must be a multiple of 8.");
   alpha_ = static_cast<float>(std::pow(2.0 * w.encoder.size(), -0.25));
   eps_ = pe_dense_ ? 1e-3f : 1e-6f;   // src/neural/backends/blas/network_blas.cc:719
@@ -979,19 +1092,9 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   }
 
   // Heads.
-  pol_emb_ = static_cast<int>(ph.ip_pol_b.size());
-  pol_d_ = static_cast<int>(ph.ip2_pol_b.size());
-  if (pol_emb_ % 8 || pol_d_ % 8 || pol_d_ <= 0) throw Error("Unsupported policy head sizes.");
-  pol_emb_lin_ = MakeLinear(ph.ip_pol_w, ph.ip_pol_b, pol_emb_, emb_);
-  {
-    Vec qk_w(ph.ip2_pol_w), qk_b(ph.ip2_pol_b);
-    qk_w.insert(qk_w.end(), ph.ip3_pol_w.begin(), ph.ip3_pol_w.end());
-    qk_b.insert(qk_b.end(), ph.ip3_pol_b.begin(), ph.ip3_pol_b.end());
-    pol_qk_lin_ = MakeLinear(qk_w, qk_b, 2 * pol_d_, pol_emb_);
-  }
-  if (ph.ip4_pol_w.size() != static_cast<size_t>(4) * pol_d_) throw Error("Promotion weights have a wrong size.");
-  ppo_ = UploadF(ph.ip4_pol_w);
-  inv_map_ = arena_.Upload(AttnPolicyInverseMap());
+  pol_emb_act_ = default_act_;
+  pe_ffn_act_ = ffn_act_;
+  BuildAttentionPolicy(ph, emb_);
 
   val_ch_ = static_cast<int>(vh.ip_val_b.size());
   val_fc_ = static_cast<int>(vh.ip1_val_b.size());
@@ -1060,7 +1163,9 @@ template <typename T>
 void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
   const NetWeights& w = file.weights;
   const NetworkFormat& nf = file.format;
-  if (attn_policy_) throw Error("The attention policy head on a residual tower is not supported.");
+  if (attn_policy_ && sizeof(T) != 2) {
+    throw Error("The attention policy head on a residual tower needs precision=fp16.");
+  }
   if (w.residual.empty() && w.input.weights.empty()) throw Error("Network has no input convolution.");
   const PolicyHead& ph = w.policy_heads.at(policy_head_);
   const ValueHead& vh = w.value_heads.at(value_head_);
@@ -1129,7 +1234,13 @@ void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
   };
 
   int max_head_ch = 8;
-  if (conv_policy_) {
+  if (attn_policy_) {
+    // Attention policy on a convolutional body: SELU on the embedding and in the policy
+    // encoders' FFN (hard-coded in the reference, network_blas.cc:822-842).
+    pol_emb_act_ = kActSelu;
+    pe_ffn_act_ = kActSelu;
+    BuildAttentionPolicy(ph, filters_);
+  } else if (conv_policy_) {
     res_policy1_ = make_conv(ph.policy1, filters_, filters_);
     const int pol_out = static_cast<int>(ph.policy.biases.size());
     if (pol_out < 73 || pol_out > 1024) throw Error("Convolutional policy head has an unexpected size.");
@@ -1209,7 +1320,9 @@ void Mi355xNetwork::ForwardResnet(int B) {
     fc("gemm_mlh_fc2", r_h2_, res_mov_fc2_, d_mlh_, B, kActRelu, true);
   }
   // Policy head.
-  if (conv_policy_) {
+  if (attn_policy_) {
+    if constexpr (sizeof(T) == 2) ForwardAttentionPolicy(static_cast<const half_t*>(r_x_), filters_, B);
+  } else if (conv_policy_) {
     WinogradConv<T>("gemm_winograd_policy", res_policy1_, r_x_, nullptr, nullptr, default_act_, r_y_, B);
     WinogradConv<T>("gemm_winograd_policy", res_policy_conv_, r_y_, nullptr, nullptr, kActNone, r_h1_, B);
     Timed("policy_gather", 0.0, B * (sizeof(T) * 73.0 * 64 + 4.0 * 1858), [&] {
@@ -1297,18 +1410,18 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       Gemm("gemm_qkv", x_, emb_, e.qkv, qkv_, 3 * d_model_, T, kActNone);
     }
     if (e.has_smolgen && ss != stream_) HIP_CHECK(hipStreamWaitEvent(stream_, join_events_[li], 0));
-    const double att_flops = 4.0 * 2 * 64 * 64 * 32 * B * heads_ / 2.0;
+    const double att_flops = 4.0 * 64 * 64 * depth_ * B * heads_;
     const bool att_f8 = f8 && q_dense_;
     const double att_bytes =
-        B * heads_ * (2.0 * 3 * 64 * 32 + (att_f8 ? 1.0 : 2.0) * 64 * 32 + (bias ? 2.0 * 4096 : 0.0));
-    const float att_scale = 1.0f / std::sqrt(32.0f);
+        B * heads_ * (2.0 * 3 * 64 * depth_ + (att_f8 ? 1.0 : 2.0) * 64 * depth_ + (bias ? 2.0 * 4096 : 0.0));
+    const float att_scale = 1.0f / std::sqrt(static_cast<float>(depth_));
     if (att_f8) {
       Timed("attention", att_flops, att_bytes,
-            [&] { LaunchAttentionF8Out(qkv_, bias, attq_, 1.0f / e.s_att, B, heads_, att_scale, stream_); });
+            [&] { LaunchAttentionF8Out(qkv_, bias, attq_, 1.0f / e.s_att, B, heads_, att_scale, stream_, depth_); });
       GemmF8("gemm_mha_dense", attq_, e.dense, e.dense8, t_, T, kActNone, false, 1.0f);
     } else {
       Timed("attention", att_flops, att_bytes,
-            [&] { LaunchAttention(qkv_, bias, att_, B, heads_, att_scale, stream_); });
+            [&] { LaunchAttention(qkv_, bias, att_, B, heads_, att_scale, stream_, depth_); });
       if (calibrating_) RecordAbsMax(att_, static_cast<size_t>(T) * d_model_, static_cast<int>(4 * li + 1));
       Gemm("gemm_mha_dense", att_, d_model_, e.dense, t_, emb_, T, kActNone);
     }
@@ -1355,24 +1468,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     Gemm("gemm_mlh_fc2", head2_, mov_fc_, mov_fc2_, d_mlh_, 1, B, kActRelu, /*out_f32=*/true);
   }
   // Policy head.
-  Gemm("gemm_policy_embed", x_, emb_, pol_emb_lin_, pol_e_, pol_emb_, T, default_act_);
-  Gemm("gemm_policy_qk", pol_e_, pol_emb_, pol_qk_lin_, pol_qk_, 2 * pol_d_, T, kActNone);
-  {
-    GemmArgs g;
-    g.A = pol_qk_; g.lda = 2 * pol_d_; g.strideA = 64LL * 2 * pol_d_;
-    g.W = pol_qk_ + pol_d_; g.ldw = 2 * pol_d_; g.strideW = 64LL * 2 * pol_d_;
-    g.C = pol_logits_; g.ldc = 64; g.strideC = 4096;
-    g.M = 64; g.N = 64; g.K = pol_d_; g.batch = B;
-    g.scale = 1.0f / std::sqrt(static_cast<float>(pol_d_));
-    g.act = kActNone;
-    g.out_f32 = true;
-    const std::string label = std::string("gemm_policy_logits|") + GemmVariantName(g);
-    Timed(label.c_str(), 2.0 * 64 * 64 * pol_d_ * B, B * (2.0 * 2 * 64 * pol_d_ + 4.0 * 4096),
-          [&] { LaunchGemm(g, stream_); });
-  }
-  Timed("policy_gather", 0.0, B * (4.0 * 4288 + 4.0 * 1858), [&] {
-    LaunchAttnPolicyGather(pol_logits_, pol_qk_, 2 * pol_d_, pol_d_, ppo_, pol_d_, inv_map_, d_policy_, B, stream_);
-  });
+  ForwardAttentionPolicy(x_, emb_, B);
 }
 
 void Mi355xNetwork::LaunchEager(int batch) {

@@ -23,7 +23,7 @@ def _lib():
         lib.lc0mi_k_expand_planes_nhwc.argtypes = [vp, vp, ci, vp]
         lib.lc0mi_k_gemm_f32.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, ci, vp, ci]
         lib.lc0mi_k_layer_norm.argtypes = [vp, vp, vp, vp, ci, ci, cf, cf, vp, ci, cd]
-        lib.lc0mi_k_attention.argtypes = [vp, vp, ci, ci, cf, vp, ci, cd]
+        lib.lc0mi_k_attention.argtypes = [vp, vp, ci, ci, ci, cf, vp, ci, cd]
         lib.lc0mi_k_expand_planes_attn.argtypes = [vp, vp, ci, ci, vp, ci, cd]
         lib.lc0mi_k_expand_planes_nchw.argtypes = [vp, vp, ci, vp]
         lib.lc0mi_k_attn_policy_gather.argtypes = [vp, vp, vp, ci, ci, vp]
@@ -119,13 +119,14 @@ def layer_norm(x, skip, gamma, beta, alpha, eps, time_iters=0):
     return (y, ms.value) if time_iters else y
 
 
-def attention(qkv, bias, batch, heads, scale, time_iters=0):
-    """qkv [B*64, 3*heads*32], bias [B, heads, 64, 64] or None -> [B*64, heads*32]."""
+def attention(qkv, bias, batch, heads, scale, time_iters=0, depth=32):
+    """qkv [B*64, 3*heads*depth], bias [B, heads, 64, 64] or None -> [B*64, heads*depth]."""
     qkv = _h(qkv)
     b = _h(bias) if bias is not None else None
-    out = np.zeros((batch * 64, heads * 32), np.float16)
+    out = np.zeros((batch * 64, heads * depth), np.float16)
     ms = C.c_double(0)
-    _check(_lib().lc0mi_k_attention(_ptr(qkv), _ptr(b), batch, heads, scale, _ptr(out), time_iters, C.byref(ms)))
+    _check(_lib().lc0mi_k_attention(_ptr(qkv), _ptr(b), batch, heads, depth, scale, _ptr(out), time_iters,
+                                    C.byref(ms)))
     return (out, ms.value) if time_iters else out
 
 

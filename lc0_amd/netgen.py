@@ -36,9 +36,46 @@ class _Gen:
         return (self.rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
 
 
+def _encoder_layer(g, emb, d_model, dff, std, bias_std, smolgen=None, heads=None, perturb_ln=False):
+    """One EncoderLayer message (q/k/v/dense, layer norms, FFN, optional smolgen)."""
+    def fc(cout, cin, bias=True):
+        w = g.normal((cout, cin), std)
+        return (w, g.normal((cout,), bias_std)) if bias else w
+
+    def ln(n):
+        if perturb_ln:
+            return 1.0 + g.normal((n,), 0.1), g.normal((n,), 0.1)
+        return np.ones(n, np.float32), np.zeros(n, np.float32)
+
+    mha = {}
+    mha["q_w"], mha["q_b"] = fc(d_model, emb)
+    mha["k_w"], mha["k_b"] = fc(d_model, emb)
+    mha["v_w"], mha["v_b"] = fc(d_model, emb)
+    mha["dense_w"], mha["dense_b"] = fc(emb, d_model)
+    if smolgen:
+        hc, hs, gsz = smolgen
+        sg = {"compress": fc(hc, emb, bias=False)}
+        sg["dense1_w"], sg["dense1_b"] = fc(hs, 64 * hc)
+        sg["ln1_gammas"], sg["ln1_betas"] = ln(hs)
+        sg["dense2_w"], sg["dense2_b"] = fc(heads * gsz, hs)
+        sg["ln2_gammas"], sg["ln2_betas"] = ln(heads * gsz)
+        mha["smolgen"] = sg
+    layer = {"mha": mha}
+    layer["ln1_gammas"], layer["ln1_betas"] = ln(emb)
+    ffn = {}
+    ffn["dense1_w"], ffn["dense1_b"] = fc(dff, emb)
+    ffn["dense2_w"], ffn["dense2_b"] = fc(emb, dff)
+    layer["ffn"] = ffn
+    layer["ln2_gammas"], layer["ln2_betas"] = ln(emb)
+    return layer
+
+
 def se_resnet(filters, blocks, se_channels, seed, policy_channels=32, value_channels=32,
-              value_fc=128, bias_std=0.02, moves_left=False, conv_policy=False):
-    """Classical SE-ResNet: weights N(0, 1/fan_in) (std = fan_in**-0.5)."""
+              value_fc=128, bias_std=0.02, moves_left=False, conv_policy=False, attn_policy=None):
+    """Classical SE-ResNet: weights N(0, 1/fan_in) (std = fan_in**-0.5).
+
+    attn_policy = (embedding, d_model, encoder_layers, encoder_heads, encoder_dff): attention policy
+    head on the convolutional body (the "apmish" family, network_blas.cc:806-842)."""
     g = _Gen(seed)
 
     def conv(cout, cin, k):
@@ -57,7 +94,16 @@ def se_resnet(filters, blocks, se_channels, seed, policy_channels=32, value_chan
             w2, b2 = fc(2 * filters, se_channels)
             blk["se"] = {"w1": w1, "b1": b1, "w2": w2, "b2": b2}
         w["residual"].append(blk)
-    if conv_policy:
+    if attn_policy:
+        pe, pd, n_enc, enc_heads, enc_dff = attn_policy
+        w["ip_pol_w"], w["ip_pol_b"] = fc(pe, filters)
+        w["pol_encoder"] = [_encoder_layer(g, pe, pe, enc_dff, pe ** -0.5, bias_std, perturb_ln=True)
+                            for _ in range(n_enc)]
+        w["pol_headcount"] = enc_heads
+        w["ip2_pol_w"], w["ip2_pol_b"] = fc(pd, pe)
+        w["ip3_pol_w"], w["ip3_pol_b"] = fc(pd, pe)
+        w["ip4_pol_w"] = g.normal((4, pd), pd ** -0.5)
+    elif conv_policy:
         w["policy1"] = conv(filters, filters, 3)
         w["policy"] = conv(80, filters, 3)
     else:
@@ -72,7 +118,7 @@ def se_resnet(filters, blocks, se_channels, seed, policy_channels=32, value_chan
         w["ip2_mov_w"], w["ip2_mov_b"] = fc(1, value_fc)
     nf = {"input": INPUT_CLASSICAL_112_PLANE, "output": OUTPUT_WDL,
           "network": NETWORK_SE_WITH_HEADFORMAT,
-          "policy": POLICY_CONVOLUTION if conv_policy else POLICY_CLASSICAL,
+          "policy": POLICY_ATTENTION if attn_policy else POLICY_CONVOLUTION if conv_policy else POLICY_CLASSICAL,
           "value": VALUE_WDL,
           "moves_left": MOVES_LEFT_V1 if moves_left else MOVES_LEFT_NONE,
           "default_activation": DEFAULT_ACTIVATION_RELU}
@@ -81,7 +127,7 @@ def se_resnet(filters, blocks, se_channels, seed, policy_channels=32, value_chan
 
 def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_std=0.02,
                    policy_d=None, value_channels=32, value_fc=128, mlh_channels=32, mlh_fc=128,
-                   perturb_ln=False, pe_dense=None, gating=False, multihead=False):
+                   perturb_ln=False, pe_dense=None, gating=False, multihead=False, d_model=None, pol_encoder=None):
     """Attention-body net (attention policy, WDL, MLH).
 
     smolgen = (hidden_channels, hidden_sz, gen_sz) or None. Weights N(0, std),
@@ -90,9 +136,10 @@ def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_s
     embedding FFN (src/neural/backends/blas/network_blas.cc:612-712) instead of PE_MAP.
     gating: ip_mult_gate / ip_add_gate. multihead: network format 7 with policy heads
     vanilla / optimistic_st / soft (shared embedding) and value heads winner / q / st.
+    pol_encoder = (layers, heads, dff): encoder layers inside the policy head (legacy format only).
     """
     g = _Gen(seed)
-    d_model = emb
+    d_model = d_model or emb          # heads * head depth
     policy_d = policy_d or emb
 
     def fc(cout, cin, bias=True):
@@ -119,29 +166,8 @@ def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_s
     if gating:
         w["ip_mult_gate"] = 1.0 + g.normal((emb * 64,), 0.1)
         w["ip_add_gate"] = g.normal((emb * 64,), 0.1)
-    w["encoder"] = []
-    for _ in range(layers):
-        mha = {}
-        mha["q_w"], mha["q_b"] = fc(d_model, emb)
-        mha["k_w"], mha["k_b"] = fc(d_model, emb)
-        mha["v_w"], mha["v_b"] = fc(d_model, emb)
-        mha["dense_w"], mha["dense_b"] = fc(emb, d_model)
-        if smolgen:
-            hc, hs, gsz = smolgen
-            sg = {"compress": fc(hc, emb, bias=False)}
-            sg["dense1_w"], sg["dense1_b"] = fc(hs, 64 * hc)
-            sg["ln1_gammas"], sg["ln1_betas"] = ln(hs)
-            sg["dense2_w"], sg["dense2_b"] = fc(heads * gsz, hs)
-            sg["ln2_gammas"], sg["ln2_betas"] = ln(heads * gsz)
-            mha["smolgen"] = sg
-        layer = {"mha": mha}
-        layer["ln1_gammas"], layer["ln1_betas"] = ln(emb)
-        ffn = {}
-        ffn["dense1_w"], ffn["dense1_b"] = fc(dff, emb)
-        ffn["dense2_w"], ffn["dense2_b"] = fc(emb, dff)
-        layer["ffn"] = ffn
-        layer["ln2_gammas"], layer["ln2_betas"] = ln(emb)
-        w["encoder"].append(layer)
+    w["encoder"] = [_encoder_layer(g, emb, d_model, dff, std, bias_std, smolgen=smolgen, heads=heads,
+                                   perturb_ln=perturb_ln) for _ in range(layers)]
     w["headcount"] = heads
 
     def policy_head():
@@ -167,6 +193,11 @@ def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_s
         w["value_heads"] = {name: value_head() for name in ("winner", "q", "st")}
     else:
         w["ip_pol_w"], w["ip_pol_b"] = fc(policy_d, emb)
+        if pol_encoder:
+            n_enc, enc_heads, enc_dff = pol_encoder
+            w["pol_encoder"] = [_encoder_layer(g, policy_d, policy_d, enc_dff, std, bias_std, perturb_ln=perturb_ln)
+                                for _ in range(n_enc)]
+            w["pol_headcount"] = enc_heads
         w.update(policy_head())
         w.update(value_head())
     w["ip_mov_w"], w["ip_mov_b"] = fc(mlh_channels, emb)
@@ -210,12 +241,17 @@ CONFIGS = {
     # BT4 as published: 15 layers, d=1024, 32 heads, dff 1536, smolgen, PE_DENSE (64 channels, FFN 1536), multi-head
     "bt4_dense_15x1024": lambda: attention_body(1024, 15, 32, 1536, seed=1004, smolgen=(32, 256, 256),
                                                 pe_dense=(64, 1536), multihead=True),
+    # head depth 64 (d_model 128 over 2 heads) and two encoder layers inside the policy head
+    "tiny_attn_d64": lambda: attention_body(128, 2, 2, 128, seed=2007, smolgen=(8, 32, 32), perturb_ln=True, std=0.07,
+                                            pol_encoder=(2, 4, 96)),
+    # convolutional body with the attention policy head and one policy encoder layer
+    "tiny_resnet_attnpolicy": lambda: se_resnet(32, 2, 8, seed=2008, attn_policy=(64, 64, 1, 2, 96)),
     "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True, std=0.1),
 }
 
 
 # Part of the cache file name: bump when a generator or a configuration changes.
-CACHE_VERSION = "-g2"
+CACHE_VERSION = "-g3"
 
 
 def write_config(name, path):

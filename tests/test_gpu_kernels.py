@@ -296,3 +296,21 @@ def test_attention_f8_output_matches_half_output():
     half_out = K.attention(qkv, bias, batch, heads, 32 ** -0.5).astype(f32)
     got = K.attention_f8(qkv, bias, batch, heads, 32 ** -0.5, 100.0)
     _f8_close(got, half_out, 100.0)   # same fp32 result, rounded to e4m3 instead of fp16 (fp16 error << e4m3 step)
+
+
+@pytest.mark.parametrize("depth", [64, 128])
+def test_attention_head_depths(depth):
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(depth)
+    batch, heads = 3, 3
+    d = heads * depth
+    qkv = _h(rng.standard_normal((batch * 64, 3 * d)))
+    bias = _h(rng.standard_normal((batch, heads, 64, 64)))
+    scale = 1.0 / np.sqrt(float(depth))
+    got = K.attention(qkv, bias, batch, heads, scale, depth=depth).astype(f32)
+    q = qkv[:, :d].reshape(batch, 64, heads, depth).transpose(0, 2, 1, 3)
+    k = qkv[:, d:2 * d].reshape(batch, 64, heads, depth).transpose(0, 2, 1, 3)
+    v = qkv[:, 2 * d:].reshape(batch, 64, heads, depth).transpose(0, 2, 1, 3)
+    p = onn.softmax_rows(bias + np.matmul(q, k.transpose(0, 1, 3, 2)) * f32(scale))
+    want = np.matmul(p, v).transpose(0, 2, 1, 3).reshape(batch * 64, d)
+    np.testing.assert_allclose(got, want, rtol=4e-3, atol=4e-3)

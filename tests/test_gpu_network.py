@@ -402,3 +402,21 @@ def test_concurrent_computations_from_several_threads(name, options, positions):
     for key, w in want.items():
         for field in ("policy", "q", "d", "m"):
             np.testing.assert_array_equal(got[key][field], w[field])
+
+
+@pytest.mark.parametrize("name,batch", [("tiny_attn_d64", 40), ("tiny_resnet_attnpolicy", 33)])
+def test_head_depth_64_policy_encoders_and_attention_policy_on_a_tower(name, batch, positions):
+    """tiny_attn_d64: attention heads of depth 64 and two encoder layers inside the policy head
+    (network_blas.cc:836-842). tiny_resnet_attnpolicy: attention policy head with one policy encoder
+    on a convolutional body, SELU on the embedding and in the encoder FFN (network_blas.cc:806-842)."""
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    _, res = _run_gpu(path, masks, values)
+    _compare(res, want, positions["legal"][:batch])
+
+
+def test_attention_policy_on_a_tower_needs_fp16():
+    from lc0_amd import BackendError, Network
+    with pytest.raises(BackendError, match="precision=fp16"):
+        Network(netgen.cached_config("tiny_resnet_attnpolicy"), "precision=fp32")
