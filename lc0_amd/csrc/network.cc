@@ -332,6 +332,13 @@ class Mi355xNetwork : public Network, protected ModelState {
   void CalibrateExclusive(int n, const uint64_t* masks, const float* values);
   void DefaultCalibration();
   float* UploadF(const Vec& v) { return arena_.Upload(v); }
+  // Uploads a per-channel parameter vector after checking its length.
+  float* UploadN(const Vec& v, int n, const char* what) {
+    if (static_cast<int>(v.size()) != n) {
+      throw Error(std::string(what) + " has " + std::to_string(v.size()) + " elements, expected " + std::to_string(n) + ".");
+    }
+    return arena_.Upload(v);
+  }
   half_t* AllocH(size_t n) { return static_cast<half_t*>(arena_.Alloc(n * sizeof(half_t))); }
   float* AllocF(size_t n) { return static_cast<float*>(arena_.Alloc(n * sizeof(float))); }
 
@@ -881,11 +888,8 @@ EncoderDev Mi355xNetwork::MakeEncoderLayer(const EncoderLayer& l, int emb, int d
   e.dense = MakeLinear(l.mha.dense_w, l.mha.dense_b, emb, d_model);
   e.ffn1 = MakeLinear(l.ffn.dense1_w, l.ffn.dense1_b, dff, emb);
   e.ffn2 = MakeLinear(l.ffn.dense2_w, l.ffn.dense2_b, emb, dff);
-  if (static_cast<int>(l.ln1_gammas.size()) != emb || static_cast<int>(l.ln2_gammas.size()) != emb) {
-    throw Error("Layer norm parameters do not match the embedding size.");
-  }
-  e.ln1_g = UploadF(l.ln1_gammas); e.ln1_b = UploadF(l.ln1_betas);
-  e.ln2_g = UploadF(l.ln2_gammas); e.ln2_b = UploadF(l.ln2_betas);
+  e.ln1_g = UploadN(l.ln1_gammas, emb, "Encoder layer norm gamma"); e.ln1_b = UploadN(l.ln1_betas, emb, "Encoder layer norm beta");
+  e.ln2_g = UploadN(l.ln2_gammas, emb, "Encoder layer norm gamma"); e.ln2_b = UploadN(l.ln2_betas, emb, "Encoder layer norm beta");
   return e;
 }
 
@@ -997,13 +1001,15 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     if (static_cast<int>(w.ip_emb_ln_gammas.size()) != emb_ || static_cast<int>(w.ip_emb_ln_betas.size()) != emb_) {
       throw Error("Embedding layer norm parameters do not match the embedding size.");
     }
-    emb_ln_g_ = UploadF(w.ip_emb_ln_gammas); emb_ln_b_ = UploadF(w.ip_emb_ln_betas);
+    emb_ln_g_ = UploadN(w.ip_emb_ln_gammas, emb_, "Embedding layer norm gamma");
+    emb_ln_b_ = UploadN(w.ip_emb_ln_betas, emb_, "Embedding layer norm beta");
     emb_dff_ = static_cast<int>(w.ip_emb_ffn.dense1_b.size());
     if (emb_dff_ <= 0 || emb_dff_ % 8) throw Error("Embedding FFN width must be a positive multiple of 8.");
     emb_ffn1_ = MakeLinear(w.ip_emb_ffn.dense1_w, w.ip_emb_ffn.dense1_b, emb_dff_, emb_);
     emb_ffn2_ = MakeLinear(w.ip_emb_ffn.dense2_w, w.ip_emb_ffn.dense2_b, emb_, emb_dff_);
     if (static_cast<int>(w.ip_emb_ffn_ln_gammas.size()) != emb_) throw Error("Embedding FFN layer norm has a wrong size.");
-    emb_ffn_ln_g_ = UploadF(w.ip_emb_ffn_ln_gammas); emb_ffn_ln_b_ = UploadF(w.ip_emb_ffn_ln_betas);
+    emb_ffn_ln_g_ = UploadN(w.ip_emb_ffn_ln_gammas, emb_, "Embedding FFN layer norm gamma");
+    emb_ffn_ln_b_ = UploadN(w.ip_emb_ffn_ln_betas, emb_, "Embedding FFN layer norm beta");
   } else {
     emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + 64);
   }
@@ -1050,8 +1056,8 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
       e.ffn18 = MakeLinearF8(l.ffn.dense1_w, dff_, emb_);
       e.ffn28 = MakeLinearF8(l.ffn.dense2_w, emb_, dff_);
     }
-    e.ln1_g = UploadF(l.ln1_gammas); e.ln1_b = UploadF(l.ln1_betas);
-    e.ln2_g = UploadF(l.ln2_gammas); e.ln2_b = UploadF(l.ln2_betas);
+    e.ln1_g = UploadN(l.ln1_gammas, emb_, "Encoder layer norm gamma"); e.ln1_b = UploadN(l.ln1_betas, emb_, "Encoder layer norm beta");
+    e.ln2_g = UploadN(l.ln2_gammas, emb_, "Encoder layer norm gamma"); e.ln2_b = UploadN(l.ln2_betas, emb_, "Encoder layer norm beta");
     if (static_cast<int>(l.ln1_gammas.size()) != emb_ || static_cast<int>(l.ln2_gammas.size()) != emb_) {
       throw Error("Layer norm parameters do not match the embedding size.");
     }
@@ -1073,8 +1079,8 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
       e.sg_compress = MakeLinear(s.compress, Vec(), hc, emb_);
       e.sg_dense1 = MakeLinear(s.dense1_w, s.dense1_b, hs, 64 * hc);
       e.sg_dense2 = MakeLinear(s.dense2_w, s.dense2_b, gen, hs);
-      e.sg_ln1_g = UploadF(s.ln1_gammas); e.sg_ln1_b = UploadF(s.ln1_betas);
-      e.sg_ln2_g = UploadF(s.ln2_gammas); e.sg_ln2_b = UploadF(s.ln2_betas);
+      e.sg_ln1_g = UploadN(s.ln1_gammas, hs, "Smolgen layer norm gamma"); e.sg_ln1_b = UploadN(s.ln1_betas, hs, "Smolgen layer norm beta");
+      e.sg_ln2_g = UploadN(s.ln2_gammas, gen, "Smolgen layer norm gamma"); e.sg_ln2_b = UploadN(s.ln2_betas, gen, "Smolgen layer norm beta");
     }
     encoders_.push_back(e);
   }

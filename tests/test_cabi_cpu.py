@@ -105,3 +105,37 @@ def test_null_arguments_are_rejected():
     assert lib.lc0mi_comp_batch_size(None) == 0
     lib.lc0mi_comp_q.restype = ctypes.c_float
     assert np.isnan(lib.lc0mi_comp_q(None, 0))
+
+
+def test_mutated_weight_files_never_crash_the_loader():
+    """Robustness of the wire reader: random byte flips, truncations and length-field corruption of a
+    valid net must end in an error return (a parse error, or "No HIP device" when the bytes still
+    parse), never in a crash or a hang. Runs without a GPU."""
+    import ctypes as C
+    import numpy as np
+    from lc0_amd import netgen, netproto
+    from lc0_amd.backend import load_library
+    lib = load_library()
+    raw = bytearray(netproto.serialize_net(netgen.CONFIGS["tiny_attn"]()))
+    rng = np.random.default_rng(123)
+    seen = set()
+    for trial in range(400):
+        data = bytearray(raw)
+        kind = trial % 4
+        if kind == 0:      # flip a few bytes anywhere
+            for pos in rng.integers(0, len(data), 4):
+                data[pos] ^= int(rng.integers(1, 256))
+        elif kind == 1:    # truncate
+            data = data[:int(rng.integers(0, len(data)))]
+        elif kind == 2:    # corrupt bytes near the start (tags and lengths of the outer messages)
+            for pos in rng.integers(0, 64, 3):
+                data[pos] = int(rng.integers(0, 256))
+        else:              # splice a random chunk somewhere
+            pos = int(rng.integers(0, len(data)))
+            data[pos:pos] = bytes(rng.integers(0, 256, int(rng.integers(1, 40)), dtype=np.uint8))
+        buf = (C.c_char * len(data)).from_buffer(data) if len(data) else None
+        net = C.c_void_p()
+        rc = lib.lc0mi_net_create_from_buffer(buf, len(data), b"", C.byref(net))
+        assert rc != 0 and not net.value
+        seen.add(lib.lc0mi_last_error().decode(errors="replace")[:40])
+    assert len(seen) >= 3, seen      # several distinct failure paths were exercised

@@ -420,3 +420,42 @@ def test_attention_policy_on_a_tower_needs_fp16():
     from lc0_amd import BackendError, Network
     with pytest.raises(BackendError, match="precision=fp16"):
         Network(netgen.cached_config("tiny_resnet_attnpolicy"), "precision=fp32")
+
+
+@pytest.mark.parametrize("name", ["tiny_attn", "tiny_attn_d64", "tiny_resnet", "tiny_resnet_convpolicy",
+                                  "tiny_resnet_attnpolicy"])
+def test_every_resized_tensor_is_rejected_at_load(name):
+    """Size validation: a net in which any one tensor has a few elements too many or too few must be
+    refused when the network is built (no kernel ever runs on inconsistent shapes)."""
+    from lc0_amd import BackendError, Network, netproto
+
+    def leaves(node, path=()):
+        if isinstance(node, dict):
+            for k, v in node.items():
+                yield from leaves(v, path + (k,))
+        elif isinstance(node, list):
+            for i, v in enumerate(node):
+                yield from leaves(v, path + (i,))
+        elif isinstance(node, np.ndarray):
+            yield path
+
+    base = netgen.CONFIGS[name]()
+    paths = list(leaves(base["weights"]))
+    rng = np.random.default_rng(11)
+    accepted = []
+    for path in paths:
+        net = netgen.CONFIGS[name]()
+        node = net["weights"]
+        for key in path[:-1]:
+            node = node[key]
+        flat = node[path[-1]].reshape(-1)
+        delta = int(rng.choice([-8, -1, 1, 8]))
+        if flat.size + delta <= 0:
+            delta = 1          # an absent bias is a valid "no bias" layer, not a size error
+        node[path[-1]] = np.concatenate([flat, np.zeros(delta, np.float32)]) if delta > 0 else flat[:delta]
+        try:
+            Network(netproto.serialize_net(net), "max_batch=8,lanes=1")
+            accepted.append(path)
+        except BackendError:
+            pass
+    assert not accepted, accepted
