@@ -506,29 +506,40 @@ void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
 }  // namespace
 
 namespace {
-enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64 };
+enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128 };
 
 int g_variant_override = -1;
 
 GemmVariant PickGemmVariant(const GemmArgs& a) {
   if (g_variant_override >= 0) {
     const bool dma_ok = !a.out_f32 && a.split_k == 1 && a.K % 64 == 0;
-    if (g_variant_override >= kTile128 || dma_ok) return static_cast<GemmVariant>(g_variant_override);
+    const bool is_dma = g_variant_override <= kDma256x128 || g_variant_override == kDma128x128;
+    if (!is_dma || dma_ok) return static_cast<GemmVariant>(g_variant_override);
   }
-  const long long tiles256 = (long long)((a.M + 255) / 256) * ((a.N + 255) / 256) * a.batch;
-  const long long big_tiles = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
-  if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= 128 && a.N >= 192 && tiles256 >= 128) {
-    // One workgroup per CU at a time: time ~ rounds over 256 CUs x tile width,
-    // with a small efficiency penalty for the narrower tiles.
-    const long long m_tiles = (a.M + 255) / 256;
-    auto cost = [&](int bn, double penalty) {
-      const long long tiles = m_tiles * ((a.N + bn - 1) / bn) * a.batch;
-      return (double)((tiles + 255) / 256) * bn * penalty;
+  const long long tiles128 = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
+  if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= 128 && a.N >= 128 && a.M >= 1024 && tiles128 >= 64) {
+    // Direct-to-LDS kernels. Cost = rounds over the 256 CUs x tile area x a measured cost per
+    // output element and round (ns per element at K = 1024): 0.60 for 256x256, 0.61 for 256x192;
+    // the two small shapes run two workgroups per CU, 0.68 (256x128) and 0.75 (128x128) per element
+    // while sharing a CU, 0.84 and 0.95 when a single round leaves every workgroup alone on its CU.
+    auto rounds = [&](int bm, int bn) {
+      const long long tiles = (long long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * a.batch;
+      return (double)((tiles + 255) / 256);
     };
-    const double c256 = cost(256, 1.0), c192 = cost(192, 1.04), c128 = cost(128, 1.15);
-    if (c256 <= c192 && c256 <= c128) return kDma256x256;
-    return c192 <= c128 ? kDma256x192 : kDma256x128;
+    const double r256 = rounds(256, 256), r192 = rounds(256, 192), r128 = rounds(256, 128), rs = rounds(128, 128);
+    const double c256 = r256 * 256 * 256 * 0.60;
+    const double c192 = r192 * 256 * 192 * 0.61;
+    const double c128 = r128 * 256 * 128 * (r128 > 1 ? 0.68 : 0.84);
+    // (short reductions are dominated by the epilogue, where the smallest tile loses a little more)
+    const double cs = rs * 128 * 128 * (rs > 1 ? 0.75 : 0.95) * (a.K <= 256 ? 1.12 : 1.0);
+    GemmVariant best = kDma256x256;
+    double cost = c256;
+    if (c192 < cost) { best = kDma256x192; cost = c192; }
+    if (c128 < cost) { best = kDma256x128; cost = c128; }
+    if (cs < cost) { best = kDma128x128; cost = cs; }
+    return best;
   }
+  const long long big_tiles = tiles128;
   return big_tiles >= 192 ? kTile128 : kTile64;
 }
 }  // namespace
@@ -540,6 +551,7 @@ const char* GemmVariantName(const GemmArgs& a) {
     case kDma256x256: return "gemm_dma_256x256x64";
     case kDma256x192: return "gemm_dma_256x192x64";
     case kDma256x128: return "gemm_dma_256x128x32";
+    case kDma128x128: return "gemm_dma_128x128x64";
     case kTile128: return "gemm_128x128x64";
     default: return a.split_k > 1 ? "gemm_64x64x64_splitk" : "gemm_64x64x64";
   }
@@ -551,23 +563,32 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
     case kDma256x256: LaunchGemmDma<256, 256, 64, 2, 4>(a, stream); break;
     case kDma256x192: LaunchGemmDma<256, 192, 64, 4, 2>(a, stream); break;
     case kDma256x128: LaunchGemmDma<256, 128, 32, 4, 2>(a, stream); break;
+    case kDma128x128: LaunchGemmDma<128, 128, 64, 2, 2>(a, stream); break;
     case kTile128: LaunchGemmTile<128, 128, 64, 2, 2>(a, stream); break;
     default: LaunchGemmTile<64, 64, 64, 2, 2>(a, stream); break;
   }
 }
 
 namespace {
-// 0: 256x256, 1: 256x192, 2: 256x128 (fewest rounds over the 256 CUs, as for fp16).
+// 0: 256x256, 1: 256x192, 2: 256x128, 5: 128x128 with 4 waves (two workgroups per CU); chosen by
+// the cost model of the fp16 kernels (the k-tile structure is the same).
 int PickGemmF8Variant(const GemmF8Args& a) {
-  if (g_variant_override >= 0 && g_variant_override <= 2) return g_variant_override;
-  const long long m_tiles = (a.M + 255) / 256;
-  auto cost = [&](int bn, double penalty) {
-    const long long tiles = m_tiles * ((a.N + bn - 1) / bn);
-    return (double)((tiles + 255) / 256) * bn * penalty;
+  if (g_variant_override >= 0 && (g_variant_override <= 2 || g_variant_override == kDma128x128)) return g_variant_override;
+  auto rounds = [&](int bm, int bn) {
+    const long long tiles = (long long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn);
+    return (double)((tiles + 255) / 256);
   };
-  const double c256 = cost(256, 1.0), c192 = cost(192, 1.04), c128 = cost(128, 1.15);
-  if (c256 <= c192 && c256 <= c128) return 0;
-  return c192 <= c128 ? 1 : 2;
+  const double r128 = rounds(256, 128), rs = rounds(128, 128);
+  const double c256 = rounds(256, 256) * 256 * 256 * 0.60;
+  const double c192 = rounds(256, 192) * 256 * 192 * 0.61;
+  const double c128 = r128 * 256 * 128 * 0.84;   // 96 KiB of LDS: one workgroup per CU
+  const double cs = rs * 128 * 128 * (rs > 1 ? 0.75 : 0.95);
+  int best = 0;
+  double cost = c256;
+  if (c192 < cost) { best = 1; cost = c192; }
+  if (c128 < cost) { best = 2; cost = c128; }
+  if (cs < cost) { best = kDma128x128; cost = cs; }
+  return best;
 }
 }  // namespace
 
@@ -575,7 +596,8 @@ const char* GemmF8VariantName(const GemmF8Args& a) {
   switch (PickGemmF8Variant(a)) {
     case 0: return "gemm_f8_256x256x128";
     case 1: return "gemm_f8_256x192x128";
-    default: return "gemm_f8_256x128x128";
+    case 2: return "gemm_f8_256x128x128";
+    default: return "gemm_f8_128x128x128";
   }
 }
 
@@ -584,7 +606,8 @@ void LaunchGemmF8(const GemmF8Args& a, hipStream_t stream) {
   switch (PickGemmF8Variant(a)) {
     case 0: LaunchGemmDmaF8<256, 256, 2, 4>(a, stream); break;
     case 1: LaunchGemmDmaF8<256, 192, 4, 2>(a, stream); break;
-    default: LaunchGemmDmaF8<256, 128, 4, 2>(a, stream); break;
+    case 2: LaunchGemmDmaF8<256, 128, 4, 2>(a, stream); break;
+    default: LaunchGemmDmaF8<128, 128, 2, 2>(a, stream); break;
   }
 }
 
