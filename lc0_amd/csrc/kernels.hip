@@ -241,6 +241,94 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 }
 
 // ---------------------------------------------------------------------------
+// Row-panel GEMM for small problems (few rows, or few columns): a workgroup owns a
+// 64 x 32 output panel and its eight waves split the reduction dimension, so even
+// a 64 x 32 x K problem keeps eight waves busy, the serial chain is K / 128 MFMA
+// steps instead of K / 16, and up to eight steps of operand loads are in flight per
+// wave (these problems are bound by memory latency, not by arithmetic). Fragments go
+// from global memory straight into registers; the eight partial sums are added in
+// wave order through LDS, so results do not depend on timing.
+// ---------------------------------------------------------------------------
+template <typename OutT>
+__global__ __launch_bounds__(512) void gemm_rowpanel_kernel(GemmArgs p) {
+  constexpr int NW = 8;
+  __shared__ float part[NW][64 * 33];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, g = lane >> 5;
+  const int m0 = blockIdx.x * 64, n0 = blockIdx.y * 32;
+  const int M = p.M, N = p.N, K = p.K;
+  const half_t* A = p.A + (long long)blockIdx.z * p.strideA;
+  const half_t* W = p.W + (long long)blockIdx.z * p.strideW;
+  // K range of this wave, in steps of 16.
+  const int steps = (K + 15) / 16;
+  const int per_wave = (steps + NW - 1) / NW;
+  const int s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
+  const half_t* a0 = A + (long long)min(m0 + r, M - 1) * p.lda + 8 * g;
+  const half_t* a1 = A + (long long)min(m0 + 32 + r, M - 1) * p.lda + 8 * g;
+  const half_t* w0 = W + (long long)min(n0 + r, N - 1) * p.ldw + 8 * g;
+  floatx16 acc0, acc1;
+#pragma unroll
+  for (int e = 0; e < 16; e++) acc0[e] = acc1[e] = 0.0f;
+  // All steps but a possible half-step at the very end of K are loaded without a
+  // predicate, so that the compiler can put the loads of eight steps in flight at once.
+  const int full_end = (K % 16 == 0) ? s_end : min(s_end, steps - 1);
+  for (int st = s_begin; st < full_end; st += 8) {
+    half8 fa0[8], fa1[8], fw[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {   // steps past the end re-read the last one (never used)
+      const int k = min(st + u, full_end - 1) * 16;
+      fa0[u] = *reinterpret_cast<const half8*>(a0 + k);
+      fa1[u] = *reinterpret_cast<const half8*>(a1 + k);
+      fw[u] = *reinterpret_cast<const half8*>(w0 + k);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      if (st + u < full_end) {
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[u], fa0[u], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[u], fa1[u], acc1, 0, 0, 0);
+      }
+    }
+  }
+  if (s_end > full_end && s_end > s_begin) {   // K is a multiple of 8: the upper half of the last step is zero-filled
+    const int k = (steps - 1) * 16;
+    const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bool in = g == 0;
+    const half8 fa0 = in ? *reinterpret_cast<const half8*>(a0 + k) : zero;
+    const half8 fa1 = in ? *reinterpret_cast<const half8*>(a1 + k) : zero;
+    const half8 fw = in ? *reinterpret_cast<const half8*>(w0 + k) : zero;
+    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw, fa0, acc0, 0, 0, 0);
+    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw, fa1, acc1, 0, 0, 0);
+  }
+  // Accumulator lane (r, g) holds rows m = r (+32), columns n = 8 blk + 4 g + j.
+  float* mine = part[wave];
+#pragma unroll
+  for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int n = 8 * blk + 4 * g + j;
+      mine[r * 33 + n] = acc0[blk * 4 + j];
+      mine[(32 + r) * 33 + n] = acc1[blk * 4 + j];
+    }
+  __syncthreads();
+  OutT* C = reinterpret_cast<OutT*>(p.C) + (long long)blockIdx.z * p.strideC;
+  DispatchAct(p.act, [&](auto act_fn) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int idx = tid + 512 * i;        // 64 x 32 outputs, consecutive threads along n
+      const int row = idx >> 5, col = idx & 31;
+      const int m = m0 + row, n = n0 + col;
+      if (m < M && n < N) {
+        float sum = part[0][row * 33 + col];
+#pragma unroll
+        for (int w = 1; w < NW; w++) sum += part[w][row * 33 + col];
+        const float v = act_fn(sum * p.scale + (p.bias ? p.bias[n] : 0.0f));
+        C[(long long)m * p.ldc + n] = (OutT)v;
+      }
+    }
+  });
+}
+
+// ---------------------------------------------------------------------------
 // Large-shape GEMM: same contract as gemm_kernel for K % BK == 0 and half output.
 //
 // Operand tiles travel from global memory straight into LDS (16 bytes per lane,
@@ -506,7 +594,7 @@ void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
 }  // namespace
 
 namespace {
-enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128 };
+enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128, kRowPanel };
 
 int g_variant_override = -1;
 
@@ -514,7 +602,8 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
   if (g_variant_override >= 0) {
     const bool dma_ok = !a.out_f32 && a.split_k == 1 && a.K % 64 == 0;
     const bool is_dma = g_variant_override <= kDma256x128 || g_variant_override == kDma128x128;
-    if (!is_dma || dma_ok) return static_cast<GemmVariant>(g_variant_override);
+    const bool ok = is_dma ? dma_ok : (g_variant_override != kRowPanel || a.split_k == 1);
+    if (ok) return static_cast<GemmVariant>(g_variant_override);
   }
   const long long tiles128 = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
   if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= 128 && a.N >= 128 && a.M >= 1024 && tiles128 >= 64) {
@@ -539,6 +628,12 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
     if (cs < cost) { best = kDma128x128; cost = cs; }
     return best;
   }
+  // Small problems with a long reduction: the 64x64 kernel walks K serially in one workgroup;
+  // when it would start at most 64 workgroups, the row-panel kernel (8-way K split inside the
+  // workgroup, 64x32 panels) is faster (64x3072x1024: 8.5 vs 9.7 us; 8192x32x1024: 9.2 vs 11.9 us).
+  // With a short K and many columns it loses (128x8192x256: 15.8 vs 5.6 us).
+  const long long tiles64 = (long long)((a.M + 63) / 64) * ((a.N + 63) / 64) * a.batch;
+  if (a.split_k == 1 && tiles64 <= 64 && a.K >= 512) return kRowPanel;
   const long long big_tiles = tiles128;
   return big_tiles >= 192 ? kTile128 : kTile64;
 }
@@ -552,6 +647,7 @@ const char* GemmVariantName(const GemmArgs& a) {
     case kDma256x192: return "gemm_dma_256x192x64";
     case kDma256x128: return "gemm_dma_256x128x32";
     case kDma128x128: return "gemm_dma_128x128x64";
+    case kRowPanel: return "gemm_rowpanel_64x32";
     case kTile128: return "gemm_128x128x64";
     default: return a.split_k > 1 ? "gemm_64x64x64_splitk" : "gemm_64x64x64";
   }
@@ -564,6 +660,15 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
     case kDma256x192: LaunchGemmDma<256, 192, 64, 4, 2>(a, stream); break;
     case kDma256x128: LaunchGemmDma<256, 128, 32, 4, 2>(a, stream); break;
     case kDma128x128: LaunchGemmDma<128, 128, 64, 2, 2>(a, stream); break;
+    case kRowPanel: {
+      dim3 grid((a.M + 63) / 64, (a.N + 31) / 32, a.batch);
+      if (a.out_f32) {
+        hipLaunchKernelGGL(gemm_rowpanel_kernel<float>, grid, dim3(512), 0, stream, a);
+      } else {
+        hipLaunchKernelGGL(gemm_rowpanel_kernel<half_t>, grid, dim3(512), 0, stream, a);
+      }
+      break;
+    }
     case kTile128: LaunchGemmTile<128, 128, 64, 2, 2>(a, stream); break;
     default: LaunchGemmTile<64, 64, 64, 2, 2>(a, stream); break;
   }
