@@ -281,8 +281,11 @@ def test_bt4_shape_fp8_batch_sweep(positions):
         assert np.isfinite(r["policy"]).all()
         k = min(n, 64)
         # other batch sizes may pick other GEMM tiles (summation order), then e4m3 rounding
-        # of activations amplifies the difference: equal to the fp8 noise level, not bitwise
-        np.testing.assert_allclose(r["policy"][:k], res["policy"][:k], rtol=0, atol=4 * s["logit_rms"] + 5e-3)
+        # of activations amplifies the difference: two evaluations differ like two independent
+        # draws of the fp8 noise (rms bound), with a tail over ~1e5 logits (max bound)
+        diff = r["policy"][:k] - res["policy"][:k]
+        assert np.sqrt(np.mean(diff * diff)) <= 2 * s["logit_rms"]
+        assert np.abs(diff).max() <= 10 * s["logit_rms"] + 5e-3
         np.testing.assert_allclose(r["q"][:k], res["q"][:k], rtol=0, atol=1e-2)
 
 
