@@ -63,10 +63,14 @@ int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const 
  * (WinogradConvolution3::Forward + BiasActivate / BiasResidual / ApplySEUnit,
  *  src/neural/backends/blas/winograd_convolution3.cc:47-324, se_unit.cc:31-91).
  * x, skip, out: [B][64][C] floats (NHWC); filter: [cout][cin][3][3]; use_fp16 selects
- * the half-precision kernels (operands rounded to fp16 on the way in). */
+ * the half-precision kernels (operands rounded to fp16 on the way in).
+ * v_fused / v_separate (both or neither, [36][B*4][cout]): the transformed input of a following
+ * convolution, from the output transform kernel that fuses it and from the stand-alone input
+ * transform applied to `out`. */
 int lc0mi_k_winograd_conv(const float* x, const float* filter, const float* bias, const float* skip,
                           const float* se_w1, const float* se_b1, const float* se_w2, const float* se_b2, int se_k,
-                          int batch, int cin, int cout, int act, int use_fp16, float* out);
+                          int batch, int cin, int cout, int act, int use_fp16, float* out, float* v_fused,
+                          float* v_separate);
 /* e4m3 GEMM: C = act(col_scale[n] * A.W^T + bias[n]); A [M][lda], W [N][ldw] e4m3 bytes, K % 128 == 0.
  * out_f8 != 0: C receives e4m3(C * out_mul) bytes, else halves. Counterpart of FullyConnectedLayer::Forward1D
  * (src/neural/backends/blas/fully_connected_layer.cc:66-106) on quantised operands. */

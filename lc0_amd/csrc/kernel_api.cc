@@ -300,7 +300,7 @@ namespace {
 template <typename T>
 void WinogradConvHost(const float* x, const float* filter, const float* bias, const float* skip, const float* se_w1,
                       const float* se_b1, const float* se_w2, const float* se_b2, int se_k, int batch, int cin,
-                      int cout, int act, float* out) {
+                      int cout, int act, float* out, float* v_fused, float* v_separate) {
   Dev dev;
   const int ld = (cin + 7) / 8 * 8;
   const size_t nx = (size_t)batch * 64 * cin, no = (size_t)batch * 64 * cout;
@@ -348,12 +348,30 @@ void WinogradConvHost(const float* x, const float* filter, const float* bias, co
     g.M = tiles; g.N = cout; g.K = ld; g.batch = 36;
     lc0mi::LaunchGemmF32(g, nullptr);
   }
-  lc0mi::LaunchWinogradOutputTransform<T, T>(dm, dbias, dskip, w1, b1, w2, b2, se_k, dout, batch, cout, act, nullptr);
+  // Optionally also the next convolution's transformed input, once from the fused kernel and
+  // once from the stand-alone input transform applied to the output (they must be identical).
+  T *dvf = nullptr, *dvs = nullptr;
+  const size_t nv = (size_t)36 * tiles * cout;
+  if (v_fused) {
+    if (cout % 8 || !lc0mi::WinogradFusedInputTransform(cout, sizeof(T), se_k)) throw Error("shape cannot be fused");
+    dvf = static_cast<T*>(dev.Alloc(sizeof(T) * nv));
+    dvs = static_cast<T*>(dev.Alloc(sizeof(T) * nv));
+  }
+  lc0mi::LaunchWinogradOutputTransform<T, T>(dm, dbias, dskip, w1, b1, w2, b2, se_k, dout, batch, cout, act, nullptr,
+                                             dvf, cout);
+  if (v_fused) lc0mi::LaunchWinogradInputTransform<T>(dout, dvs, batch, cout, cout, nullptr);
   K_CHECK(hipDeviceSynchronize());
   K_CHECK(hipGetLastError());
   std::vector<T> ho(no);
   K_CHECK(hipMemcpy(ho.data(), dout, sizeof(T) * no, hipMemcpyDeviceToHost));
   for (size_t i = 0; i < no; i++) out[i] = (float)ho[i];
+  if (v_fused) {
+    std::vector<T> hv(nv);
+    K_CHECK(hipMemcpy(hv.data(), dvf, sizeof(T) * nv, hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < nv; i++) v_fused[i] = (float)hv[i];
+    K_CHECK(hipMemcpy(hv.data(), dvs, sizeof(T) * nv, hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < nv; i++) v_separate[i] = (float)hv[i];
+  }
 }
 }  // namespace
 
@@ -361,14 +379,18 @@ extern "C" {
 
 int lc0mi_k_winograd_conv(const float* x, const float* filter, const float* bias, const float* skip,
                           const float* se_w1, const float* se_b1, const float* se_w2, const float* se_b2, int se_k,
-                          int batch, int cin, int cout, int act, int use_fp16, float* out) {
+                          int batch, int cin, int cout, int act, int use_fp16, float* out, float* v_fused,
+                          float* v_separate) {
   return Guard([&] {
     RequireDevice();
     if (batch < 1 || cin < 1 || cout < 1 || cout > 1024 || se_k < 0 || se_k > 256) throw Error("bad convolution shape");
+    if ((v_fused == nullptr) != (v_separate == nullptr)) throw Error("v_fused and v_separate go together");
     if (use_fp16) {
-      WinogradConvHost<half_t>(x, filter, bias, skip, se_w1, se_b1, se_w2, se_b2, se_k, batch, cin, cout, act, out);
+      WinogradConvHost<half_t>(x, filter, bias, skip, se_w1, se_b1, se_w2, se_b2, se_k, batch, cin, cout, act, out,
+                               v_fused, v_separate);
     } else {
-      WinogradConvHost<float>(x, filter, bias, skip, se_w1, se_b1, se_w2, se_b2, se_k, batch, cin, cout, act, out);
+      WinogradConvHost<float>(x, filter, bias, skip, se_w1, se_b1, se_w2, se_b2, se_k, batch, cin, cout, act, out,
+                              v_fused, v_separate);
     }
   });
 }

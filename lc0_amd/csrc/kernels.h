@@ -165,10 +165,15 @@ void LaunchWinogradInputTransform(const T* x, T* v, int batch, int C, int ldv, h
 //           out = act(gamma * y + skip + beta)
 // m: [36][B*4][C] (M_IS_F32 selects float m for T = half_t), out/skip: [B][64][C].
 // se_w1: [K][C], se_w2: [K][2C] floats (the transpose of lc0's [2C][K]). C <= 1024, K <= 256.
+// v_next (optional, only when WinogradFusedInputTransform(C, sizeof(T), se_k)): the input transform of the next
+// convolution is applied to the result in the same kernel and written to v_next[36][B*4][ldv_next];
+// out may then be null if nobody else reads the activations.
 template <typename T, typename MT>
 void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip, const float* se_w1,
                                    const float* se_b1, const float* se_w2, const float* se_b2, int se_k, T* out,
-                                   int batch, int C, int act, hipStream_t stream);
+                                   int batch, int C, int act, hipStream_t stream, T* v_next = nullptr,
+                                   int ldv_next = 0);
+bool WinogradFusedInputTransform(int C, int elem_size, int se_k);
 
 // Gather of the convolutional policy head: out[b][j] = t[b][sq][plane] for
 // kConvPolicyMap[plane*64+sq] = j. t: [B][64][ld] (NHWC), inv_map: [1858] holding plane*64+sq.

@@ -315,8 +315,8 @@ class Mi355xNetwork : public Network, protected ModelState {
   template <typename T>
   void ForwardResnet(int B);
   template <typename T>
-  void WinogradConv(const char* name, const struct ConvDev& conv, const void* x, const void* skip, const struct SeDev* se,
-                    int act, void* out, int B);
+  bool WinogradConv(const char* name, const struct ConvDev& conv, const void* x, const void* skip, const struct SeDev* se,
+                    int act, void* out, int B, bool have_v = false, const struct ConvDev* next = nullptr);
   template <typename T>
   void GemmT(const char* name, const void* A, int lda, long long strideA, const void* W, int ldw, long long strideW,
              void* C, int ldc, long long strideC, const float* bias, int M, int N, int K, int batch, int act,
@@ -1280,26 +1280,36 @@ void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
   res_cmax_ = static_cast<size_t>(std::max(filters_, max_head_ch));
 }
 
-// One 3x3 convolution: input transform, 36 batched GEMMs, output transform with the fused tail.
+// One 3x3 convolution: input transform (unless the previous convolution's output transform
+// has already produced it: have_v), 36 batched GEMMs, output transform with the fused tail.
+// next: the convolution that consumes the result; when the shapes allow it, its input
+// transform is fused into this output transform (returns true), and `out` may be null if
+// nothing else reads the activations.
 template <typename T>
-void Mi355xNetwork::WinogradConv(const char* name, const ConvDev& conv, const void* x, const void* skip,
-                                 const SeDev* se, int act, void* out, int B) {
+bool Mi355xNetwork::WinogradConv(const char* name, const ConvDev& conv, const void* x, const void* skip,
+                                 const SeDev* se, int act, void* out, int B, bool have_v, const ConvDev* next) {
   const int tiles = B * 4;
-  Timed("winograd_input_transform", 0.0, sizeof(T) * B * (64.0 + 144.0) * conv.cin, [&] {
-    LaunchWinogradInputTransform<T>(static_cast<const T*>(x), static_cast<T*>(r_v_), B, conv.cin, conv.ld, stream_);
-  });
+  if (!have_v) {
+    Timed("winograd_input_transform", 0.0, sizeof(T) * B * (64.0 + 144.0) * conv.cin, [&] {
+      LaunchWinogradInputTransform<T>(static_cast<const T*>(x), static_cast<T*>(r_v_), B, conv.cin, conv.ld, stream_);
+    });
+  }
   // Winograd-domain products M in the tower's own type (half products are accurate enough
   // because the transform matrices are row-balanced; float M would double the traffic of
   // both the GEMM epilogue and the output transform).
   GemmT<T>(name, r_v_, conv.ld, static_cast<long long>(tiles) * conv.ld, conv.u, conv.ld,
            static_cast<long long>(conv.cout) * conv.ld, r_m_, conv.cout, static_cast<long long>(tiles) * conv.cout,
            nullptr, tiles, conv.cout, conv.ld, 36, kActNone, /*out_f32=*/false);
-  Timed("winograd_output_transform", 0.0, B * conv.cout * sizeof(T) * (144.0 + 64.0 * (skip ? 2 : 1)), [&] {
+  const bool fuse = next != nullptr && next->cin == conv.cout && next->ld == conv.cout &&
+                    WinogradFusedInputTransform(conv.cout, sizeof(T), se ? se->k : 0);
+  Timed(fuse ? "winograd_output_input_transform" : "winograd_output_transform", 0.0,
+        B * conv.cout * sizeof(T) * (144.0 + 64.0 * ((skip ? 1 : 0) + (out ? 1 : 0)) + (fuse ? 144.0 : 0.0)), [&] {
     LaunchWinogradOutputTransform<T, T>(static_cast<const T*>(r_m_), conv.bias, static_cast<const T*>(skip),
                                         se ? se->w1 : nullptr, se ? se->b1 : nullptr, se ? se->w2 : nullptr,
                                         se ? se->b2 : nullptr, se ? se->k : 0, static_cast<T*>(out), B, conv.cout,
-                                        act, stream_);
+                                        act, stream_, fuse ? static_cast<T*>(r_v_) : nullptr, fuse ? next->ld : 0);
   });
+  return fuse;
 }
 
 template <typename T>
@@ -1308,11 +1318,23 @@ void Mi355xNetwork::ForwardResnet(int B) {
   Timed("expand_planes", 0.0, B * (112.0 * 12 + sizeof(T) * 64.0 * 112), [&] {
     LaunchExpandPlanesNhwc<T>(d_masks_, d_values_, static_cast<T*>(r_in_), B, stream_);
   });
-  WinogradConv<T>("gemm_winograd_input", res_input_, r_in_, nullptr, nullptr, default_act_, r_x_, B);
-  for (const ResBlockDev& blk : res_blocks_) {
-    WinogradConv<T>("gemm_winograd", blk.conv1, r_x_, nullptr, nullptr, default_act_, r_y_, B);
-    WinogradConv<T>("gemm_winograd", blk.conv2, r_y_, r_x_, blk.has_se ? &blk.se : nullptr, default_act_, r_x_, B);
+  // Every output transform also produces the next convolution's transformed input when the
+  // shapes allow it; r_y_ (a block's inner activations) is then never written.
+  const ConvDev* after_tower = (conv_policy_ && !attn_policy_) ? &res_policy1_ : nullptr;
+  const ConvDev* first = res_blocks_.empty() ? after_tower : &res_blocks_[0].conv1;
+  bool have_v = WinogradConv<T>("gemm_winograd_input", res_input_, r_in_, nullptr, nullptr, default_act_, r_x_, B,
+                                false, first);
+  for (size_t i = 0; i < res_blocks_.size(); i++) {
+    const ResBlockDev& blk = res_blocks_[i];
+    const ConvDev* next = i + 1 < res_blocks_.size() ? &res_blocks_[i + 1].conv1 : after_tower;
+    const bool inner = WinogradFusedInputTransform(blk.conv1.cout, sizeof(T), 0) && blk.conv2.cin == blk.conv1.cout &&
+                       blk.conv2.ld == blk.conv1.cout;
+    have_v = WinogradConv<T>("gemm_winograd", blk.conv1, r_x_, nullptr, nullptr, default_act_, inner ? nullptr : r_y_, B,
+                             have_v, &blk.conv2);
+    have_v = WinogradConv<T>("gemm_winograd", blk.conv2, r_y_, r_x_, blk.has_se ? &blk.se : nullptr, default_act_, r_x_,
+                             B, have_v, next);
   }
+  const bool policy_have_v = have_v;
   auto fc = [&](const char* name, const void* a, const LinearT& l, void* c, int m, int act, bool out_f32) {
     GemmT<T>(name, a, l.ld, 0, l.w, l.ld, 0, c, l.out, 0, l.b, m, l.out, l.ld, 1, act, out_f32);
   };
@@ -1329,8 +1351,10 @@ void Mi355xNetwork::ForwardResnet(int B) {
   if (attn_policy_) {
     if constexpr (sizeof(T) == 2) ForwardAttentionPolicy(static_cast<const half_t*>(r_x_), filters_, B);
   } else if (conv_policy_) {
-    WinogradConv<T>("gemm_winograd_policy", res_policy1_, r_x_, nullptr, nullptr, default_act_, r_y_, B);
-    WinogradConv<T>("gemm_winograd_policy", res_policy_conv_, r_y_, nullptr, nullptr, kActNone, r_h1_, B);
+    // (the heads above do not touch r_v_, so the tower's last fused transform is still there)
+    const bool v2 = WinogradConv<T>("gemm_winograd_policy", res_policy1_, r_x_, nullptr, nullptr, default_act_, r_y_, B,
+                                    policy_have_v, &res_policy_conv_);
+    WinogradConv<T>("gemm_winograd_policy", res_policy_conv_, r_y_, nullptr, nullptr, kActNone, r_h1_, B, v2);
     Timed("policy_gather", 0.0, B * (sizeof(T) * 73.0 * 64 + 4.0 * 1858), [&] {
       LaunchConvPolicyGather<T>(static_cast<const T*>(r_h1_), res_policy_conv_.cout, conv_inv_map_, d_policy_, B,
                                 stream_);

@@ -183,11 +183,12 @@ template <typename T, typename MT>
 __global__ __launch_bounds__(1024) void winograd_output_transform_tiles_kernel(
     const MT* __restrict__ m, const float* __restrict__ bias, const T* skip, const float* __restrict__ se_w1,
     const float* __restrict__ se_b1, const float* __restrict__ se_w2, const float* __restrict__ se_b2, int se_k,
-    T* out, int batch, int C, int act) {
+    T* out, T* __restrict__ v_next, int ldv, int batch, int C, int act) {
   extern __shared__ float shm[];
   float* part = shm;               // [4][C], then pool[C] in its first row
   float* hidden = shm + 4 * C;     // [K]
   float* gate = hidden + se_k;     // gamma[C] | beta[C]
+  T* xs = reinterpret_cast<T*>(gate + 2 * C + ((se_k & 1) ? 1 : 0));   // [64][C] activations for the fused input transform
   const int b = blockIdx.x;
   const int tile = threadIdx.x / C, c = threadIdx.x - tile * C;
   const long long kstride = (long long)batch * 4 * C;
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(1024) void winograd_output_transform_tiles_kernel(
   }
   const int ty = (tile >> 1) * 4, tx = (tile & 1) * 4;
   const T* sk = skip ? skip + (long long)b * 64 * C + c : nullptr;
-  T* o = out + (long long)b * 64 * C + c;
+  T* o = out ? out + (long long)b * 64 * C + c : nullptr;
 #pragma unroll
   for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -257,8 +258,49 @@ __global__ __launch_bounds__(1024) void winograd_output_transform_tiles_kernel(
       const int sq = (ty + i) * 8 + tx + j;
       float v = gamma * y[i][j] + beta;
       if (sk) v += (float)sk[(long long)sq * C];
-      o[(long long)sq * C] = (T)RActivate(v, act);
+      const T r = (T)RActivate(v, act);
+      if (o) o[(long long)sq * C] = r;
+      if (v_next) xs[sq * C + c] = r;
     }
+  if (!v_next) return;
+  // Fused input transform of the next convolution: this thread's tile reads its 6x6
+  // patch (with the halo owned by the other three tiles) from LDS.
+  __syncthreads();
+  const int y0 = ty - 1, x0 = tx - 1;
+  float d[6][6];
+#pragma unroll
+  for (int i = 0; i < 6; i++)
+#pragma unroll
+    for (int j = 0; j < 6; j++) {
+      const int yy = y0 + i, xx = x0 + j;
+      d[i][j] = (yy >= 0 && yy < 8 && xx >= 0 && xx < 8) ? (float)xs[(yy * 8 + xx) * C + c] : 0.0f;
+    }
+  float t[6][6];
+#pragma unroll
+  for (int j = 0; j < 6; j++) {
+    const float d0 = d[0][j], d1 = d[1][j], d2 = d[2][j], d3 = d[3][j], d4 = d[4][j], d5 = d[5][j];
+    t[0][j] = d0 - 1.25f * d2 + 0.25f * d4;
+    t[1][j] = (-4.0f * (d1 + d2) + d3 + d4) * (1.0f / 6.0f);
+    t[2][j] = (4.0f * (d1 - d2) - d3 + d4) * (1.0f / 6.0f);
+    t[3][j] = (-2.0f * d1 - d2 + 2.0f * d3 + d4) * (1.0f / 24.0f);
+    t[4][j] = (2.0f * d1 - d2 - 2.0f * d3 + d4) * (1.0f / 24.0f);
+    t[5][j] = 4.0f * d1 - 5.0f * d3 + d5;
+  }
+  T* vo = v_next + (long long)(b * 4 + tile) * ldv + c;
+  const long long vstride = (long long)batch * 4 * ldv;
+#pragma unroll
+  for (int i = 0; i < 6; i++) {
+    const float t0 = t[i][0], t1 = t[i][1], t2 = t[i][2], t3 = t[i][3], t4 = t[i][4], t5 = t[i][5];
+    float r[6];
+    r[0] = t0 - 1.25f * t2 + 0.25f * t4;
+    r[1] = (-4.0f * (t1 + t2) + t3 + t4) * (1.0f / 6.0f);
+    r[2] = (4.0f * (t1 - t2) - t3 + t4) * (1.0f / 6.0f);
+    r[3] = (-2.0f * t1 - t2 + 2.0f * t3 + t4) * (1.0f / 24.0f);
+    r[4] = (2.0f * t1 - t2 - 2.0f * t3 + t4) * (1.0f / 24.0f);
+    r[5] = 4.0f * t1 - 5.0f * t3 + t5;
+#pragma unroll
+    for (int j = 0; j < 6; j++) vo[(long long)(i * 6 + j) * vstride] = (T)r[j];
+  }
 }
 
 template <typename T>
@@ -312,28 +354,35 @@ template void LaunchWinogradInputTransform<float>(const float*, float*, int, int
 template <typename T, typename MT>
 void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip, const float* se_w1,
                                    const float* se_b1, const float* se_w2, const float* se_b2, int se_k, T* out,
-                                   int batch, int C, int act, hipStream_t stream) {
+                                   int batch, int C, int act, hipStream_t stream, T* v_next, int ldv_next) {
   if (batch <= 0) return;
   const int k = se_k > 0 ? se_k : 0;
   if (C <= 256) {
-    const size_t shm = sizeof(float) * (size_t)(6 * C + k);
+    size_t shm = sizeof(float) * (size_t)(6 * C + k + (k & 1));
+    if (v_next) shm += sizeof(T) * 64 * (size_t)C;
     hipLaunchKernelGGL((winograd_output_transform_tiles_kernel<T, MT>), dim3(batch), dim3(4 * C), shm, stream, m, bias,
-                       skip, se_w1, se_b1, se_w2, se_b2, se_k, out, batch, C, act);
+                       skip, se_w1, se_b1, se_w2, se_b2, se_k, out, v_next, ldv_next, batch, C, act);
     return;
   }
+  // Wide towers: separate kernels (the caller checks WinogradFusedInputTransform before asking for v_next).
   const size_t shm = sizeof(float) * (size_t)(C + k);
   hipLaunchKernelGGL((winograd_output_transform_kernel<T, MT>), dim3(batch), dim3(C), shm, stream, m, bias, skip,
                      se_w1, se_b1, se_w2, se_b2, se_k, out, batch, C, act);
 }
+// The fused kernel needs 4 * C threads and its staging area in the 64 KiB of dynamic LDS.
+bool WinogradFusedInputTransform(int C, int elem_size, int se_k) {
+  return C <= 256 && sizeof(float) * (6 * C + se_k + 1) + (size_t)elem_size * 64 * C <= 64 * 1024;
+}
+
 template void LaunchWinogradOutputTransform<half_t, half_t>(const half_t*, const float*, const half_t*, const float*,
                                                             const float*, const float*, const float*, int, half_t*,
-                                                            int, int, int, hipStream_t);
+                                                            int, int, int, hipStream_t, half_t*, int);
 template void LaunchWinogradOutputTransform<half_t, float>(const float*, const float*, const half_t*, const float*,
                                                            const float*, const float*, const float*, int, half_t*, int,
-                                                           int, int, hipStream_t);
+                                                           int, int, hipStream_t, half_t*, int);
 template void LaunchWinogradOutputTransform<float, float>(const float*, const float*, const float*, const float*,
                                                           const float*, const float*, const float*, int, float*, int,
-                                                          int, int, hipStream_t);
+                                                          int, int, hipStream_t, float*, int);
 
 template <typename T>
 void LaunchConvPolicyGather(const T* t, int ld, const int16_t* inv_map, float* out, int batch, hipStream_t stream) {

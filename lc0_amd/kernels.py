@@ -19,7 +19,7 @@ def _lib():
         lib.lc0mi_k_gemm.argtypes = [vp, ci, ll, vp, ci, ll, vp, ci, ci, ci, ci, cf, ci, ci, vp, ci, ll, ci, cd]
         lib.lc0mi_k_gemm_splitk.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, ci, cf, vp, ci]
         lib.lc0mi_k_layer_norm_rows.argtypes = [vp, vp, ci, vp, vp, vp, ci, ci, cf, cf, vp]
-        lib.lc0mi_k_winograd_conv.argtypes = [vp] * 8 + [ci] * 6 + [vp]
+        lib.lc0mi_k_winograd_conv.argtypes = [vp] * 8 + [ci] * 6 + [vp] * 3
         lib.lc0mi_k_expand_planes_nhwc.argtypes = [vp, vp, ci, vp]
         lib.lc0mi_k_gemm_f32.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, ci, vp, ci]
         lib.lc0mi_k_layer_norm.argtypes = [vp, vp, vp, vp, ci, ci, cf, cf, vp, ci, cd]
@@ -203,8 +203,10 @@ def attn_policy_gather(logits, keys, ppo):
     return out
 
 
-def winograd_conv(x, filt, bias, skip=None, se=None, act=ACT_RELU, fp16=False):
-    """x [B,64,Cin] (NHWC), filt [Cout,Cin,3,3], se = (w1 [K,C], b1, w2 [2C,K], b2) or None -> [B,64,Cout]."""
+def winograd_conv(x, filt, bias, skip=None, se=None, act=ACT_RELU, fp16=False, fused_next=False):
+    """x [B,64,Cin] (NHWC), filt [Cout,Cin,3,3], se = (w1 [K,C], b1, w2 [2C,K], b2) or None -> [B,64,Cout].
+    fused_next: also returns the next convolution's transformed input [36, B*4, Cout] twice: from the
+    fused output+input transform kernel and from the stand-alone input transform of the output."""
     x = np.ascontiguousarray(x, np.float32)
     filt = np.ascontiguousarray(filt, np.float32)
     bias = np.ascontiguousarray(bias, np.float32)
@@ -218,9 +220,11 @@ def winograd_conv(x, filt, bias, skip=None, se=None, act=ACT_RELU, fp16=False):
         w1 = b1 = w2 = b2 = None
         k = 0
     out = np.zeros((b, 64, cout), np.float32)
+    vf = np.zeros((36, b * 4, cout), np.float32) if fused_next else None
+    vs = np.zeros((36, b * 4, cout), np.float32) if fused_next else None
     _check(_lib().lc0mi_k_winograd_conv(_ptr(x), _ptr(filt), _ptr(bias), _ptr(sk), _ptr(w1), _ptr(b1), _ptr(w2),
-                                        _ptr(b2), k, b, cin, cout, act, int(fp16), _ptr(out)))
-    return out
+                                        _ptr(b2), k, b, cin, cout, act, int(fp16), _ptr(out), _ptr(vf), _ptr(vs)))
+    return (out, vf, vs) if fused_next else out
 
 
 def expand_planes_nhwc(masks, values):

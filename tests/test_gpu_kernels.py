@@ -314,3 +314,29 @@ def test_attention_head_depths(depth):
     p = onn.softmax_rows(bias + np.matmul(q, k.transpose(0, 1, 3, 2)) * f32(scale))
     want = np.matmul(p, v).transpose(0, 2, 1, 3).reshape(batch * 64, d)
     np.testing.assert_allclose(got, want, rtol=4e-3, atol=4e-3)
+
+
+@pytest.mark.parametrize("fp16", [True, False])
+@pytest.mark.parametrize("batch,c,se_k,with_skip", [(3, 32, 8, True), (2, 64, 0, False), (5, 256, 64, True)])
+def test_fused_output_input_transform_equals_separate_kernels(batch, c, se_k, with_skip, fp16):
+    """The output transform that also produces the next convolution's transformed input must give
+    exactly what the stand-alone input transform gives on the stored activations (fp32 at 256
+    channels does not fit the fused kernel's LDS budget and is refused)."""
+    from lc0_amd import BackendError, kernels as K
+    rng = np.random.default_rng(batch + c)
+    x = rng.standard_normal((batch, 64, c)).astype(f32)
+    filt = (rng.standard_normal((c, c, 3, 3)) * (c * 9) ** -0.5).astype(f32)
+    bias = (0.1 * rng.standard_normal(c)).astype(f32)
+    skip = rng.standard_normal((batch, 64, c)).astype(f32) if with_skip else None
+    se = None
+    if se_k:
+        se = (rng.standard_normal((se_k, c)).astype(f32) * 0.3, rng.standard_normal(se_k).astype(f32) * 0.1,
+              rng.standard_normal((2 * c, se_k)).astype(f32) * 0.3, rng.standard_normal(2 * c).astype(f32) * 0.1)
+    if not fp16 and c == 256:
+        with pytest.raises(BackendError, match="cannot be fused"):
+            K.winograd_conv(x, filt, bias, skip, se, fp16=fp16, fused_next=True)
+        return
+    out, vf, vs = K.winograd_conv(x, filt, bias, skip, se, fp16=fp16, fused_next=True)
+    np.testing.assert_array_equal(vf, vs)
+    np.testing.assert_array_equal(out, K.winograd_conv(x, filt, bias, skip, se, fp16=fp16))
+    assert np.abs(vf).max() > 0.1
