@@ -139,3 +139,24 @@ def test_mutated_weight_files_never_crash_the_loader():
         assert rc != 0 and not net.value
         seen.add(lib.lc0mi_last_error().decode(errors="replace")[:40])
     assert len(seen) >= 3, seen      # several distinct failure paths were exercised
+
+
+@pytest.mark.parametrize("options,message", [
+    ("precision=int4", "Precision 'int4' is not supported"),
+    ("max_batch=0", "max_batch must be in 1..4096"),
+    ("max_batch=5000", "max_batch must be in 1..4096"),
+    ("lanes=0", "lanes must be in 1..8"),
+    ("lanes=9", "lanes must be in 1..8"),
+    ("precision=fp8,fp8_gemms=qkv+nope", "fp8_gemms"),
+    ("policy_head=soft", "does not exist in this net"),
+    ("value_head=q", "does not exist in this net"),
+    ("max_batch=abc", "max_batch"),
+    ("mlh=perhaps", "mlh"),
+])
+def test_option_validation_happens_before_the_device_is_touched(options, message):
+    """Backend options are checked while the network is set up, so their error messages can be
+    pinned without a GPU (unknown keys are reported after construction, as in lc0,
+    src/utils/optionsdict.cc:330-341, and therefore need a device)."""
+    from lc0_amd import BackendError, Network, netgen
+    with pytest.raises(BackendError, match=message):
+        Network(netgen.cached_config("tiny_attn"), options)
