@@ -357,7 +357,7 @@ void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip
                                    int batch, int C, int act, hipStream_t stream, T* v_next, int ldv_next) {
   if (batch <= 0) return;
   const int k = se_k > 0 ? se_k : 0;
-  if (C <= 256) {
+  if (C <= 256 && C % 16 == 0) {   // 4 * C threads in whole waves (the SE reduction shuffles across a wave)
     size_t shm = sizeof(float) * (size_t)(6 * C + k + (k & 1));
     if (v_next) shm += sizeof(T) * 64 * (size_t)C;
     hipLaunchKernelGGL((winograd_output_transform_tiles_kernel<T, MT>), dim3(batch), dim3(4 * C), shm, stream, m, bias,
@@ -371,7 +371,7 @@ void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip
 }
 // The fused kernel needs 4 * C threads and its staging area in the 64 KiB of dynamic LDS.
 bool WinogradFusedInputTransform(int C, int elem_size, int se_k) {
-  return C <= 256 && sizeof(float) * (6 * C + se_k + 1) + (size_t)elem_size * 64 * C <= 64 * 1024;
+  return C <= 256 && C % 16 == 0 && sizeof(float) * (6 * C + se_k + 1) + (size_t)elem_size * 64 * C <= 64 * 1024;
 }
 
 template void LaunchWinogradOutputTransform<half_t, half_t>(const half_t*, const float*, const half_t*, const float*,

@@ -230,6 +230,8 @@ CONFIGS = {
     "tiny_resnet": lambda: se_resnet(32, 2, 8, seed=2000, moves_left=True),
     "tiny_resnet_convpolicy": lambda: se_resnet(32, 2, 8, seed=2003, conv_policy=True),
     "tiny_resnet_nose": lambda: se_resnet(24, 3, 0, seed=2004, moves_left=True),
+    # 40 filters with SE: a channel count that is not a multiple of 16 (separate transform kernels)
+    "tiny_resnet_40se": lambda: se_resnet(40, 2, 8, seed=2009, moves_left=True),
     # (std 0.1 instead of 0.02: at width 64 that gives policy logits of order 0.1-1, so absolute
     # tolerances in the parity tests mean something)
     "tiny_attn": lambda: attention_body(64, 2, 2, 96, seed=2001, smolgen=(8, 32, 32), perturb_ln=True, std=0.1),

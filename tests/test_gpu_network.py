@@ -85,6 +85,8 @@ def test_attention_nets_match_oracle(name, batch, positions):
 @pytest.mark.parametrize("name,batch,options,tol", [
     ("tiny_resnet", 19, "precision=fp32", 1e-3), ("tiny_resnet", 19, "precision=fp16", 5e-3),
     ("tiny_resnet_convpolicy", 8, "precision=fp32", 1e-3), ("tiny_resnet_nose", 8, "precision=fp32", 1e-3),
+    ("tiny_resnet_convpolicy", 8, "precision=fp16", 5e-3), ("tiny_resnet_nose", 8, "precision=fp16", 5e-3),
+    ("tiny_resnet_40se", 9, "precision=fp32", 1e-3), ("tiny_resnet_40se", 9, "precision=fp16", 5e-3),
     ("c0_resnet_6x64", 32, "precision=fp32", 1e-3), ("c0_resnet_6x64", 32, "precision=fp16", 5e-3)])
 def test_residual_tower_nets_match_oracle(name, batch, options, tol, positions):
     """SE-ResNet family through the winograd F(4x4,3x3) path; configs[0] in fp32 within 1e-3."""
