@@ -248,6 +248,9 @@ CONFIGS = {
                                             pol_encoder=(2, 4, 96)),
     # convolutional body with the attention policy head and one policy encoder layer
     "tiny_resnet_attnpolicy": lambda: se_resnet(32, 2, 8, seed=2008, attn_policy=(64, 64, 1, 2, 96)),
+    # fp8-capable widths with the dense position encoding, gating and the multi-head format
+    "tiny_attn_dense_f8": lambda: attention_body(128, 2, 4, 256, seed=2010, smolgen=(8, 32, 32), perturb_ln=True, std=0.07,
+                                                 pe_dense=(16, 128), gating=True, multihead=True),
     "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True, std=0.1),
 }
 

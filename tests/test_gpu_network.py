@@ -257,6 +257,17 @@ def test_fp8_tiny_net_and_calibration_api(positions):
         fp16_net.CalibrateFp8(masks, values)
 
 
+def test_fp8_with_dense_embedding_and_named_heads(positions):
+    """fp8 on a format-7 net: the calibration point of the first layer sits after the embedding FFN."""
+    path = netgen.cached_config("tiny_attn_dense_f8")
+    masks, values, legal = positions["masks"][:48], positions["values"][:48], positions["legal"][:48]
+    want = onn.BlasNetwork(nr.load(path), policy_head="soft", value_head="q").forward(masks, values)
+    _, res = _run_gpu(path, masks, values, "precision=fp8,policy_head=soft,value_head=q")
+    s = _fp8_report(res, want, legal)
+    assert s["logit_rms"] <= 0.08 * s["logit_std"] and s["kl_max"] <= 5e-4 and s["top1_decisive"] >= 0.99
+    assert s["q"] <= 0.08 and s["d"] <= 0.04
+
+
 @pytest.mark.timeout(900)
 def test_bt4_shape_fp8_batch_sweep(positions):
     """configs[4]: the BT4-shape net with e4m3 GEMM operands. Oracle comparison on 64 positions,
