@@ -190,6 +190,11 @@ def main():
         "kernel_ms_per_step": {k.name: round(k.ms / prof_iters, 4) for k in kernels},
         "kernel_variant_ms_per_step": {g.name: round(g.ms / prof_iters, 4) for g in sorted(groups.values(), key=lambda g: -g.ms)},
         "sum_kernel_ms_per_step": total_kernel_ms,
+        # bandwidth-bound kernels: algorithmic bytes / HIP-event time against the 8 TB/s HBM peak
+        "hbm_kernels": {g.name: {"GBps": round(g.bytes / (g.ms * 1e-3) / 1e9, 1),
+                                 "frac_of_hbm_peak": round(g.bytes / (g.ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 3),
+                                 "avg_launch_us": round(g.ms / g.launches * 1e3, 2)}
+                        for g in sorted(groups.values(), key=lambda g: -g.ms) if g.flops == 0 and g.ms > 0},
         "policy_checksum": checksum,
     }
     if sweep:

@@ -351,11 +351,6 @@ __device__ __forceinline__ void DmaToLds16(const void* gptr, void* lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory", "m0");
 }
 
-template <int... Is, typename F>
-__device__ __forceinline__ void StaticFor(std::integer_sequence<int, Is...>, F&& f) {
-  (f(std::integral_constant<int, Is>{}), ...);
-}
-
 // 4 floats -> 4 e4m3 bytes (round to nearest even, saturating at +-448; the
 // hardware conversion alone would turn |v| > 464 into NaN).
 __device__ __forceinline__ unsigned PackFp8x4(float a, float b, float c, float d) {
