@@ -26,21 +26,25 @@ typedef int intx8 __attribute__((ext_vector_type(8)));
 
 namespace {
 
-// Activation functions with the reference's formulas (shared/activation.cc:51-100).
+// Activation functions (values as shared/activation.cc:51-100). The GEMM epilogues are bound by
+// vector-ALU issue, so mish and swish use one hardware exponential and one hardware reciprocal
+// (1 ulp each) instead of a correctly rounded division:
+//   mish(v) = v * tanh(log(1 + e^v)) = v * n / (n + 2),  n = e^v * (e^v + 2).
+// The exponent is clamped at 20, where n / (n + 2) already rounds to 1 in float.
 __device__ __forceinline__ float ActMish(float v) {
-  float e = __expf(v);
-  float n = e * e + 2.0f * e;
-  float d = v / (n + 2.0f);
-  return v <= -0.125f ? n * d : v - 2.0f * d;
+  const float e = __expf(__builtin_fminf(v, 20.0f));
+  const float n = e * (e + 2.0f);
+  return v * n * __builtin_amdgcn_rcpf(n + 2.0f);
 }
+__device__ __forceinline__ float ActSigmoid(float v) { return __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
 __device__ __forceinline__ float Activate(float v, int act) {
   switch (act) {
     case 1: return ActMish(v);
     case 2: return v > 0.0f ? v : 0.0f;
     case 4: return tanhf(v);
-    case 5: return 1.0f / (1.0f + __expf(-v));
+    case 5: return ActSigmoid(v);
     case 6: return v > 0.0f ? 1.05070098f * v : 1.05070098f * 1.67326324f * (__expf(v) - 1.0f);
-    case 7: return v / (1.0f + __expf(-v));
+    case 7: return v * ActSigmoid(v);
     case 8: return v > 0.0f ? v * v : 0.0f;
     default: return v;
   }
@@ -53,7 +57,7 @@ __device__ __forceinline__ void DispatchAct(int act, F&& f) {
   switch (act) {
     case 1: f([](float v) { return ActMish(v); }); break;
     case 2: f([](float v) { return v > 0.0f ? v : 0.0f; }); break;
-    case 7: f([](float v) { return v / (1.0f + __expf(-v)); }); break;
+    case 7: f([](float v) { return v * ActSigmoid(v); }); break;
     case 8: f([](float v) { return v > 0.0f ? v * v : 0.0f; }); break;
     case 3: f([](float v) { return v; }); break;
     default: f([act](float v) { return Activate(v, act); }); break;

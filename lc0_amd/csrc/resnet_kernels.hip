@@ -17,17 +17,16 @@ namespace {
 
 __device__ __forceinline__ float RActivate(float v, int act) {
   switch (act) {
-    case 1: {
-      float e = __expf(v);
-      float n = e * e + 2.0f * e;
-      float d = v / (n + 2.0f);
-      return v <= -0.125f ? n * d : v - 2.0f * d;
+    case 1: {  // mish = v * n / (n + 2), n = e^v (e^v + 2); exponent clamped where the ratio rounds to 1
+      const float e = __expf(__builtin_fminf(v, 20.0f));
+      const float n = e * (e + 2.0f);
+      return v * n * __builtin_amdgcn_rcpf(n + 2.0f);
     }
     case 2: return v > 0.0f ? v : 0.0f;
     case 4: return tanhf(v);
-    case 5: return 1.0f / (1.0f + __expf(-v));
+    case 5: return __builtin_amdgcn_rcpf(1.0f + __expf(-v));
     case 6: return v > 0.0f ? 1.05070098f * v : 1.05070098f * 1.67326324f * (__expf(v) - 1.0f);
-    case 7: return v / (1.0f + __expf(-v));
+    case 7: return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
     case 8: return v > 0.0f ? v * v : 0.0f;
     default: return v;
   }
