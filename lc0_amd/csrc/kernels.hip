@@ -358,10 +358,10 @@ __device__ __forceinline__ void DmaToLds16(const void* gptr, void* lds_base) {
 // 4 floats -> 4 e4m3 bytes (round to nearest even, saturating at +-448; the
 // hardware conversion alone would turn |v| > 464 into NaN).
 __device__ __forceinline__ unsigned PackFp8x4(float a, float b, float c, float d) {
-  a = __builtin_fminf(__builtin_fmaxf(a, -448.0f), 448.0f);
-  b = __builtin_fminf(__builtin_fmaxf(b, -448.0f), 448.0f);
-  c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
-  d = __builtin_fminf(__builtin_fmaxf(d, -448.0f), 448.0f);
+  a = __builtin_amdgcn_fmed3f(a, -448.0f, 448.0f);  // median of three = clamp, one instruction
+  b = __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f);
+  c = __builtin_amdgcn_fmed3f(c, -448.0f, 448.0f);
+  d = __builtin_amdgcn_fmed3f(d, -448.0f, 448.0f);
   int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
   v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
   return (unsigned)v;
@@ -1128,8 +1128,10 @@ void LaunchQuantizeF8(const half_t* x, uint8_t* y, long long n, float mul, hipSt
 // ---------------------------------------------------------------------------
 namespace {
 // DEPTH = head depth (32, 64 or 128); OutT = half_t, or uint8_t for e4m3 output scaled by out_mul.
+// Second launch bound = waves per SIMD the register allocation must allow: the kernel is a chain of
+// dependent memory phases (q/k/v loads, bias loads, stores), so resident waves are what hides latency.
 template <int DEPTH, typename OutT>
-__global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict__ qkv,
+__global__ __launch_bounds__(256, DEPTH == 32 ? 4 : DEPTH == 64 ? 3 : 1) void attention_kernel(const half_t* __restrict__ qkv,
                                                         const half_t* __restrict__ bias,
                                                         OutT* __restrict__ out, int total_heads, int heads,
                                                         float scale, float out_mul) {
@@ -1243,20 +1245,38 @@ __global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict
     }
   }
   if (!live) return;
-  OutT* O = out + (long long)b * 64 * d_model + h * DEPTH;
+  // The accumulator layout would store 2 bytes per lane; go through this wave's LDS region (V is consumed)
+  // so that the global stores are 16 bytes per lane and cover whole rows of the head.
+  constexpr int kRowBytes = DEPTH * (int)sizeof(OutT);
+  constexpr int kOStride = kRowBytes + 16;  // bytes per query row in LDS
+  constexpr int kChunksPerRow = kRowBytes / 16;
+  static_assert(64 * kOStride <= 64 * kVStride * (int)sizeof(half_t), "output staging fits the V region");
+  unsigned char* os = reinterpret_cast<unsigned char*>(vs);
+  __builtin_amdgcn_wave_barrier();
 #pragma unroll
   for (int nt = 0; nt < 2; nt++)
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
 #pragma unroll
       for (int e = 0; e < 16; e++) {
-        int q = 32 * nt + 8 * (e / 4) + 4 * g + (e % 4);
+        const int q = 32 * nt + 8 * (e / 4) + 4 * g + (e % 4);
+        OutT* dst = reinterpret_cast<OutT*>(os + q * kOStride) + dt * 32 + r;
         if constexpr (sizeof(OutT) == 1) {
-          O[(long long)q * d_model + dt * 32 + r] = (uint8_t)(PackFp8x4(o[nt][dt][e] * out_mul, 0.0f, 0.0f, 0.0f) & 0xffu);
+          *dst = (uint8_t)(PackFp8x4(o[nt][dt][e] * out_mul, 0.0f, 0.0f, 0.0f) & 0xffu);
         } else {
-          O[(long long)q * d_model + dt * 32 + r] = (half_t)o[nt][dt][e];
+          *dst = (half_t)o[nt][dt][e];
         }
       }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the region is private to this wave
+  __builtin_amdgcn_wave_barrier();
+  unsigned char* O = reinterpret_cast<unsigned char*>(out + (long long)b * 64 * d_model + h * DEPTH);
+  const long long o_row_bytes = (long long)d_model * (long long)sizeof(OutT);
+#pragma unroll
+  for (int i = 0; i < kChunksPerRow; i++) {
+    const int idx = i * 64 + lane;
+    const int q = idx / kChunksPerRow, c = idx - q * kChunksPerRow;
+    *reinterpret_cast<uint4*>(O + q * o_row_bytes + c * 16) = *reinterpret_cast<const uint4*>(os + q * kOStride + c * 16);
+  }
 }
 }  // namespace
 
