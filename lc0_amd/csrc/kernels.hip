@@ -1203,11 +1203,12 @@ __global__ __launch_bounds__(256, DEPTH == 32 ? 4 : DEPTH == 64 ? 3 : 1) void at
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     float sum = 0.0f;
+    const float kLog2e = 1.44269504f, neg_mx = -mx * kLog2e;
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
 #pragma unroll
       for (int e = 0; e < 16; e++) {
-        float ev = __expf(st[mt][nt][e] - mx);
+        float ev = __builtin_amdgcn_exp2f(__builtin_fmaf(st[mt][nt][e], kLog2e, neg_mx));  // e^(s - mx)
         st[mt][nt][e] = ev;
         sum += ev;
       }
