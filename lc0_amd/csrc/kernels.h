@@ -98,7 +98,7 @@ void LaunchZero(float* p, long long n, hipStream_t stream);
 // Forces LaunchGemm to use one kernel variant (-1 = automatic choice): 0 256x256x64,
 // 1 256x192x64, 2 256x128x32 (direct-to-LDS, need K % 64 == 0 and half output),
 // 3 128x128x64, 4 64x64x64 (register-staged), 5 128x128x64 direct-to-LDS with 4 waves,
-// 6 row-panel 64x32 (K split over the four waves). For tests and tuning only.
+// 6 row-panel 64x32 (K split over the waves), 7 128x64x64 direct-to-LDS with 4 waves. For tests and tuning only.
 void SetGemmVariantOverride(int variant);
 
 // Layer norm for few, long rows (one workgroup per row): t = act(x) * alpha + skip,

@@ -54,7 +54,7 @@ def test_gemm_splitk_vs_oracle_fc(m, n, k, split):
     np.testing.assert_allclose(got, onn.fc(a, w.reshape(-1), b, nr.ACT_NONE), rtol=3e-4, atol=3e-4)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("m,n,k", [(2048, 1024, 256), (777, 200, 128), (300, 1858, 64), (64, 64, 192)])
 def test_every_gemm_variant_vs_oracle_fc(variant, m, n, k):
     """Every tile variant (the three direct-to-LDS kernels and the two
