@@ -626,10 +626,12 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
     if (c192 < cost) { best = kDma256x192; cost = c192; }
     if (c128 < cost) { best = kDma256x128; cost = c128; }
     if (cs < cost) { best = kDma128x128; cost = cs; }
-    // Short reductions only: 128x64 tiles (three workgroups per CU) move more operand bytes from L2 per
-    // flop but split odd tile counts evenly (36 x 2048x256x256: 23.1 us against 26.0 for 256x128).
-    if (a.K <= 256) {
-      const double c64 = rounds(128, 64) * 128 * 64 * 0.80;
+    // 128x64 tiles (three workgroups per CU, so partial rounds are counted as fractions) move more operand
+    // bytes from L2 per flop, but they split small problems over all CUs and odd tile counts evenly
+    // (4096x512x1024: 10.5 us against 14.6 for 128x128; 36 x 2048x256x256: 23.1 us against 26.0 for 256x128).
+    {
+      const double tiles = (double)((a.M + 127) / 128) * ((a.N + 63) / 64) * a.batch;
+      const double c64 = std::max(1.0, tiles / 256.0) * 128 * 64 * 0.80;
       if (c64 < cost) { best = kDma128x64; cost = c64; }
     }
     return best;
@@ -683,10 +685,13 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
 }
 
 namespace {
-// 0: 256x256, 1: 256x192, 2: 256x128, 5: 128x128 with 4 waves (two workgroups per CU); chosen by
+// 0: 256x256, 1: 256x192, 2: 256x128, 5: 128x128 and 7: 128x64 with 4 waves (two / three workgroups per CU); chosen by
 // the cost model of the fp16 kernels (the k-tile structure is the same).
 int PickGemmF8Variant(const GemmF8Args& a) {
-  if (g_variant_override >= 0 && (g_variant_override <= 2 || g_variant_override == kDma128x128)) return g_variant_override;
+  if (g_variant_override >= 0 &&
+      (g_variant_override <= 2 || g_variant_override == kDma128x128 || g_variant_override == kDma128x64)) {
+    return g_variant_override;
+  }
   auto rounds = [&](int bm, int bn) {
     const long long tiles = (long long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn);
     return (double)((tiles + 255) / 256);
@@ -701,6 +706,9 @@ int PickGemmF8Variant(const GemmF8Args& a) {
   if (c192 < cost) { best = 1; cost = c192; }
   if (c128 < cost) { best = 2; cost = c128; }
   if (cs < cost) { best = kDma128x128; cost = cs; }
+  const double tiles64 = (double)((a.M + 127) / 128) * ((a.N + 63) / 64);
+  const double c64 = std::max(1.0, tiles64 / 256.0) * 128 * 64 * 0.80;
+  if (c64 < cost) { best = kDma128x64; cost = c64; }
   return best;
 }
 }  // namespace
@@ -710,6 +718,7 @@ const char* GemmF8VariantName(const GemmF8Args& a) {
     case 0: return "gemm_f8_256x256x128";
     case 1: return "gemm_f8_256x192x128";
     case 2: return "gemm_f8_256x128x128";
+    case kDma128x64: return "gemm_f8_128x64x128";
     default: return "gemm_f8_128x128x128";
   }
 }
@@ -720,6 +729,7 @@ void LaunchGemmF8(const GemmF8Args& a, hipStream_t stream) {
     case 0: LaunchGemmDmaF8<256, 256, 2, 4>(a, stream); break;
     case 1: LaunchGemmDmaF8<256, 192, 4, 2>(a, stream); break;
     case 2: LaunchGemmDmaF8<256, 128, 4, 2>(a, stream); break;
+    case kDma128x64: LaunchGemmDmaF8<128, 64, 2, 2>(a, stream); break;
     default: LaunchGemmDmaF8<128, 128, 2, 2>(a, stream); break;
   }
 }

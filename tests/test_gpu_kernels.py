@@ -248,7 +248,7 @@ def test_quantize_f8_bit_exact():
         np.testing.assert_array_equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 5])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 5, 7])
 @pytest.mark.parametrize("m,n,k", [(512, 512, 128), (300, 200, 256), (2048, 1536, 1024), (64, 3072, 1024), (1, 17, 128)])
 def test_gemm_f8_vs_exact_product(variant, m, n, k):
     """e4m3 operands are exact inputs, so the product is pinned by float64 arithmetic on the decoded
