@@ -70,6 +70,23 @@ float lc0mi_comp_p(const lc0mi_comp* comp, int sample, int move_id);
  * valid until it is destroyed); NULL on error. Bulk form of GetPVal. */
 const float* lc0mi_comp_policy_row(const lc0mi_comp* comp, int sample);
 
+/* ---- legal-move policy on the device ----
+ * Replaces NetworkAsBackendComputation::SoftmaxPolicy (src/neural/wrapper.cc:135-156): the search wrapper
+ * fetches the logit of every legal move with GetPVal, subtracts the maximum, multiplies by 1 / temperature,
+ * applies FastExp (src/utils/fastmath.h:59-86) and normalises. Given the policy indices of the legal moves
+ * (MoveToNNIndex, src/neural/encoder.cc:339-619) the same arithmetic runs on the GPU and only those
+ * probabilities are copied to the host, not the 1858 logits.
+ *
+ * lc0mi_comp_add_legal_moves lists the moves of the input added last (n in 0..256, ids < 1858). Once used it
+ * must be called for every input of the computation, right after the input; lc0mi_comp_p and
+ * lc0mi_comp_policy_row then fail (the logits stay on the device). */
+int lc0mi_comp_add_legal_moves(lc0mi_comp* comp, int n, const uint16_t* move_ids);
+/* lc0's PolicyTemperature (src/neural/shared_params.cc:33-36,69); default 1.359. */
+int lc0mi_comp_set_policy_softmax_temperature(lc0mi_comp* comp, float temperature);
+/* Probabilities of the listed moves of one sample in the order they were listed (host memory owned by the
+ * computation); *n receives their number. NULL on error. */
+const float* lc0mi_comp_legal_policy(const lc0mi_comp* comp, int sample, int* n);
+
 /* Message of the last failed call on this thread (never NULL). */
 const char* lc0mi_last_error(void);
 

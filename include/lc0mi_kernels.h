@@ -56,6 +56,12 @@ int lc0mi_k_expand_planes_nchw(const uint64_t* masks, const float* values, int b
 int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const float* ppo, int pd, int batch,
                                float* out);
 
+/* Softmax over listed moves with lc0's FastExp (NetworkAsBackendComputation::SoftmaxPolicy,
+ * src/neural/wrapper.cc:135-156; src/utils/fastmath.h:59-86): policy [batch][1858]; sample b lists
+ * ids[offsets[b] .. offsets[b + 1]) (at most 256); probs is laid out like ids. */
+int lc0mi_k_legal_softmax(const float* policy, const int* offsets, const uint16_t* ids, float inv_temperature,
+                          int batch, float* probs);
+
 /* One 3x3 convolution of the residual tower through the winograd F(4x4,3x3) path
  * (input transform, 36 batched GEMMs, output transform with the fused tail):
  *   out = act(conv(x) + bias (+ skip))                      when se_k == 0

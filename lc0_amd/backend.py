@@ -59,6 +59,10 @@ def load_library():
     lib.lc0mi_comp_p.restype = cf
     lib.lc0mi_comp_policy_row.argtypes = [vp, ci]
     lib.lc0mi_comp_policy_row.restype = C.POINTER(cf)
+    lib.lc0mi_comp_add_legal_moves.argtypes = [vp, ci, vp]
+    lib.lc0mi_comp_set_policy_softmax_temperature.argtypes = [vp, cf]
+    lib.lc0mi_comp_legal_policy.argtypes = [vp, ci, C.POINTER(ci)]
+    lib.lc0mi_comp_legal_policy.restype = C.POINTER(cf)
     lib.lc0mi_last_error.restype = C.c_char_p
     lib.lc0mi_net_set_profiling.argtypes = [vp, ci]
     lib.lc0mi_net_take_profile.argtypes = [vp, C.c_char_p, ci]
@@ -236,6 +240,27 @@ class NetworkComputation:
         if not ptr:
             raise BackendError(load_library().lc0mi_last_error().decode(errors="replace"))
         return np.ctypeslib.as_array(ptr, (1858,)).copy()
+
+    def AddLegalMoves(self, move_ids):
+        """Policy indices (0..1857) of the legal moves of the input added last. Once used, every input
+        needs its list; the policy then comes from GetLegalPolicy (softmax over these moves, computed on
+        the device as lc0's search wrapper does on the host) and the raw logits are not downloaded."""
+        ids = np.ascontiguousarray(move_ids, dtype=np.uint16)
+        if ids.ndim != 1:
+            raise BackendError("AddLegalMoves expects a one-dimensional list of move ids.")
+        _check(load_library().lc0mi_comp_add_legal_moves(self._h, ids.shape[0], ids.ctypes.data))
+
+    def SetPolicySoftmaxTemperature(self, temperature):
+        _check(load_library().lc0mi_comp_set_policy_softmax_temperature(self._h, float(temperature)))
+
+    def GetLegalPolicy(self, sample):
+        n = C.c_int(0)
+        ptr = load_library().lc0mi_comp_legal_policy(self._h, sample, C.byref(n))
+        if not ptr:
+            raise BackendError(load_library().lc0mi_last_error().decode(errors="replace"))
+        if n.value == 0:
+            return np.zeros(0, np.float32)
+        return np.ctypeslib.as_array(ptr, (n.value,)).copy()
 
     def results(self):
         """All outputs as arrays: dict(policy [n,1858], q [n], d [n], m [n])."""

@@ -158,6 +158,29 @@ const float* lc0mi_comp_policy_row(const lc0mi_comp* comp, int sample) {
   return row;
 }
 
+int lc0mi_comp_add_legal_moves(lc0mi_comp* comp, int n, const uint16_t* move_ids) {
+  return Guard([&] {
+    if (!comp) throw lc0mi::Error("null computation");
+    comp->impl->AddLegalMoves(n, move_ids);
+  });
+}
+
+int lc0mi_comp_set_policy_softmax_temperature(lc0mi_comp* comp, float temperature) {
+  return Guard([&] {
+    if (!comp) throw lc0mi::Error("null computation");
+    comp->impl->SetPolicySoftmaxTemperature(temperature);
+  });
+}
+
+const float* lc0mi_comp_legal_policy(const lc0mi_comp* comp, int sample, int* n) {
+  const float* probs = nullptr;
+  Guard([&] {
+    if (!comp) throw lc0mi::Error("null computation");
+    probs = comp->impl->GetLegalPolicy(sample, n);
+  });
+  return probs;
+}
+
 const char* lc0mi_last_error(void) { return g_last_error.c_str(); }
 
 int lc0mi_net_set_profiling(lc0mi_net* net, int on) {

@@ -293,6 +293,31 @@ int lc0mi_k_attn_policy_gather(const float* logits, const uint16_t* keys, const 
   });
 }
 
+int lc0mi_k_legal_softmax(const float* policy, const int* offsets, const uint16_t* ids, float inv_temperature,
+                          int batch, float* probs) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1) throw Error("bad batch");
+    if (offsets[0] != 0) throw Error("offsets must start at 0");
+    for (int b = 0; b < batch; b++) {
+      const int n = offsets[b + 1] - offsets[b];
+      if (n < 0 || n > lc0mi::kMaxLegalMoves) throw Error("bad move count");
+    }
+    const int total = offsets[batch];
+    for (int i = 0; i < total; i++) {
+      if (ids[i] >= 1858) throw Error("move id out of range");
+    }
+    Dev dev;
+    float* dp = dev.Put(policy, (size_t)batch * 1858);
+    int* doff = dev.Put(offsets, (size_t)batch + 1);
+    uint16_t* di = dev.Put(ids, (size_t)total);
+    auto* dout = static_cast<float*>(dev.Alloc((size_t)std::max(total, 1) * 4));
+    lc0mi::LaunchLegalSoftmax(dp, doff, di, inv_temperature, dout, batch, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    if (total > 0) K_CHECK(hipMemcpy(probs, dout, (size_t)total * 4, hipMemcpyDeviceToHost));
+  });
+}
 
 }  // extern "C"
 

@@ -135,6 +135,15 @@ int SmolgenBiasIndex(int q, int k);
 void LaunchAttnPolicyGather(const float* logits, const half_t* kq, int ld_kq, int key_off, const float* ppo,
                             int pd, const int16_t* inv_map, float* out, int batch, hipStream_t stream);
 
+// Most legal moves one sample may list for LaunchLegalSoftmax (chess positions have at most 218).
+constexpr int kMaxLegalMoves = 256;
+// Softmax over the listed moves of every sample with lc0's polynomial exponential
+// (src/neural/wrapper.cc:135-156, src/utils/fastmath.h:59-86):
+//   probs[offsets[b] + i] = FastExp((policy[b][ids[offsets[b] + i]] - max_b) * inv_temperature) / total_b
+// policy: [B][1858]; offsets: [B + 1], non-decreasing, at most kMaxLegalMoves apart; ids < 1858.
+void LaunchLegalSoftmax(const float* policy, const int* offsets, const uint16_t* ids, float inv_temperature,
+                        float* probs, int batch, hipStream_t stream);
+
 }  // namespace lc0mi
 
 // ---------------------------------------------------------------------------

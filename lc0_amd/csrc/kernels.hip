@@ -1384,4 +1384,84 @@ void LaunchAttnPolicyGather(const float* logits, const half_t* kq, int ld_kq, in
                      pd, inv_map, out);
 }
 
+// ---------------------------------------------------------------------------
+// Policy softmax over the legal moves of every sample: what lc0's search wrapper does on the host
+// with the 1858 downloaded logits (NetworkAsBackendComputation::SoftmaxPolicy, src/neural/wrapper.cc:135-156,
+// with FastExp of src/utils/fastmath.h:59-86), done here so that only the probabilities of the legal moves
+// leave the device. Every float operation is a separately rounded IEEE operation in the reference's order
+// (no fused multiply-add, the total is accumulated move by move by one lane).
+// ---------------------------------------------------------------------------
+namespace {
+// 2^a for a <= 0 as a quadratic in the fractional part, exponent added to the float's bits.
+// Contraction is switched off for the plain operators of these two functions: a fused multiply-add
+// rounds once where the reference rounds twice.
+__device__ __forceinline__ float FastExp2Ref(float a) {
+#pragma clang fp contract(off)
+  int e;
+  if (a < 0.0f) {
+    if (a < -126.0f) return 0.0f;
+    e = (int)(a - 1.0f);   // truncation of a - 1 stands in for floor(a)
+  } else {
+    e = (int)a;
+  }
+  float out = a - (float)e;
+  const float inner = 0.33976606f * out;
+  const float lin = 0.6602339f + inner;
+  const float prod = out * lin;
+  out = 1.0f + prod;
+  return __int_as_float(__float_as_int(out) + (int)((unsigned)e << 23));
+}
+
+__global__ __launch_bounds__(64) void legal_softmax_kernel(const float* __restrict__ policy,
+                                                          const int* __restrict__ offsets,
+                                                          const uint16_t* __restrict__ ids, float inv_temperature,
+                                                          float* __restrict__ probs) {
+#pragma clang fp contract(off)
+  __shared__ float vals[kMaxLegalMoves];
+  __shared__ float scale_s;
+  const int b = blockIdx.x, lane = threadIdx.x;
+  const int start = offsets[b], n = offsets[b + 1] - start;
+  const float* row = policy + (long long)b * 1858;
+  constexpr int kPerLane = kMaxLegalMoves / 64;
+  float v[kPerLane];
+  float mx = -__builtin_inff();
+#pragma unroll
+  for (int j = 0; j < kPerLane; j++) {
+    const int i = lane + 64 * j;
+    v[j] = i < n ? row[ids[start + i]] : -__builtin_inff();
+    mx = fmaxf(mx, v[j]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+#pragma unroll
+  for (int j = 0; j < kPerLane; j++) {
+    const int i = lane + 64 * j;
+    if (i < n) {
+      const float scaled = (v[j] - mx) * inv_temperature;
+      vals[i] = FastExp2Ref(1.442695040f * scaled);
+    }
+  }
+  __syncthreads();
+  if (lane == 0) {
+    float total = 0.0f;
+    for (int i = 0; i < n; i++) total = total + vals[i];
+    scale_s = total > 0.0f ? 1.0f / total : 1.0f;
+  }
+  __syncthreads();
+  const float scale = scale_s;
+#pragma unroll
+  for (int j = 0; j < kPerLane; j++) {
+    const int i = lane + 64 * j;
+    if (i < n) probs[start + i] = vals[i] * scale;
+  }
+}
+}  // namespace
+
+void LaunchLegalSoftmax(const float* policy, const int* offsets, const uint16_t* ids, float inv_temperature,
+                        float* probs, int batch, hipStream_t stream) {
+  if (batch <= 0) return;
+  hipLaunchKernelGGL(legal_softmax_kernel, dim3(batch), dim3(64), 0, stream, policy, offsets, ids, inv_temperature,
+                     probs);
+}
+
 }  // namespace lc0mi

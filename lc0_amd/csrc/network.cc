@@ -169,7 +169,17 @@ struct HostSlot {
   float* wdl = nullptr;   // raw value-head outputs, 3 (WDL) or 1 per sample
   float* mlh = nullptr;
   int capacity = 0;
+  // Legal-move lists (allocated when a computation first gives one): legal_off[i] .. legal_off[i + 1] index the
+  // ids and the probabilities of sample i; legal_samples counts the samples that have a list.
+  int* legal_off = nullptr;        // [capacity + 1]
+  uint16_t* legal_ids = nullptr;   // [capacity * kMaxLegalMoves]
+  float* legal_probs = nullptr;    // [capacity * kMaxLegalMoves]
+  int legal_samples = 0;
+  float inv_temperature = 1.0f;
   ~HostSlot() {
+    if (legal_off) (void)hipHostFree(legal_off);
+    if (legal_ids) (void)hipHostFree(legal_ids);
+    if (legal_probs) (void)hipHostFree(legal_probs);
     if (masks) (void)hipHostFree(masks);
     if (values) (void)hipHostFree(values);
     if (policy) (void)hipHostFree(policy);
@@ -202,6 +212,9 @@ class Mi355xComputation : public NetworkComputation {
   float GetPVal(int sample, int move_id) const override { return GetPolicyRow(sample)[move_id]; }
   float GetMVal(int sample) const override;
   const float* GetPolicyRow(int sample) const override;
+  void AddLegalMoves(int n, const uint16_t* move_ids) override;
+  void SetPolicySoftmaxTemperature(float temperature) override;
+  const float* GetLegalPolicy(int sample, int* n) const override;
 
  private:
   void CheckSample(int sample) const {
@@ -220,6 +233,8 @@ class Mi355xComputation : public NetworkComputation {
   std::vector<std::unique_ptr<HostSlot>> slots_;
   int batch_ = 0;
   bool computed_ = false;
+  bool legal_mode_ = false;           // legal-move lists were given: probabilities instead of raw logits
+  float temperature_ = 1.359f;        // src/neural/shared_params.cc:69
 };
 
 // Everything that describes the loaded network and is the same for every lane: options,
@@ -365,6 +380,10 @@ class Mi355xNetwork : public Network, protected ModelState {
   half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
   half_t *pe_qkv_ = nullptr, *pe_att_ = nullptr, *pe_t_ = nullptr, *pe_ffn_ = nullptr;   // policy encoder scratch
   float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
+  // Legal-move softmax: per-sample offsets, policy indices and probabilities.
+  int* d_legal_off_ = nullptr;
+  uint16_t* d_legal_ids_ = nullptr;
+  float* d_legal_probs_ = nullptr;
   half_t *pre_in_ = nullptr, *pre_out_ = nullptr;
   bool calibrating_ = false;
   float* d_absmax_ = nullptr;   // [4 * layers + 1] calibration maxima (float bits, non-negative)
@@ -814,6 +833,9 @@ void Mi355xNetwork::AllocActivations() {
   d_policy_ = AllocF(static_cast<size_t>(kPolicyOutputs) * max_batch_);
   d_wdl_ = AllocF(3 * static_cast<size_t>(max_batch_));
   d_mlh_ = AllocF(max_batch_);
+  d_legal_off_ = static_cast<int*>(arena_.Alloc(sizeof(int) * (static_cast<size_t>(max_batch_) + 1)));
+  d_legal_ids_ = static_cast<uint16_t*>(arena_.Alloc(sizeof(uint16_t) * kMaxLegalMoves * max_batch_));
+  d_legal_probs_ = AllocF(static_cast<size_t>(kMaxLegalMoves) * max_batch_);
   if (attn_policy_) {
     const size_t T = static_cast<size_t>(max_batch_) * 64;
     pol_e_ = AllocH(T * pol_emb_);
@@ -1618,10 +1640,33 @@ void Mi355xNetwork::EvaluateOnLane(HostSlot* slot, int batch) {
                            stream_));
   HIP_CHECK(hipMemcpyAsync(d_values_, slot->values, sizeof(float) * kInputPlanes * batch, hipMemcpyHostToDevice,
                            stream_));
+  const bool legal = slot->legal_samples > 0;
+  if (legal) {
+    if (slot->legal_samples != batch) throw Error("legal moves were given for some inputs of the batch only");
+    const int total = slot->legal_off[batch];
+    HIP_CHECK(hipMemcpyAsync(d_legal_off_, slot->legal_off, sizeof(int) * (batch + 1), hipMemcpyHostToDevice, stream_));
+    if (total > 0) {
+      HIP_CHECK(hipMemcpyAsync(d_legal_ids_, slot->legal_ids, sizeof(uint16_t) * total, hipMemcpyHostToDevice,
+                               stream_));
+    }
+  }
   ForwardDevice(batch);
   HIP_CHECK(hipGetLastError());
-  HIP_CHECK(hipMemcpyAsync(slot->policy, d_policy_, sizeof(float) * kPolicyOutputs * batch, hipMemcpyDeviceToHost,
-                           stream_));
+  if (legal) {
+    // Only the probabilities of the listed moves are downloaded (tens of floats per sample instead of 1858).
+    const int total = slot->legal_off[batch];
+    Timed("legal_softmax", 0.0, total * 10.0 + batch * 4.0, [&] {
+      LaunchLegalSoftmax(d_policy_, d_legal_off_, d_legal_ids_, slot->inv_temperature, d_legal_probs_, batch, stream_);
+    });
+    HIP_CHECK(hipGetLastError());
+    if (total > 0) {
+      HIP_CHECK(hipMemcpyAsync(slot->legal_probs, d_legal_probs_, sizeof(float) * total, hipMemcpyDeviceToHost,
+                               stream_));
+    }
+  } else {
+    HIP_CHECK(hipMemcpyAsync(slot->policy, d_policy_, sizeof(float) * kPolicyOutputs * batch, hipMemcpyDeviceToHost,
+                             stream_));
+  }
   HIP_CHECK(hipMemcpyAsync(slot->wdl, d_wdl_, sizeof(float) * (wdl_ ? 3 : 1) * batch, hipMemcpyDeviceToHost,
                            stream_));
   if (moves_left_) {
@@ -1675,6 +1720,7 @@ std::unique_ptr<HostSlot> Mi355xNetwork::GetSlot() {
     if (!pool_->free_slots.empty()) {
       auto s = std::move(pool_->free_slots.back());
       pool_->free_slots.pop_back();
+      s->legal_samples = 0;
       return s;
     }
   }
@@ -1749,15 +1795,66 @@ void Mi355xComputation::ComputeBlocking() {
   Mi355xNetwork* net = Net();
   for (size_t si = 0; si < slots_.size(); si++) {
     const int n = std::min(max_batch_, batch_ - static_cast<int>(si) * max_batch_);
-    net->Evaluate(slots_[si].get(), n);
+    HostSlot* s = slots_[si].get();
+    if (legal_mode_ && s->legal_samples != n) {
+      throw Error("AddLegalMoves must be called for every input, right after it is added");
+    }
+    // The same reciprocal the search wrapper keeps (src/neural/wrapper.cc:81-82).
+    s->inv_temperature = 1.0f / temperature_;
+    net->Evaluate(s, n);
   }
   computed_ = true;
 }
 
 const float* Mi355xComputation::GetPolicyRow(int sample) const {
   CheckSample(sample);
+  if (legal_mode_) {
+    throw Error("raw policy logits are not downloaded when legal moves were given: use GetLegalPolicy");
+  }
   const int cap = max_batch_;
   return slots_[sample / cap]->policy + static_cast<size_t>(sample % cap) * kPolicyOutputs;
+}
+
+void Mi355xComputation::AddLegalMoves(int n, const uint16_t* move_ids) {
+  if (batch_ == 0) throw Error("AddLegalMoves needs an input: call it after AddInput");
+  if (n < 0 || n > kMaxLegalMoves) throw Error("legal move count out of range (0.." + std::to_string(kMaxLegalMoves) + ")");
+  if (n > 0 && !move_ids) throw Error("null move list");
+  const int sample = batch_ - 1;
+  HostSlot* s = slots_[static_cast<size_t>(sample / max_batch_)].get();
+  const int at = sample % max_batch_;
+  if (s->legal_samples != at) {
+    throw Error(s->legal_samples > at ? "AddLegalMoves was already called for this input"
+                                      : "AddLegalMoves must be called for every input, right after it is added");
+  }
+  if (sample > 0 && !legal_mode_) throw Error("AddLegalMoves must be called for every input, right after it is added");
+  for (int i = 0; i < n; i++) {
+    if (move_ids[i] >= kPolicyOutputs) throw Error("move id out of range");
+  }
+  if (!s->legal_off) {
+    HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&s->legal_off), sizeof(int) * (s->capacity + 1)));
+    HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&s->legal_ids), sizeof(uint16_t) * kMaxLegalMoves * s->capacity));
+    HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&s->legal_probs), sizeof(float) * kMaxLegalMoves * s->capacity));
+  }
+  if (at == 0) s->legal_off[0] = 0;
+  const int off = s->legal_off[at];
+  if (n > 0) std::memcpy(s->legal_ids + off, move_ids, sizeof(uint16_t) * n);
+  s->legal_off[at + 1] = off + n;
+  s->legal_samples = at + 1;
+  legal_mode_ = true;
+}
+
+void Mi355xComputation::SetPolicySoftmaxTemperature(float temperature) {
+  if (!(temperature > 0.0f)) throw Error("policy softmax temperature must be positive");
+  temperature_ = temperature;
+}
+
+const float* Mi355xComputation::GetLegalPolicy(int sample, int* n) const {
+  CheckSample(sample);
+  if (!legal_mode_) throw Error("no legal moves were given to this computation");
+  const HostSlot* s = slots_[static_cast<size_t>(sample / max_batch_)].get();
+  const int at = sample % max_batch_;
+  if (n) *n = s->legal_off[at + 1] - s->legal_off[at];
+  return s->legal_probs + s->legal_off[at];
 }
 
 float Mi355xComputation::GetQVal(int sample) const {

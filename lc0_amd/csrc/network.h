@@ -38,6 +38,17 @@ class NetworkComputation {
   virtual float GetMVal(int sample) const = 0;
   // 1858 raw policy logits of one sample (host memory owned by the computation).
   virtual const float* GetPolicyRow(int sample) const = 0;
+
+  // Legal-move policy: the softmax that lc0's search wrapper applies to the logits of the legal moves
+  // (NetworkAsBackendComputation::SoftmaxPolicy, src/neural/wrapper.cc:135-156) runs on the device and only
+  // those probabilities are downloaded. AddLegalMoves lists the policy indices (MoveToNNIndex,
+  // src/neural/encoder.cc:339-619) of the legal moves of the input added last; it must then be called for
+  // every input of the computation, and the raw logits (GetPVal, GetPolicyRow) are not available.
+  virtual void AddLegalMoves(int n, const uint16_t* move_ids) = 0;
+  // Policy softmax temperature (lc0's PolicyTemperature, default 1.359, src/neural/shared_params.cc:69).
+  virtual void SetPolicySoftmaxTemperature(float temperature) = 0;
+  // Probabilities of the listed moves of one sample, in the order they were listed.
+  virtual const float* GetLegalPolicy(int sample, int* n) const = 0;
 };
 
 // src/neural/network.h:85-114

@@ -31,6 +31,7 @@ def _lib():
         lib.lc0mi_k_quantize_f8.argtypes = [vp, ll, cf, vp]
         lib.lc0mi_k_layer_norm_f8.argtypes = [vp, vp, vp, vp, ci, ci, cf, cf, cf, vp, vp]
         lib.lc0mi_k_attention_f8.argtypes = [vp, vp, ci, ci, cf, cf, vp]
+        lib.lc0mi_k_legal_softmax.argtypes = [vp, vp, vp, cf, ci, vp]
         lib._k_ready = True
     return lib
 
@@ -202,6 +203,22 @@ def attn_policy_gather(logits, keys, ppo):
     out = np.zeros((n, 1858), np.float32)
     _check(_lib().lc0mi_k_attn_policy_gather(_ptr(logits), _ptr(keys), _ptr(ppo), keys.shape[1], n, _ptr(out)))
     return out
+
+
+def legal_softmax(policy, move_lists, temperature=1.359):
+    """policy f32 [B,1858]; move_lists: B sequences of policy indices -> list of B probability arrays
+    (softmax over the listed moves with lc0's FastExp, 1/temperature formed in float as the search wrapper does)."""
+    policy = np.ascontiguousarray(policy, np.float32)
+    n = policy.shape[0]
+    offsets = np.zeros(n + 1, np.int32)
+    offsets[1:] = np.cumsum([len(m) for m in move_lists])
+    ids = np.ascontiguousarray(np.concatenate([np.asarray(m, np.uint16) for m in move_lists]) if offsets[-1]
+                               else np.zeros(0, np.uint16), np.uint16)
+    probs = np.zeros(max(int(offsets[-1]), 1), np.float32)
+    inv_t = float(np.float32(1.0) / np.float32(temperature))
+    _check(_lib().lc0mi_k_legal_softmax(_ptr(policy), _ptr(offsets), _ptr(ids) if ids.size else None, inv_t, n,
+                                        _ptr(probs)))
+    return [probs[offsets[i]:offsets[i + 1]].copy() for i in range(n)]
 
 
 def winograd_conv(x, filt, bias, skip=None, se=None, act=ACT_RELU, fp16=False, fused_next=False):

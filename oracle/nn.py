@@ -466,21 +466,32 @@ class BlasNetwork:
 # ---------------------------------------------------- caller-side helpers ----
 def fast_exp(a):
     """FastExp (fastmath.h:59-86) on a float32 array."""
-    a = (np.asarray(a, f32) * f32(1.442695040)).astype(f32)
-    exp = np.where(a < 0, (a - f32(1)).astype(np.int32), a.astype(np.int32)).astype(np.int32)
-    out = (a - exp.astype(f32)).astype(f32)
-    out = (f32(1.0) + out * (f32(0.6602339) + f32(0.33976606) * out)).astype(f32)
-    bits = out.view(np.int32) + (exp.astype(np.int64) << 23).astype(np.int32)
-    res = bits.view(f32).copy()
-    res[a < -126] = 0.0
+    with np.errstate(all="ignore"):   # arguments below -126 (down to -inf) take the early return, as in the reference
+        a = (np.asarray(a, f32) * f32(1.442695040)).astype(f32)
+        safe = np.where(a < -126, f32(0), a)
+        exp = np.where(safe < 0, (safe - f32(1)).astype(np.int32), safe.astype(np.int32)).astype(np.int32)
+        out = (safe - exp.astype(f32)).astype(f32)
+        out = (f32(1.0) + out * (f32(0.6602339) + f32(0.33976606) * out)).astype(f32)
+        bits = out.view(np.int32) + (exp.astype(np.int64) << 23).astype(np.int32)
+        res = bits.view(f32).copy()
+        res[a < -126] = 0.0
     return res
 
 
 def softmax_policy_legal(logits, legal_idx, temperature=1.359):
-    """NetworkAsBackendComputation::SoftmaxPolicy (wrapper.cc:135-156)."""
+    """NetworkAsBackendComputation::SoftmaxPolicy (wrapper.cc:135-156): every step in float, the
+    reciprocal temperature formed once (wrapper.cc:81-82), the total accumulated move by move
+    (std::accumulate) and applied as a multiplication by 1/total (1 when the total is 0)."""
+    legal_idx = np.asarray(legal_idx, np.int64)
+    if legal_idx.size == 0:
+        return np.zeros(0, f32)
     l = np.asarray(logits, f32)[legal_idx]
-    p = fast_exp((l - l.max()) * f32(1.0 / temperature))
-    return (p / p.sum(dtype=f32)).astype(f32)
+    inv_t = f32(1.0) / f32(temperature)
+    with np.errstate(over="ignore"):
+        p = fast_exp(((l - l.max()).astype(f32) * inv_t).astype(f32))
+    total = np.add.accumulate(p, dtype=f32)[-1]          # sequential, left to right
+    scale = f32(1.0) / total if total > 0 else f32(1.0)
+    return (p * scale).astype(f32)
 
 
 def check_softmax_legal(logits, legal_idx):

@@ -340,3 +340,24 @@ def test_fused_output_input_transform_equals_separate_kernels(batch, c, se_k, wi
     np.testing.assert_array_equal(vf, vs)
     np.testing.assert_array_equal(out, K.winograd_conv(x, filt, bias, skip, se, fp16=fp16))
     assert np.abs(vf).max() > 0.1
+
+
+def test_legal_softmax_bit_exact_vs_oracle():
+    """legal_softmax_kernel against SoftmaxPolicy's restatement (oracle/nn.py: FastExp pinned on the
+    compiled reference header): list lengths around the wave size and the 256 limit, an empty list,
+    equal logits, logits so far below the maximum that FastExp returns 0, and several temperatures."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(11)
+    lens = [0, 1, 2, 35, 63, 64, 65, 128, 218, 255, 256, 20, 31]
+    policy = (rng.standard_normal((len(lens), 1858)) * 3).astype(f32)
+    policy[3, :] = 0.25                              # all equal
+    policy[4, ::2] = -1.0e4                          # FastExp underflow branch (a < -126)
+    policy[5, :] = -3.0e38
+    policy[5, 17] = 3.0e38                           # difference overflows to -inf
+    lists = [rng.permutation(1858)[:n] for n in lens]
+    lists[5][0] = 17
+    for t in (1.359, 1.0, 0.37, 2.2, 10.0):
+        got = K.legal_softmax(policy, lists, t)
+        for i, ids in enumerate(lists):
+            want = onn.softmax_policy_legal(policy[i], ids, t)
+            np.testing.assert_array_equal(got[i].view(np.uint32), want.view(np.uint32), err_msg="row %d T %g" % (i, t))

@@ -475,3 +475,84 @@ def test_every_resized_tensor_is_rejected_at_load(name):
         except BackendError:
             pass
     assert not accepted, accepted
+
+
+# ---- legal-move policy on the device ------------------------------------------------------------
+@pytest.mark.parametrize("name,options,batch,temperature", [
+    ("tiny_attn", "", 37, 1.359), ("tiny_resnet", "", 64, 1.0), ("tiny_attn", "max_batch=16", 40, 2.2)])
+def test_legal_move_policy_equals_caller_side_softmax(name, options, batch, temperature, positions):
+    """The probabilities computed on the device from the legal-move lists are, bit for bit, what
+    SoftmaxPolicy (wrapper.cc:135-156, restated in oracle/nn.py with the compiled-reference-pinned
+    FastExp) makes of the raw logits that the same network returns without the lists; q, d, m do
+    not change. max_batch=16 splits the computation over several device passes."""
+    from lc0_amd import Network
+    path = netgen.cached_config(name)
+    masks, values, legal = positions["masks"][:batch], positions["values"][:batch], positions["legal"][:batch]
+    net = Network(path, options)
+    raw = net.NewComputation()
+    raw.AddInputs(masks, values)
+    raw.ComputeBlocking()
+    want = raw.results()
+    comp = net.NewComputation()
+    comp.SetPolicySoftmaxTemperature(temperature)
+    rng = np.random.default_rng(5)
+    lists = []
+    for i in range(batch):
+        ids = np.array(legal[i], np.int64)
+        if i % 7 == 3:
+            ids = ids[:0]                       # a position without moves (mate / stalemate)
+        elif i % 7 == 5:
+            ids = rng.permutation(1858)[:256]   # longest list the interface takes
+        else:
+            ids = rng.permutation(ids)          # caller's order, not sorted
+        lists.append(ids)
+        comp.AddInput([(int(m), float(v)) for m, v in zip(masks[i], values[i])])
+        comp.AddLegalMoves(ids)
+    comp.ComputeBlocking()
+    for i in range(batch):
+        got = comp.GetLegalPolicy(i)
+        exp = onn.softmax_policy_legal(want["policy"][i], lists[i], temperature)
+        assert got.shape == exp.shape
+        np.testing.assert_array_equal(got.view(np.uint32), exp.view(np.uint32), err_msg="sample %d" % i)
+        if len(lists[i]):
+            assert abs(float(got.sum()) - 1.0) < 1e-5
+        assert comp.GetQVal(i) == want["q"][i] and comp.GetDVal(i) == want["d"][i] and comp.GetMVal(i) == want["m"][i]
+    with pytest.raises(Exception, match="GetLegalPolicy"):
+        comp.GetPolicyRow(0)
+    with pytest.raises(Exception, match="no legal moves"):
+        raw.GetLegalPolicy(0)
+    comp.close()
+    raw.close()
+
+
+def test_legal_move_policy_call_order_errors(positions):
+    from lc0_amd import Network
+    net = Network(netgen.cached_config("tiny_attn"), "")
+    masks, values = positions["masks"], positions["values"]
+    planes = lambda i: [(int(m), float(v)) for m, v in zip(masks[i], values[i])]
+    c = net.NewComputation()
+    with pytest.raises(Exception, match="after AddInput"):
+        c.AddLegalMoves([1, 2])
+    c.AddInput(planes(0))
+    c.AddLegalMoves([1, 2, 3])
+    with pytest.raises(Exception, match="already called"):
+        c.AddLegalMoves([4])
+    with pytest.raises(Exception, match="positive"):
+        c.SetPolicySoftmaxTemperature(0.0)
+    c.AddInput(planes(1))
+    with pytest.raises(Exception, match="every input"):
+        c.ComputeBlocking()                      # second input has no list
+    with pytest.raises(Exception, match="out of range"):
+        c.AddLegalMoves([1858])
+    with pytest.raises(Exception, match="out of range"):
+        c.AddLegalMoves(list(range(257)))
+    c.AddLegalMoves([7])
+    c.ComputeBlocking()
+    assert c.GetLegalPolicy(1).tolist() == [1.0]
+    c.close()
+    c = net.NewComputation()
+    c.AddInput(planes(0))
+    c.AddInput(planes(1))
+    with pytest.raises(Exception, match="every input"):
+        c.AddLegalMoves([1])                     # first input was added without a list
+    c.close()

@@ -356,10 +356,26 @@ def test_fast_exp_and_legal_softmax(ref):
     want = np.array([ref.ref_fast_exp(float(v)) for v in x], f32)
     np.testing.assert_allclose(onn.fast_exp(x), want, rtol=1e-6)
     np.testing.assert_allclose(onn.fast_exp(x), np.exp(x.astype(np.float64)), rtol=4e-3)
-    logits = np.random.default_rng(8).standard_normal(1858).astype(f32)
-    legal = np.array([3, 77, 500, 1857])
-    p = onn.softmax_policy_legal(logits, legal)
-    assert abs(p.sum() - 1) < 1e-5 and p.argmax() == logits[legal].argmax()
+    np.testing.assert_array_equal(onn.fast_exp(x), want)      # same float operations in the same order
+    assert onn.fast_exp(np.array([-200.0, -np.inf], f32)).tolist() == [0.0, 0.0]
+    rng = np.random.default_rng(8)
+    logits = (rng.standard_normal(1858) * 3).astype(f32)
+    for n, t in ((4, 1.359), (35, 1.0), (218, 2.2)):
+        legal = rng.permutation(1858)[:n]
+        p = onn.softmax_policy_legal(logits, legal, t)
+        assert abs(p.sum() - 1) < 1e-5 and p.argmax() == logits[legal].argmax()
+        # wrapper.cc:135-156 step by step on float scalars with the compiled FastExp
+        inv_t = f32(1.0) / f32(t)
+        mx = max(logits[i] for i in legal)
+        vals = [f32(ref.ref_fast_exp(float(f32(f32(logits[i] - mx) * inv_t)))) for i in legal]
+        total = f32(0)
+        for v in vals:
+            total = f32(total + v)
+        scale = f32(1.0) / total
+        np.testing.assert_array_equal(p, np.array([f32(v * scale) for v in vals], f32))
+        # the polynomial exponential stays within a few 1e-3 of the exact softmax at this temperature
+        exact = np.exp((logits[legal].astype(np.float64) - float(mx)) / t)
+        np.testing.assert_allclose(p, exact / exact.sum(), rtol=8e-3)
 
 
 def test_e4m3_codec_vs_compiled_reference(ref):
