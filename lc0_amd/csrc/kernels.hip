@@ -798,7 +798,7 @@ void LaunchGemmF32(const GemmArgsF32& a, hipStream_t stream) {
 // Input plane expansion.
 // ---------------------------------------------------------------------------
 namespace {
-template <typename T>
+template <typename T, int V>   // V channels per thread and store: 8 when ld % 8 == 0, else 1
 __global__ __launch_bounds__(256) void expand_planes_attn_kernel(const uint64_t* __restrict__ masks,
                                                                  const float* __restrict__ values,
                                                                  const T* __restrict__ extra, int n_extra,
@@ -814,15 +814,30 @@ __global__ __launch_bounds__(256) void expand_planes_attn_kernel(const uint64_t*
   }
   __syncthreads();
   T* o = out + (long long)b * 64 * ld;
-  for (int i = threadIdx.x; i < 64 * ld; i += 256) {
-    int sq = i / ld, c = i - sq * ld;
-    T v = (T)0.0f;
-    if (c < 112) {
-      if ((smask[c] >> sq) & 1ull) v = (T)sval[c];
-    } else if (c < 112 + n_extra) {
-      v = ex[sq * n_extra + (c - 112)];
+  const int chunks = ld / V;
+  for (int i = threadIdx.x; i < 64 * chunks; i += 256) {
+    const int sq = i / chunks, c0 = (i - sq * chunks) * V;
+    T v[V];
+#pragma unroll
+    for (int e = 0; e < V; e++) {
+      const int c = c0 + e;
+      T x = (T)0.0f;
+      if (c < 112) {
+        if ((smask[c] >> sq) & 1ull) x = (T)sval[c];
+      } else if (c < 112 + n_extra) {
+        x = ex[sq * n_extra + (c - 112)];
+      }
+      v[e] = x;
     }
-    o[i] = v;
+    T* dst = o + (long long)sq * ld + c0;
+    if constexpr (V == 1) {
+      dst[0] = v[0];
+    } else if constexpr (sizeof(T) == 2) {
+      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(v);
+    } else {
+      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(v);
+      *reinterpret_cast<uint4*>(dst + 4) = *reinterpret_cast<const uint4*>(v + 4);
+    }
   }
 }
 
@@ -864,15 +879,25 @@ template <typename T>
 void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T* pos_enc, T* out, int ld,
                             int batch, hipStream_t stream) {
   if (batch <= 0) return;
-  hipLaunchKernelGGL(expand_planes_attn_kernel<T>, dim3(batch), dim3(256), 0, stream, masks, values, pos_enc, 64, 0LL,
-                     out, ld);
+  if (ld % 8 == 0) {
+    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 8>), dim3(batch), dim3(256), 0, stream, masks, values, pos_enc, 64,
+                       0LL, out, ld);
+  } else {
+    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 1>), dim3(batch), dim3(256), 0, stream, masks, values, pos_enc, 64,
+                       0LL, out, ld);
+  }
 }
 
 void LaunchExpandPlanesDense(const uint64_t* masks, const float* values, const half_t* extra, int n_extra,
                              half_t* out, int ld, int batch, hipStream_t stream) {
   if (batch <= 0) return;
-  hipLaunchKernelGGL(expand_planes_attn_kernel<half_t>, dim3(batch), dim3(256), 0, stream, masks, values, extra,
-                     n_extra, 64LL * n_extra, out, ld);
+  if (ld % 8 == 0) {
+    hipLaunchKernelGGL((expand_planes_attn_kernel<half_t, 8>), dim3(batch), dim3(256), 0, stream, masks, values, extra,
+                       n_extra, 64LL * n_extra, out, ld);
+  } else {
+    hipLaunchKernelGGL((expand_planes_attn_kernel<half_t, 1>), dim3(batch), dim3(256), 0, stream, masks, values, extra,
+                       n_extra, 64LL * n_extra, out, ld);
+  }
 }
 
 void LaunchPiecePlanes(const uint64_t* masks, const float* values, half_t* out, int batch, hipStream_t stream) {
@@ -1351,14 +1376,35 @@ __global__ __launch_bounds__(256) void attn_policy_gather_kernel(const float* __
                                                                  float* __restrict__ out) {
   __shared__ float off[4][8];
   const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int u = 0; u < 8; u++) {
-    int t = wave * 8 + u;
-    int i = t / 8, j = t % 8;
-    const half_t* krow = kq + (long long)(b * 64 + 56 + j) * ld_kq + key_off;
-    float s = 0.0f;
-    for (int k = lane; k < pd; k += 64) s += (float)krow[k] * ppo[i * pd + k];
-    s = WaveSum(s);
-    if (lane == 0) off[i][j] = s;
+  // Promotion offsets off[i][j] = key row (56 + j) . ppo row i: wave i takes ppo row i against all eight keys,
+  // with the loads of the eight products in flight together.
+  {
+    const int i = wave;
+    const half_t* krow = kq + (long long)(b * 64 + 56) * ld_kq + key_off;
+    float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (((pd | ld_kq | key_off) & 7) == 0) {
+      for (int c = lane; c < pd / 8; c += 64) {
+        const floatx4 p0 = *reinterpret_cast<const floatx4*>(ppo + (long long)i * pd + c * 8);
+        const floatx4 p1 = *reinterpret_cast<const floatx4*>(ppo + (long long)i * pd + c * 8 + 4);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const half8 kv = *reinterpret_cast<const half8*>(krow + (long long)j * ld_kq + c * 8);
+#pragma unroll
+          for (int e = 0; e < 4; e++) s[j] += (float)kv[e] * p0[e] + (float)kv[4 + e] * p1[e];
+        }
+      }
+    } else {
+      for (int k = lane; k < pd; k += 64) {
+        const float pw = ppo[(long long)i * pd + k];
+#pragma unroll
+        for (int j = 0; j < 8; j++) s[j] += (float)krow[(long long)j * ld_kq + k] * pw;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float t = WaveSum(s[j]);
+      if (lane == 0) off[i][j] = t;
+    }
   }
   __syncthreads();
   const float* lg = logits + (long long)b * 4096;
