@@ -556,3 +556,46 @@ def test_legal_move_policy_call_order_errors(positions):
     with pytest.raises(Exception, match="every input"):
         c.AddLegalMoves([1])                     # first input was added without a list
     c.close()
+
+
+def test_legal_and_raw_computations_interleaved_across_threads(positions):
+    """Pinned staging slots are recycled between computations: a slot that last carried legal-move lists
+    must come back clean for a raw computation and the other way round, also with 4 threads on 2 lanes."""
+    import threading
+    from lc0_amd import Network
+    net = Network(netgen.cached_config("tiny_attn"), "lanes=2,max_batch=32")
+    masks, values, legal = positions["masks"], positions["values"], positions["legal"]
+    ref = net.NewComputation()
+    ref.AddInputs(masks[:64], values[:64])
+    ref.ComputeBlocking()
+    raw = ref.results()
+    errors = []
+
+    def worker(t):
+        try:
+            for it in range(8):
+                n = 1 + (5 * t + 7 * it) % 50          # up to 2 device passes at max_batch=32
+                comp = net.NewComputation()
+                if (t + it) % 2 == 0:
+                    comp.AddInputs(masks[:n], values[:n])
+                    comp.ComputeBlocking()
+                    np.testing.assert_array_equal(comp.results()["policy"], raw["policy"][:n])
+                else:
+                    for i in range(n):
+                        comp.AddInputs(masks[i:i + 1], values[i:i + 1])
+                        comp.AddLegalMoves(legal[i])
+                    comp.ComputeBlocking()
+                    for i in range(n):
+                        want = onn.softmax_policy_legal(raw["policy"][i], legal[i])
+                        np.testing.assert_array_equal(comp.GetLegalPolicy(i), want)
+                        assert comp.GetQVal(i) == raw["q"][i]
+                comp.close()
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
