@@ -82,6 +82,7 @@ class Mi355xNetwork : public Network {
     add("max_batch", std::to_string(options.GetOrDefault<int>("max_batch", 1024)));
     add("lanes", std::to_string(options.GetOrDefault<int>("lanes", 4)));
     add("graphs", options.GetOrDefault<bool>("graphs", true) ? "true" : "false");
+    add("overlap_min_batch", std::to_string(options.GetOrDefault<int>("overlap_min_batch", -1)));
     const std::string precision = options.GetOrDefault<std::string>("precision", "fp16");
     add("precision", precision);
     if (precision == "fp8") {
