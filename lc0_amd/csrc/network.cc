@@ -248,6 +248,7 @@ struct ModelState {
   std::string policy_head_, value_head_;
   bool use_graphs_ = true;
   int overlap_min_batch_ = 0;   // smallest batch whose smolgen chain runs on the side stream
+  int heads_overlap_min_batch_ = -1;   // smallest batch whose value and moves-left heads run beside the policy head (-1: automatic)
 
   // Attention body dimensions.
   int emb_ = 0, d_model_ = 0, heads_ = 0, dff_ = 0, in_ld_ = 192;
@@ -368,6 +369,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   hipStream_t stream_ = nullptr;
   hipStream_t side_stream_ = nullptr;  // smolgen chain, overlapped with the QKV projection
   std::vector<hipEvent_t> fork_events_, join_events_;
+  hipEvent_t heads_fork_ = nullptr, heads_join_ = nullptr;   // value / moves-left heads beside the policy head
   DeviceArena arena_;
   std::mutex eval_mutex_;
   std::shared_ptr<SlotPool> pool_ = std::make_shared<SlotPool>();
@@ -751,6 +753,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   // 1.81 -> 1.73 ms, fp8 batch 16 1.69 -> 1.57 ms; from batch 4 / 64 up the overlap wins).
   overlap_min_batch_ = options.GetInt("overlap_min_batch", -1);
   if (overlap_min_batch_ < 0) overlap_min_batch_ = fp8_ ? 48 : 2;
+  heads_overlap_min_batch_ = options.GetInt("heads_overlap_min_batch", -1);
   lane_count_ = options.GetInt("lanes", 4);
   if (lane_count_ < 1 || lane_count_ > 8) throw Error("lanes must be in 1..8.");
   policy_head_ = options.GetString("policy_head", "vanilla");
@@ -817,6 +820,8 @@ Mi355xNetwork::~Mi355xNetwork() {
     for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
     for (hipEvent_t e : fork_events_) (void)hipEventDestroy(e);
     for (hipEvent_t e : join_events_) (void)hipEventDestroy(e);
+    if (heads_fork_) (void)hipEventDestroy(heads_fork_);
+    if (heads_join_) (void)hipEventDestroy(heads_join_);
     if (side_stream_) {
       (void)hipStreamSynchronize(side_stream_);
       (void)hipStreamDestroy(side_stream_);
@@ -830,6 +835,8 @@ void Mi355xNetwork::CreateStreams() {
   HIP_CHECK(hipSetDevice(device_));
   HIP_CHECK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
   HIP_CHECK(hipStreamCreateWithFlags(&side_stream_, hipStreamNonBlocking));
+  HIP_CHECK(hipEventCreateWithFlags(&heads_fork_, hipEventDisableTiming));
+  HIP_CHECK(hipEventCreateWithFlags(&heads_join_, hipEventDisableTiming));
 }
 
 // Device buffers of one lane (inputs, activations, outputs), sized for max_batch_.
@@ -1515,18 +1522,32 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     if (calibrating_) RecordAbsMax(x_, nx, static_cast<int>(4 * li + 4));
   }
 
-  // Value head.
-  Gemm("gemm_value_embed", x_, emb_, val_emb_lin_, head1_, val_ch_, T, default_act_);
-  Gemm("gemm_value_fc1", head1_, 64 * val_ch_, val_fc1_, head2_, val_fc_, B, default_act_);
-  Gemm("gemm_value_fc2", head2_, val_fc_, val_fc2_, d_wdl_, val_out_, B, kActNone, /*out_f32=*/true);
-  // Moves-left head.
-  if (moves_left_) {
-    Gemm("gemm_mlh_embed", x_, emb_, mov_emb_lin_, head1_, mov_ch_, T, default_act_);
-    Gemm("gemm_mlh_fc1", head1_, 64 * mov_ch_, mov_fc1_, head2_, mov_fc_, B, default_act_);
-    Gemm("gemm_mlh_fc2", head2_, mov_fc_, mov_fc2_, d_mlh_, 1, B, kActRelu, /*out_f32=*/true);
+  // Value and moves-left heads: six small GEMMs that leave most CUs idle. From a batch size on (two
+  // cross-queue dependencies must be paid for) they run on the side stream beside the policy head.
+  // Measured on one machine: 15x1024 net, fp16, -0.7 % (batch 256) to -2 % (batch 16) of the pass; fp8 -2 % from
+  // batch 64, +11 % at batch 16 where nothing else uses the side stream; a 10x256 net loses 1-10 % at every
+  // batch size (its six head GEMMs are shorter than the two dependencies). Hence the automatic rule: wide
+  // bodies only, and only where the smolgen chain already runs on the side stream.
+  const int heads_min = heads_overlap_min_batch_ >= 0 ? heads_overlap_min_batch_
+                                                      : (emb_ >= 768 ? std::max(overlap_min_batch_, 16) : 1 << 30);
+  const bool heads_beside = !profiling_ && B >= heads_min;
+  hipStream_t hs = heads_beside ? side_stream_ : stream_;
+  if (heads_beside) {
+    HIP_CHECK(hipEventRecord(heads_fork_, stream_));
+    HIP_CHECK(hipStreamWaitEvent(hs, heads_fork_, 0));
   }
+  Gemm("gemm_value_embed", x_, emb_, val_emb_lin_, head1_, val_ch_, T, default_act_, false, hs);
+  Gemm("gemm_value_fc1", head1_, 64 * val_ch_, val_fc1_, head2_, val_fc_, B, default_act_, false, hs);
+  Gemm("gemm_value_fc2", head2_, val_fc_, val_fc2_, d_wdl_, val_out_, B, kActNone, /*out_f32=*/true, hs);
+  if (moves_left_) {
+    Gemm("gemm_mlh_embed", x_, emb_, mov_emb_lin_, head1_, mov_ch_, T, default_act_, false, hs);
+    Gemm("gemm_mlh_fc1", head1_, 64 * mov_ch_, mov_fc1_, head2_, mov_fc_, B, default_act_, false, hs);
+    Gemm("gemm_mlh_fc2", head2_, mov_fc_, mov_fc2_, d_mlh_, 1, B, kActRelu, /*out_f32=*/true, hs);
+  }
+  if (heads_beside) HIP_CHECK(hipEventRecord(heads_join_, hs));
   // Policy head.
   ForwardAttentionPolicy(x_, emb_, B);
+  if (heads_beside) HIP_CHECK(hipStreamWaitEvent(stream_, heads_join_, 0));
 }
 
 void Mi355xNetwork::LaunchEager(int batch) {

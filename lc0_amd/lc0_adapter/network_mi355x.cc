@@ -83,6 +83,7 @@ class Mi355xNetwork : public Network {
     add("lanes", std::to_string(options.GetOrDefault<int>("lanes", 4)));
     add("graphs", options.GetOrDefault<bool>("graphs", true) ? "true" : "false");
     add("overlap_min_batch", std::to_string(options.GetOrDefault<int>("overlap_min_batch", -1)));
+    add("heads_overlap_min_batch", std::to_string(options.GetOrDefault<int>("heads_overlap_min_batch", -1)));
     const std::string precision = options.GetOrDefault<std::string>("precision", "fp16");
     add("precision", precision);
     if (precision == "fp8") {
