@@ -16,6 +16,7 @@ from . import netproto
 
 # pblczero.NetworkFormat enums (proto/net.proto:275-366)
 INPUT_CLASSICAL_112_PLANE = 1
+INPUT_112_WITH_CANONICALIZATION_HECTOPLIES = 4
 OUTPUT_WDL = 2
 NETWORK_SE_WITH_HEADFORMAT = 4
 NETWORK_ATTENTIONBODY_WITH_HEADFORMAT = 6
@@ -216,6 +217,11 @@ def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_s
     return {"format": {"weights_encoding": netproto.LINEAR16, "network_format": nf}, "weights": w}
 
 
+def _with_input_format(net, input_format):
+    net["format"]["network_format"]["input"] = input_format
+    return net
+
+
 # The benchmark configurations (name -> builder). Seeds are part of the spec.
 CONFIGS = {
     # 6 blocks x 64 filters SE-ResNet, SE ratio 4, classical policy, WDL.
@@ -252,6 +258,10 @@ CONFIGS = {
     "tiny_attn_dense_f8": lambda: attention_body(128, 2, 4, 256, seed=2010, smolgen=(8, 32, 32), perturb_ln=True, std=0.07,
                                                  pe_dense=(16, 128), gating=True, multihead=True),
     "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True, std=0.1),
+    # canonical input format with hectoplies: board transforms, en-passant plane, fractional rule-50 plane values
+    "tiny_attn_canonical": lambda: _with_input_format(
+        attention_body(64, 2, 2, 96, seed=2011, smolgen=(8, 32, 32), perturb_ln=True, std=0.1),
+        INPUT_112_WITH_CANONICALIZATION_HECTOPLIES),
 }
 
 

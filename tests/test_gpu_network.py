@@ -599,3 +599,27 @@ def test_legal_and_raw_computations_interleaved_across_threads(positions):
     for th in threads:
         th.join()
     assert not errors, errors
+
+
+def test_canonical_hectoplies_input_format_with_legal_policy():
+    """A net that declares INPUT_112_WITH_CANONICALIZATION_HECTOPLIES: positions are encoded for that format
+    (board transform chosen per position, en-passant plane, rule-50 plane in hundredths), the capabilities
+    report it, the outputs match the oracle, and the legal-move lists (policy indices under each position's
+    transform, MoveToNNIndex(move, transform)) give the caller-side softmax bit for bit."""
+    from lc0_amd import Network
+    fmt = oc.INPUT_112_WITH_CANONICALIZATION_HECTOPLIES
+    pos = oc.random_positions(48, seed=777, input_format=fmt)
+    assert len({float(v) for v in pos["values"][:, 109]}) > 4          # fractional rule-50 values present
+    path = netgen.cached_config("tiny_attn_canonical")
+    net, res = _run_gpu(path, pos["masks"], pos["values"])
+    assert net.GetCapabilities().input_format == fmt
+    bn = onn.BlasNetwork(nr.load(path))
+    _compare(res, bn.forward(pos["masks"], pos["values"]), pos["legal"])
+    comp = net.NewComputation()
+    for i in range(48):
+        comp.AddInputs(pos["masks"][i:i + 1], pos["values"][i:i + 1])
+        comp.AddLegalMoves(pos["legal"][i])
+    comp.ComputeBlocking()
+    for i in range(48):
+        np.testing.assert_array_equal(comp.GetLegalPolicy(i), onn.softmax_policy_legal(res["policy"][i], pos["legal"][i]))
+    comp.close()
