@@ -31,6 +31,9 @@ struct GemmArgs {
   // the slices.
   int split_k = 1;
   long long split_stride = 0;
+  // Choose the variant with the shortest latency even if it occupies more of the GPU (for a kernel on the
+  // critical path; the default favours the variant that leaves room for a concurrent stream).
+  bool latency_first = false;
 };
 void LaunchGemm(const GemmArgs& args, hipStream_t stream);
 // Name of the kernel variant LaunchGemm picks for these arguments (tile shape).

@@ -640,7 +640,7 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
     if (ok) return static_cast<GemmVariant>(g_variant_override);
   }
   const long long tiles128 = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
-  if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= 128 && a.N >= 128 && a.M >= 1024 && tiles128 >= 64) {
+  if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= 128 && a.N >= 128 && a.M >= (a.latency_first ? 256 : 1024) && tiles128 >= 64) {
     // Direct-to-LDS kernels. Cost = rounds over the 256 CUs x tile area x a measured cost per
     // output element and round (ns per element at K = 1024): 0.60 for 256x256, 0.61 for 256x192;
     // the two small shapes run two workgroups per CU, 0.68 (256x128) and 0.75 (128x128) per element
@@ -676,6 +676,9 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
   // With a short K and many columns it loses (128x8192x256: 15.8 vs 5.6 us).
   const long long tiles64 = (long long)((a.M + 63) / 64) * ((a.N + 63) / 64) * a.batch;
   if (a.split_k == 1 && tiles64 <= 64 && a.K >= 512) return kRowPanel;
+  // A single 32-column panel (the smolgen compression): one workgroup per 64 rows, K split over its waves
+  // (16384x32x1024: 9.5 us against 12.3 for the 64x64 tiles, but with twice the threads on every CU).
+  if (a.latency_first && a.split_k == 1 && a.N <= 32 && a.K >= 512) return kRowPanel;
   const long long big_tiles = tiles128;
   return big_tiles >= 192 ? kTile128 : kTile64;
 }
