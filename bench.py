@@ -25,8 +25,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 # rocprofv3 --pmc on this same command; counters cannot be read from inside the process, so the figures
 # recorded under profiles/ are repeated here: (workload, batch, kernel) -> bytes.
 MEASURED_TRAFFIC = {
-    ("c2_bt4_15x1024", 256, "gemm_dma_256x256x64"): (74036 + 57080) * 1024,
-    ("c2_bt4_15x1024", 256, "gemm_dma_256x192x64"): (90618 + 49152) * 1024,
+    ("c2_bt4_15x1024", 256, "gemm_dma_256x256x64"): (72883 + 57204) * 1024,
+    ("c2_bt4_15x1024", 256, "gemm_dma_256x192x64"): (90144 + 54721) * 1024,
     ("c2_bt4_15x1024", 256, "attention"): (163959 + 32769) * 1024,
 }
 
