@@ -340,7 +340,7 @@ class Mi355xNetwork : public Network, protected ModelState {
              bool out_f32);
   template <typename T>
   struct LinearT MakeLinearT(const Vec& w, const Vec& b, int out, int in);
-  Linear MakeLinear(const Vec& w, const Vec& b, int out, int in);
+  Linear MakeLinear(const Vec& w, const Vec& b, int out, int in, int pad_to = 8);
   LinearF8 MakeLinearF8(const Vec& w, int out, int in);
   void GemmF8(const char* name, const uint8_t* A, const Linear& lin, const LinearF8& q, void* C, int M, int act,
               bool out_f8, float out_mul);
@@ -479,7 +479,7 @@ std::vector<KernelTime> Mi355xNetwork::TakeProfile() {
   return out;
 }
 
-Linear Mi355xNetwork::MakeLinear(const Vec& w, const Vec& b, int out, int in) {
+Linear Mi355xNetwork::MakeLinear(const Vec& w, const Vec& b, int out, int in, int pad_to) {
   if (static_cast<size_t>(out) * in != w.size()) {
     throw Error("Weight tensor has " + std::to_string(w.size()) + " elements, expected " + std::to_string(out) +
                 " x " + std::to_string(in) + ".");
@@ -488,7 +488,7 @@ Linear Mi355xNetwork::MakeLinear(const Vec& w, const Vec& b, int out, int in) {
   Linear l;
   l.out = out;
   l.in = in;
-  l.ld = RoundUp(in, 8);
+  l.ld = RoundUp(in, pad_to);   // zero padding: the reduction may run over ld
   std::vector<half_t> h(static_cast<size_t>(out) * l.ld, (half_t)0.0f);
   for (int o = 0; o < out; o++)
     for (int i = 0; i < in; i++) h[static_cast<size_t>(o) * l.ld + i] = (half_t)w[static_cast<size_t>(o) * in + i];
@@ -1033,7 +1033,7 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     if (w.ip_emb_preproc_b.empty() || w.ip_emb_preproc_b.size() % 64) throw Error("Bad dense position-encoding weights.");
     enc_ch_ = static_cast<int>(w.ip_emb_preproc_b.size() / 64);
     preproc_lin_ = MakeLinear(w.ip_emb_preproc_w, w.ip_emb_preproc_b, 64 * enc_ch_, 64 * 12);
-    emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + enc_ch_);
+    emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + enc_ch_, 64);
     if (static_cast<int>(w.ip_emb_ln_gammas.size()) != emb_ || static_cast<int>(w.ip_emb_ln_betas.size()) != emb_) {
       throw Error("Embedding layer norm parameters do not match the embedding size.");
     }
@@ -1047,7 +1047,8 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     emb_ffn_ln_g_ = UploadN(w.ip_emb_ffn_ln_gammas, emb_, "Embedding FFN layer norm gamma");
     emb_ffn_ln_b_ = UploadN(w.ip_emb_ffn_ln_betas, emb_, "Embedding FFN layer norm beta");
   } else {
-    emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + 64);
+    // (176 inputs padded to 192: whole k-tiles of 64 for the direct-to-LDS GEMM; the expansion kernel zeroes the padding)
+    emb_lin_ = MakeLinear(w.ip_emb_w, w.ip_emb_b, emb_, kInputPlanes + 64, 64);
   }
   in_ld_ = emb_lin_.ld;
   if (gating_) {
