@@ -166,7 +166,7 @@ void WinogradFilterTransform4x4(const float* filter, int cout, int cin, int ld_c
 
 // V[k][b*4+t][c] = (B^T d B)[k] of the 6x6 input patch of tile t (2x2 tiles of 4x4
 // outputs, zero padding), with B^T row-scaled by 1/diag(4,6,6,24,24,1).
-// x: [B][64][C], v: [36][B*4][ldv].
+// x: [B][64][C], v: [36][B*4][ldv]; columns C..ldv-1 are written as zeros.
 template <typename T>
 void LaunchWinogradInputTransform(const T* x, T* v, int batch, int C, int ldv, hipStream_t stream);
 

@@ -869,7 +869,7 @@ void Mi355xNetwork::AllocActivations() {
     r_in_ = arena_.Alloc(ts * B * 64 * kInputPlanes);
     r_x_ = arena_.Alloc(ts * B * 64 * cmax);
     r_y_ = arena_.Alloc(ts * B * 64 * cmax);
-    r_v_ = arena_.Alloc(ts * 36 * B * 4 * std::max<size_t>(filters_, kInputPlanes));
+    r_v_ = arena_.Alloc(ts * 36 * B * 4 * std::max<size_t>(filters_, RoundUp(kInputPlanes, 64)));
     r_m_ = arena_.Alloc(ts * 36 * B * 4 * cmax);
     r_h1_ = arena_.Alloc(ts * B * 64 * cmax);
     r_h2_ = arena_.Alloc(ts * B * res_max_fc_);
@@ -1223,7 +1223,9 @@ void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
       throw Error("3x3 convolution weights have an unexpected size.");
     }
     ConvDev c;
-    c.cin = cin; c.cout = cout; c.ld = RoundUp(cin, 8);
+    // The input convolution's 112 planes are padded to 128 (whole k-tiles for the direct-to-LDS GEMM; the
+    // input transform writes the padding as zeros).
+    c.cin = cin; c.cout = cout; c.ld = (cin == kInputPlanes && sizeof(T) == 2) ? RoundUp(cin, 64) : RoundUp(cin, 8);
     std::vector<float> u(static_cast<size_t>(36) * cout * c.ld);
     WinogradFilterTransform4x4(cb.weights.data(), cout, cin, c.ld, u.data());
     std::vector<T> ut(u.size());

@@ -58,7 +58,12 @@ __global__ __launch_bounds__(256) void winograd_input_transform_kernel(const T* 
                                                                        int batch, int C, int ldv) {
   const int c = blockIdx.x * 256 + threadIdx.x;
   const int bt = blockIdx.y;  // b * 4 + tile
-  if (c >= C) return;
+  if (c >= ldv) return;
+  if (c >= C) {   // padding columns of a row longer than C: zeros, so that the GEMM may reduce over ldv
+#pragma unroll
+    for (int k = 0; k < 36; k++) v[((long long)k * batch * 4 + bt) * ldv + c] = (T)0.0f;
+    return;
+  }
   const int b = bt >> 2, tile = bt & 3;
   const int y0 = (tile >> 1) * 4 - 1, x0 = (tile & 1) * 4 - 1;
   const T* xb = x + (long long)b * 64 * C + c;
@@ -344,7 +349,7 @@ void WinogradFilterTransform4x4(const float* filter, int cout, int cin, int ld_c
 template <typename T>
 void LaunchWinogradInputTransform(const T* x, T* v, int batch, int C, int ldv, hipStream_t stream) {
   if (batch <= 0) return;
-  hipLaunchKernelGGL(winograd_input_transform_kernel<T>, dim3((C + 255) / 256, batch * 4), dim3(256), 0, stream, x, v,
+  hipLaunchKernelGGL(winograd_input_transform_kernel<T>, dim3((ldv + 255) / 256, batch * 4), dim3(256), 0, stream, x, v,
                      batch, C, ldv);
 }
 template void LaunchWinogradInputTransform<half_t>(const half_t*, half_t*, int, int, int, hipStream_t);
