@@ -623,3 +623,26 @@ def test_canonical_hectoplies_input_format_with_legal_policy():
     for i in range(48):
         np.testing.assert_array_equal(comp.GetLegalPolicy(i), onn.softmax_policy_legal(res["policy"][i], pos["legal"][i]))
     comp.close()
+
+
+@pytest.mark.parametrize("name,extra", [("tiny_attn", ""), ("tiny_attn_f8", "precision=fp8,"), ("tiny_attn_dense", "")])
+def test_stream_assignment_options_do_not_change_results(name, extra, positions):
+    """overlap_min_batch / heads_overlap_min_batch only decide which stream runs the smolgen chain and the
+    value / moves-left heads: every combination must return bitwise the same outputs, on graph replays too."""
+    from lc0_amd import Network
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:40], positions["values"][:40]
+    ref = None
+    for chain in (0, 100000):
+        for heads in (0, 100000):
+            net = Network(path, "%soverlap_min_batch=%d,heads_overlap_min_batch=%d" % (extra, chain, heads))
+            for _ in range(3):                       # first call records the graph, the others replay it
+                comp = net.NewComputation()
+                comp.AddInputs(masks, values)
+                comp.ComputeBlocking()
+                res = comp.results()
+                comp.close()
+                if ref is None:
+                    ref = res
+                for field in ("policy", "q", "d", "m"):
+                    np.testing.assert_array_equal(res[field], ref[field], err_msg="%s chain=%d heads=%d" % (field, chain, heads))
