@@ -403,7 +403,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   std::vector<Mi355xNetwork*> free_lanes_;
   int lane_count_ = 1;
   bool is_lane_ = false;
-  Mi355xNetwork* AcquireLane();
+  Mi355xNetwork* AcquireLane(bool* others_busy);
   void ReleaseLane(Mi355xNetwork* lane);
   void AcquireAllLanes();
   void ReleaseAllLanes();
@@ -413,7 +413,9 @@ class Mi355xNetwork : public Network, protected ModelState {
 
   // Captured device passes, one per batch size (option graphs=true): replaying a graph
   // costs one launch instead of several hundred, which is what bounds small batches.
-  std::map<int, hipGraphExec_t> graphs_;
+  std::map<int, hipGraphExec_t> graphs_;   // key: 2 * batch + single_stream_
+  // Set for a pass that starts while another lane is busy: it stays on its main stream (see Evaluate).
+  bool single_stream_ = false;
   void DropGraphs();
   void LaunchEager(int batch);
 
@@ -1448,7 +1450,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     const half_t* bias = nullptr;
     // The smolgen chain depends only on x: it runs on the side stream next to the
     // QKV projection (on the main stream when profiling, for clean per-kernel times).
-    hipStream_t ss = (profiling_ || B < overlap_min_batch_) ? stream_ : side_stream_;
+    hipStream_t ss = (profiling_ || single_stream_ || B < overlap_min_batch_) ? stream_ : side_stream_;
     if (e.has_smolgen) {
       const int g = sg_gen_ / heads_;
       if (ss != stream_) {
@@ -1538,7 +1540,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
   // bodies only, and only where the smolgen chain already runs on the side stream.
   const int heads_min = heads_overlap_min_batch_ >= 0 ? heads_overlap_min_batch_
                                                       : (emb_ >= 768 ? std::max(overlap_min_batch_, 16) : 1 << 30);
-  const bool heads_beside = !profiling_ && B >= heads_min;
+  const bool heads_beside = !profiling_ && !single_stream_ && B >= heads_min;
   hipStream_t hs = heads_beside ? side_stream_ : stream_;
   if (heads_beside) {
     HIP_CHECK(hipEventRecord(heads_fork_, stream_));
@@ -1574,12 +1576,13 @@ void Mi355xNetwork::DropGraphs() {
 }
 
 void Mi355xNetwork::ForwardDevice(int batch) {
-  constexpr size_t kMaxGraphs = 96;
+  constexpr size_t kMaxGraphs = 192;
   if (!use_graphs_ || profiling_ || calibrating_) {
     LaunchEager(batch);
     return;
   }
-  auto it = graphs_.find(batch);
+  const int key = 2 * batch + (single_stream_ ? 1 : 0);
+  auto it = graphs_.find(key);
   if (it == graphs_.end()) {
     if (graphs_.size() >= kMaxGraphs) {
       LaunchEager(batch);
@@ -1606,16 +1609,17 @@ void Mi355xNetwork::ForwardDevice(int batch) {
       use_graphs_ = false;
       throw Error(std::string("HIP error: ") + hipGetErrorString(err) + " (hipGraphInstantiate)");
     }
-    it = graphs_.emplace(batch, exec).first;
+    it = graphs_.emplace(key, exec).first;
   }
   HIP_CHECK(hipGraphLaunch(it->second, stream_));
 }
 
-Mi355xNetwork* Mi355xNetwork::AcquireLane() {
+Mi355xNetwork* Mi355xNetwork::AcquireLane(bool* others_busy) {
   std::unique_lock<std::mutex> lock(lane_mutex_);
   lane_cv_.wait(lock, [&] { return !free_lanes_.empty(); });
   Mi355xNetwork* lane = free_lanes_.back();   // most recently used first
   free_lanes_.pop_back();
+  *others_busy = lane_count_ - static_cast<int>(free_lanes_.size()) > 1;
   return lane;
 }
 
@@ -1649,6 +1653,7 @@ void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {
   if (batch <= 0) return;
   if (profiling_.load()) {   // per-kernel timing records live in this object: run alone, on this lane
     AcquireAllLanes();
+    single_stream_ = false;
     try {
       EvaluateOnLane(slot, batch);
     } catch (...) {
@@ -1658,7 +1663,13 @@ void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {
     ReleaseAllLanes();
     return;
   }
-  Mi355xNetwork* lane = AcquireLane();
+  // A pass that starts while another lane is busy keeps to its main stream: the other passes fill the GPU,
+  // and two streams per lane are more than the hardware queues of the process (with 2 threads on the 15x1024
+  // net: batch 16 8.0k -> 14.2k evals/s, batch 64 24.9k -> 31.6k, batch 256 42.3k -> 44.9k). A lone pass
+  // uses the second stream as the batch-size rules say (single thread, batch 256: 41.8k against 38.1k without).
+  bool others_busy = false;
+  Mi355xNetwork* lane = AcquireLane(&others_busy);
+  lane->single_stream_ = others_busy && attn_body_;   // (a residual tower uses one stream anyway)
   try {
     lane->EvaluateOnLane(slot, batch);
   } catch (...) {
@@ -1735,6 +1746,7 @@ double Mi355xNetwork::TimeResidentForward(int batch, int iters) {
   HIP_CHECK(hipSetDevice(device_));
   const bool was_profiling = profiling_.load();
   profiling_ = false;
+  single_stream_ = false;
   hipEvent_t start = NewEvent(), stop = NewEvent();
   HIP_CHECK(hipEventRecord(start, stream_));
   for (int i = 0; i < iters; i++) ForwardDevice(batch);
