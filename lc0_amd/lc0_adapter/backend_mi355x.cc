@@ -12,7 +12,9 @@
 // Drop into an lc0 tree as src/neural/backends/mi355x/backend_mi355x.cc next to
 // network_mi355x.cc (register only one of the two under a given name) and link against
 // liblc0mi.so. It is not compiled as part of liblc0mi.so: it needs lc0's headers.
+#include <algorithm>
 #include <memory>
+#include <optional>
 #include <string>
 #include <vector>
 
@@ -20,6 +22,7 @@
 #include "neural/backend.h"
 #include "neural/encoder.h"
 #include "neural/loader.h"
+#include "neural/network.h"
 #include "neural/register.h"
 #include "neural/shared_params.h"
 #include "utils/exception.h"
@@ -78,7 +81,7 @@ class Mi355xBackendComputation : public BackendComputation {
 
 class Mi355xBackend : public Backend {
  public:
-  Mi355xBackend(const OptionsDict& options)
+  explicit Mi355xBackend(const OptionsDict& options)
       : backend_opts_(options.Get<std::string>(SharedBackendParams::kBackendOptionsId)),
         weights_path_(options.Get<std::string>(SharedBackendParams::kWeightsId)) {
     // --backend-opts of this backend are passed through as they are ("gpu=0,precision=fp8,...");
@@ -119,13 +122,13 @@ class Mi355xBackend : public Backend {
 
  private:
   friend class Mi355xBackendComputation;
+  const std::string backend_opts_;
+  const std::string weights_path_;
   lc0mi_net* net_ = nullptr;
   BackendAttributes attrs_;
   pblczero::NetworkFormat::InputFormat input_format_;
   float policy_temperature_ = 1.359f;
   FillEmptyHistory fill_empty_history_ = FillEmptyHistory::FEN_ONLY;
-  const std::string backend_opts_;
-  const std::string weights_path_;
 };
 
 Mi355xBackendComputation::Mi355xBackendComputation(Mi355xBackend* backend) : backend_(backend) {
