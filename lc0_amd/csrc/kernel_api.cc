@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -529,6 +530,97 @@ int lc0mi_k_expand_planes_nhwc(const uint64_t* masks, const float* values, int b
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());
     K_CHECK(hipMemcpy(out, dout, (size_t)batch * 64 * 112 * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+
+// ---------------------------------------------------------------------------
+// Split-K GEMM that allocates nothing. The float partial sums of the K slices,
+// which lc0mi_k_gemm_splitk keeps in a buffer it allocates per call, live in a
+// fixed array in device memory. In host code the array's name is only a handle
+// for hipGetSymbolAddress: the address kernels and copies use is looked up once
+// per device and kept in g_scratch_ptr.
+// ---------------------------------------------------------------------------
+}  // extern "C"
+
+namespace {
+constexpr long long kScratchFloats = 4ll << 20;  // 16 MiB on every device the library runs on
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) float scratch[kScratchFloats];
+float* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// The device's own copy of the array, with that device current.
+float* ScratchOfCurrentDevice() {
+  int dev = -1;
+  K_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) throw Error("device ordinal beyond the supported range");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    float* ptr = nullptr;
+    K_CHECK(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+    if (!ptr) throw Error("hipGetSymbolAddress returned a null scratch address");
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+// C[m][n] = part[0][m][n] + part[1][m][n] + ... in slice order, starting from 0.0f
+// like the host loop of lc0mi_k_gemm_splitk, so both give the same bits.
+__global__ __launch_bounds__(256) void sum_slices_kernel(const float* __restrict__ part, long long slice_stride,
+                                                         int slices, float* __restrict__ C, int M, int N, int ldc) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)M * N) return;
+  const int m = (int)(i / N), n = (int)(i - (long long)m * N);
+  const long long off = (long long)m * ldc + n;
+  float s = 0.0f;
+  for (int z = 0; z < slices; z++) s += part[z * slice_stride + off];
+  C[off] = s;
+}
+
+void RequireDevicePointer(const void* p, const char* what) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess || attr.type != hipMemoryTypeDevice) {
+    (void)hipGetLastError();
+    throw Error(std::string(what) + " is not a device pointer");
+  }
+}
+}  // namespace
+
+extern "C" {
+
+int lc0mi_k_gemm_splitk_noalloc(const uint16_t* dA, int lda, const uint16_t* dW, int ldw, const float* dbias, int M,
+                                int N, int K, int split_k, float scale, float* dC, int ldc, void* stream) {
+  return Guard([&] {
+    RequireDevice();
+    if (K < 8 || K % 8 || lda % 8 || ldw % 8) throw Error("K, lda and ldw must be multiples of 8");
+    if (M < 1 || N < 1 || split_k < 1 || lda < K || ldw < K || ldc < N) throw Error("bad gemm shape");
+    const long long c_elems = (long long)M * ldc;
+    if (c_elems * split_k > kScratchFloats)
+      throw Error("split-K partial sums need " + std::to_string(c_elems * split_k) + " floats; the fixed scratch array holds " +
+                  std::to_string(kScratchFloats));
+    if (!dA || !dW || !dC) throw Error("null operand");
+    RequireDevicePointer(dA, "A");
+    RequireDevicePointer(dW, "W");
+    RequireDevicePointer(dC, "C");
+    if (dbias) RequireDevicePointer(dbias, "bias");
+    if ((reinterpret_cast<uintptr_t>(dA) | reinterpret_cast<uintptr_t>(dW)) & 15) throw Error("A and W must be 16-byte aligned");
+    float* part = ScratchOfCurrentDevice();
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    lc0mi::GemmArgs g;
+    g.A = reinterpret_cast<const half_t*>(dA); g.lda = lda;
+    g.W = reinterpret_cast<const half_t*>(dW); g.ldw = ldw;
+    g.C = part; g.ldc = ldc;
+    g.bias = dbias;
+    g.M = M; g.N = N; g.K = K; g.scale = scale; g.act = 3; g.out_f32 = true;
+    g.split_k = split_k; g.split_stride = c_elems;
+    // Every (m < M, n < N) element of every slice is stored by the GEMM, so nothing of the previous call's
+    // contents is read and the array needs no clearing.
+    lc0mi::LaunchGemm(g, st);
+    const long long total = (long long)M * N;
+    hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part, c_elems, split_k,
+                       dC, M, N, ldc);
+    K_CHECK(hipGetLastError());
   });
 }
 
