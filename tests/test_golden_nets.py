@@ -58,3 +58,40 @@ def test_gpu_matches_the_fixture(name, options, tol, golden):
     assert np.abs(res["q"] - (want_wdl[:, 0] - want_wdl[:, 2])).max() <= tol
     assert np.abs(res["d"] - want_wdl[:, 1]).max() <= tol
     assert (np.abs(res["m"] - want_m) / np.maximum(np.abs(want_m), 1.0)).max() <= 2e-2
+
+
+def test_writer_schema_matches_reference_net_proto():
+    """Field numbers, nesting and repetition of lc0_amd.netproto.SCHEMA against proto/net.proto of the reference
+    (tests/golden/net_proto_fields.json, extracted from its text by tests/golden/make_net_proto_fields.py). The
+    oracle's reader and the product's reader are checked against files this writer produces, so this pins all
+    three views of the format."""
+    import json
+
+    from lc0_amd import netproto
+
+    golden = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "net_proto_fields.json")))
+    scalar = {"uint": ("uint32", "Encoding", "InputFormat", "OutputFormat", "NetworkStructure", "PolicyFormat",
+                       "ValueFormat", "MovesLeftFormat", "ActivationFunction", "DefaultActivation",
+                       "InputEmbeddingFormat"),
+              "float": ("float",), "bytes": ("bytes",), "string": ("string",), "fixed32": ("fixed32",)}
+    checked = 0
+    for message, fields in netproto.SCHEMA.items():
+        assert message in golden, message
+        for name, (number, kind) in fields.items():
+            ref = golden[message][name]
+            assert ref["number"] == number, (message, name)
+            repeated = kind.startswith("*")
+            assert (ref["label"] == "repeated") == repeated, (message, name)
+            kind = kind.lstrip("*")
+            if kind in scalar:
+                assert ref["type"] in scalar[kind], (message, name, ref["type"])
+            else:
+                assert ref["type"].split(".")[-1] == kind, (message, name, ref["type"])
+            checked += 1
+    assert checked >= 140
+    # the writer knows every field of the messages a weights file is made of
+    for message in ("Weights", "ConvBlock", "SEunit", "Residual", "Smolgen", "MHA", "FFN", "EncoderLayer",
+                    "PolicyHead", "PolicyHeads", "ValueHeads", "Layer", "NetworkFormat", "Format"):
+        # (the head maps are read by no backend: src/neural/network_legacy.cc:236-306)
+        missing = set(golden[message]) - set(netproto.SCHEMA[message]) - {"policy_head_map", "value_head_map"}
+        assert not missing, (message, missing)

@@ -338,7 +338,7 @@ def test_zero_smolgen_weights_equal_no_smolgen():
 
 def test_attention_policy_promotions_closed_form():
     """With a zero promotion matrix every promotion logit equals the plain
-    from->to logit; a constant row of ones in row p shifts only piece p."""
+    from->to logit."""
     g = netgen.CONFIGS["tiny_attn_nosmolgen"]()
     g["weights"]["ip4_pol_w"] = np.zeros_like(g["weights"]["ip4_pol_w"])
     bn = onn.BlasNetwork(nr.parse_net(netproto.serialize_net(g)))
@@ -349,6 +349,63 @@ def test_attention_policy_promotions_closed_form():
     idx = {s: i for i, s in enumerate(strs)}
     for s in strs[1792:]:
         np.testing.assert_allclose(pol[:, idx[s]], pol[:, idx[s[:4]]], rtol=1e-6)
+
+
+def test_attention_policy_promotion_offsets_closed_form():
+    """Non-zero promotion matrix (network_blas.cc:874-903). With Wk = 0 every key equals the bias vector c, so
+    promotion_offsets[i][j] = c . ip4_pol_w[i] for every file j: the logit of promoting to piece p exceeds the
+    plain from->to logit by exactly c . (row p + row 3). Rows chosen so that the three pieces get three
+    different shifts: a wrong piece index (3j+p), a missing `+= offsets[3]` or a row mix-up changes them."""
+    from oracle import chess as oc
+    g = netgen.CONFIGS["tiny_attn_nosmolgen"]()
+    w = g["weights"]
+    pd = w["ip3_pol_b"].size
+    rng = np.random.default_rng(11)
+    c = rng.standard_normal(pd).astype(f32)
+    w["ip3_pol_w"] = np.zeros_like(w["ip3_pol_w"])
+    w["ip3_pol_b"] = c
+    rows = rng.standard_normal((4, pd)).astype(f32)
+    w["ip4_pol_w"] = rows
+    pol = onn.BlasNetwork(nr.parse_net(netproto.serialize_net(g))).forward(*_random_inputs(3))["policy"]
+    shift = rows.astype(np.float64) @ c.astype(np.float64)           # c . row_i
+    strs = oc.move_strs()
+    idx = {s: i for i, s in enumerate(strs)}
+    seen = set()
+    for s in strs[1792:]:
+        piece = "qrb".index(s[4])
+        want = shift[piece] + shift[3]
+        got = pol[:, idx[s]].astype(np.float64) - pol[:, idx[s[:4]]]
+        np.testing.assert_allclose(got, want, rtol=0, atol=2e-5 * max(1.0, abs(want)))
+        seen.add(piece)
+    assert seen == {0, 1, 2}
+    assert min(abs(shift[a] - shift[b]) for a in range(3) for b in range(a)) > 1e-2   # the shifts tell pieces apart
+
+
+def test_se_unit_split_special_cases():
+    """ApplySEUnit (se_unit.cc:54-60): the first C outputs of the second dense layer are the sigmoid scale, the
+    next C the shift. (1) shift rows zero: out = act(sigma * (x + bias) + residual), sigma from rows 0..C-1;
+    (2) scale rows zero: sigma = 1/2 exactly, out = act(x/2 + residual + rows C..2C-1 + bias/2). Swapping the
+    halves turns one case into the other."""
+    rng = np.random.default_rng(4)
+    B, C, K = 2, 6, 3
+    x = rng.standard_normal((B, C, 64))
+    res = rng.standard_normal((B, C, 64))
+    bias = rng.standard_normal(C)
+    w1, b1 = rng.standard_normal((K, C)), rng.standard_normal(K)
+    w2, b2 = rng.standard_normal((2 * C, K)), rng.standard_normal(2 * C)
+    h = np.maximum((x.mean(axis=2) + bias) @ w1.T + b1, 0)          # dense 1 with ReLU on pooled + bias
+    call = lambda w2_, b2_: onn.apply_se_unit(x.astype(f32), bias.astype(f32), res.astype(f32), w1.astype(f32),
+                                              b1.astype(f32), w2_.astype(f32), b2_.astype(f32), nr.ACT_RELU)
+    w2a, b2a = w2.copy(), b2.copy()
+    w2a[C:], b2a[C:] = 0, 0
+    sigma = 1 / (1 + np.exp(-(h @ w2[:C].T + b2[:C])))
+    np.testing.assert_allclose(call(w2a, b2a), np.maximum(sigma[:, :, None] * (x + bias[None, :, None]) + res, 0),
+                               rtol=1e-4, atol=1e-5)
+    w2b, b2b = w2.copy(), b2.copy()
+    w2b[:C], b2b[:C] = 0, 0
+    shift = h @ w2[C:].T + b2[C:]
+    np.testing.assert_allclose(call(w2b, b2b),
+                               np.maximum(0.5 * x + res + (shift + 0.5 * bias)[:, :, None], 0), rtol=1e-4, atol=1e-5)
 
 
 def test_fast_exp_and_legal_softmax(ref):
