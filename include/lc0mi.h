@@ -111,6 +111,17 @@ int lc0mi_net_time_resident_forward(lc0mi_net* net, int batch, int iters, double
  * caller-supplied positions (same packed planes as lc0mi_comp_add_inputs). */
 int lc0mi_net_calibrate_fp8(lc0mi_net* net, int n, const uint64_t* masks, const float* values);
 
+/* ---- decoded weights (host only, needs no GPU) ----
+ * What the library reads from a weights file, for checking the loader: LayerAdapter decoding of the four
+ * Layer encodings (src/utils/weights_adapter.cc:38-62), the batch-norm fold of ConvBlock
+ * (src/neural/network_legacy.cc:62-131), the head resolution of MultiHeadWeights (:236-306) and the format
+ * upgrades of FixOlderWeightsFile (src/neural/loader.cc:108-158).
+ * lc0mi_weights_list writes "format key=value ..." and one "name count" line per non-empty tensor into buf
+ * (NUL-terminated, truncated to cap) and returns the bytes needed, -1 on error. */
+int lc0mi_weights_list(const void* data, size_t len, char* buf, int cap);
+/* Copies tensor `name` (as listed) into out (at most cap floats); returns its element count, -1 on error. */
+long long lc0mi_weights_tensor(const void* data, size_t len, const char* name, float* out, long long cap);
+
 /* ---- tables (closed forms of the tables under src/neural/tables, exposed for checking) ---- */
 /* kAttnPolicyMap (4288 entries), kConvPolicyMap (4672), kPosEncoding (64*64). */
 const int16_t* lc0mi_attn_policy_map(int* count);

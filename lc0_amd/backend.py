@@ -68,6 +68,9 @@ def load_library():
     lib.lc0mi_net_take_profile.argtypes = [vp, C.c_char_p, ci]
     lib.lc0mi_net_time_resident_forward.argtypes = [vp, ci, ci, C.POINTER(C.c_double)]
     lib.lc0mi_net_calibrate_fp8.argtypes = [vp, ci, vp, vp]
+    lib.lc0mi_weights_list.argtypes = [vp, C.c_size_t, C.c_char_p, ci]
+    lib.lc0mi_weights_tensor.argtypes = [vp, C.c_size_t, C.c_char_p, vp, C.c_longlong]
+    lib.lc0mi_weights_tensor.restype = C.c_longlong
     for name, typ in (("lc0mi_attn_policy_map", C.c_int16), ("lc0mi_conv_policy_map", C.c_int16),
                       ("lc0mi_pos_encoding", cf)):
         getattr(lib, name).argtypes = [C.POINTER(ci)]
@@ -86,6 +89,29 @@ def _table(fn_name, dtype):
     n = C.c_int(0)
     ptr = getattr(lib, fn_name)(C.byref(n))
     return np.ctypeslib.as_array(ptr, (n.value,)).astype(dtype).copy()
+
+
+def decoded_weights(data):
+    """What the library reads from serialized (raw or gzip) pblczero.Net bytes, without a GPU:
+    (format dict, {tensor name: float32 array}); heads resolved, batch norm folded."""
+    lib = load_library()
+    data = bytes(data)
+    need = lib.lc0mi_weights_list(data, len(data), None, 0)
+    if need < 0:
+        raise BackendError(lib.lc0mi_last_error().decode(errors="replace"))
+    buf = C.create_string_buffer(need)
+    lib.lc0mi_weights_list(data, len(data), buf, need)
+    lines = buf.value.decode().splitlines()
+    fmt = {k: int(v) for k, v in (kv.split("=") for kv in lines[0].split()[1:])}
+    tensors = {}
+    for line in lines[1:]:
+        name, count = line.split()
+        arr = np.zeros(int(count), np.float32)
+        got = lib.lc0mi_weights_tensor(data, len(data), name.encode(), arr.ctypes.data, arr.size)
+        if got != arr.size:
+            raise BackendError("tensor %s: expected %d elements, got %d" % (name, arr.size, got))
+        tensors[name] = arr
+    return fmt, tensors
 
 
 def attn_policy_map():

@@ -2,6 +2,7 @@
 // codes plus a thread-local message and owns the opaque handles.
 #include "../../include/lc0mi.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -223,6 +224,128 @@ int lc0mi_net_calibrate_fp8(lc0mi_net* net, int n, const uint64_t* masks, const 
     if (!net) throw lc0mi::Error("null network");
     net->impl->CalibrateFp8(n, masks, values);
   });
+}
+
+}  // extern "C"
+
+// ---- decoded weights, for checking the loader without a GPU ----
+namespace {
+template <typename F>
+void VisitConv(const std::string& name, const lc0mi::ConvBlock& c, F&& f) {
+  f(name + ".weights", c.weights);
+  f(name + ".biases", c.biases);
+}
+template <typename F>
+void VisitEncoder(const std::string& name, const lc0mi::EncoderLayer& l, F&& f) {
+  f(name + ".mha.q_w", l.mha.q_w); f(name + ".mha.q_b", l.mha.q_b);
+  f(name + ".mha.k_w", l.mha.k_w); f(name + ".mha.k_b", l.mha.k_b);
+  f(name + ".mha.v_w", l.mha.v_w); f(name + ".mha.v_b", l.mha.v_b);
+  f(name + ".mha.dense_w", l.mha.dense_w); f(name + ".mha.dense_b", l.mha.dense_b);
+  if (l.mha.has_smolgen) {
+    const auto& s = l.mha.smolgen;
+    f(name + ".mha.smolgen.compress", s.compress);
+    f(name + ".mha.smolgen.dense1_w", s.dense1_w); f(name + ".mha.smolgen.dense1_b", s.dense1_b);
+    f(name + ".mha.smolgen.ln1_gammas", s.ln1_gammas); f(name + ".mha.smolgen.ln1_betas", s.ln1_betas);
+    f(name + ".mha.smolgen.dense2_w", s.dense2_w); f(name + ".mha.smolgen.dense2_b", s.dense2_b);
+    f(name + ".mha.smolgen.ln2_gammas", s.ln2_gammas); f(name + ".mha.smolgen.ln2_betas", s.ln2_betas);
+  }
+  f(name + ".ln1_gammas", l.ln1_gammas); f(name + ".ln1_betas", l.ln1_betas);
+  f(name + ".ffn.dense1_w", l.ffn.dense1_w); f(name + ".ffn.dense1_b", l.ffn.dense1_b);
+  f(name + ".ffn.dense2_w", l.ffn.dense2_w); f(name + ".ffn.dense2_b", l.ffn.dense2_b);
+  f(name + ".ln2_gammas", l.ln2_gammas); f(name + ".ln2_betas", l.ln2_betas);
+}
+// Calls f(name, tensor) for every tensor of the file, heads resolved and batch norm folded.
+template <typename F>
+void VisitTensors(const lc0mi::NetWeights& w, F&& f) {
+  VisitConv("input", w.input, f);
+  for (size_t i = 0; i < w.residual.size(); i++) {
+    const std::string n = "residual." + std::to_string(i);
+    VisitConv(n + ".conv1", w.residual[i].conv1, f);
+    VisitConv(n + ".conv2", w.residual[i].conv2, f);
+    if (w.residual[i].has_se) {
+      f(n + ".se.w1", w.residual[i].se.w1); f(n + ".se.b1", w.residual[i].se.b1);
+      f(n + ".se.w2", w.residual[i].se.w2); f(n + ".se.b2", w.residual[i].se.b2);
+    }
+  }
+  f("ip_emb_preproc_w", w.ip_emb_preproc_w); f("ip_emb_preproc_b", w.ip_emb_preproc_b);
+  f("ip_emb_w", w.ip_emb_w); f("ip_emb_b", w.ip_emb_b);
+  f("ip_emb_ln_gammas", w.ip_emb_ln_gammas); f("ip_emb_ln_betas", w.ip_emb_ln_betas);
+  f("ip_mult_gate", w.ip_mult_gate); f("ip_add_gate", w.ip_add_gate);
+  f("ip_emb_ffn.dense1_w", w.ip_emb_ffn.dense1_w); f("ip_emb_ffn.dense1_b", w.ip_emb_ffn.dense1_b);
+  f("ip_emb_ffn.dense2_w", w.ip_emb_ffn.dense2_w); f("ip_emb_ffn.dense2_b", w.ip_emb_ffn.dense2_b);
+  f("ip_emb_ffn_ln_gammas", w.ip_emb_ffn_ln_gammas); f("ip_emb_ffn_ln_betas", w.ip_emb_ffn_ln_betas);
+  for (size_t i = 0; i < w.encoder.size(); i++) VisitEncoder("encoder." + std::to_string(i), w.encoder[i], f);
+  VisitConv("moves_left", w.moves_left, f);
+  f("ip_mov_w", w.ip_mov_w); f("ip_mov_b", w.ip_mov_b);
+  f("ip1_mov_w", w.ip1_mov_w); f("ip1_mov_b", w.ip1_mov_b);
+  f("ip2_mov_w", w.ip2_mov_w); f("ip2_mov_b", w.ip2_mov_b);
+  f("smolgen_w", w.smolgen_w);
+  for (const auto& kv : w.policy_heads) {
+    const std::string n = "policy_heads." + kv.first;
+    const auto& h = kv.second;
+    f(n + ".ip_pol_w", h.ip_pol_w); f(n + ".ip_pol_b", h.ip_pol_b);
+    VisitConv(n + ".policy1", h.policy1, f);
+    VisitConv(n + ".policy", h.policy, f);
+    f(n + ".ip2_pol_w", h.ip2_pol_w); f(n + ".ip2_pol_b", h.ip2_pol_b);
+    f(n + ".ip3_pol_w", h.ip3_pol_w); f(n + ".ip3_pol_b", h.ip3_pol_b);
+    f(n + ".ip4_pol_w", h.ip4_pol_w);
+    for (size_t i = 0; i < h.pol_encoder.size(); i++) VisitEncoder(n + ".pol_encoder." + std::to_string(i), h.pol_encoder[i], f);
+  }
+  for (const auto& kv : w.value_heads) {
+    const std::string n = "value_heads." + kv.first;
+    const auto& h = kv.second;
+    VisitConv(n + ".value", h.value, f);
+    f(n + ".ip_val_w", h.ip_val_w); f(n + ".ip_val_b", h.ip_val_b);
+    f(n + ".ip1_val_w", h.ip1_val_w); f(n + ".ip1_val_b", h.ip1_val_b);
+    f(n + ".ip2_val_w", h.ip2_val_w); f(n + ".ip2_val_b", h.ip2_val_b);
+  }
+}
+}  // namespace
+
+extern "C" {
+
+int lc0mi_weights_list(const void* data, size_t len, char* buf, int cap) {
+  int needed = -1;
+  const int rc = Guard([&] {
+    if (!data) throw lc0mi::Error("null argument");
+    std::string raw = lc0mi::MaybeGunzip(data, len);
+    const lc0mi::WeightsFile file = lc0mi::ParseWeightsProto(raw.data(), raw.size());
+    const auto& nf = file.format;
+    std::string text = "format input=" + std::to_string(nf.input) + " output=" + std::to_string(nf.output) +
+                       " network=" + std::to_string(nf.network) + " policy=" + std::to_string(nf.policy) +
+                       " value=" + std::to_string(nf.value) + " moves_left=" + std::to_string(nf.moves_left) +
+                       " default_activation=" + std::to_string(nf.default_activation) +
+                       " smolgen_activation=" + std::to_string(nf.smolgen_activation) +
+                       " ffn_activation=" + std::to_string(nf.ffn_activation) +
+                       " input_embedding=" + std::to_string(nf.input_embedding) +
+                       " headcount=" + std::to_string(file.weights.encoder_head_count) + "\n";
+    VisitTensors(file.weights, [&](const std::string& name, const lc0mi::Vec& v) {
+      if (!v.empty()) text += name + " " + std::to_string(v.size()) + "\n";
+    });
+    needed = static_cast<int>(text.size()) + 1;
+    if (buf && cap > 0) {
+      const size_t n = std::min<size_t>(text.size(), static_cast<size_t>(cap) - 1);
+      std::memcpy(buf, text.data(), n);
+      buf[n] = 0;
+    }
+  });
+  return rc ? -1 : needed;
+}
+
+long long lc0mi_weights_tensor(const void* data, size_t len, const char* name, float* out, long long cap) {
+  long long count = -1;
+  const int rc = Guard([&] {
+    if (!data || !name) throw lc0mi::Error("null argument");
+    std::string raw = lc0mi::MaybeGunzip(data, len);
+    const lc0mi::WeightsFile file = lc0mi::ParseWeightsProto(raw.data(), raw.size());
+    VisitTensors(file.weights, [&](const std::string& n, const lc0mi::Vec& v) {
+      if (n != name) return;
+      count = static_cast<long long>(v.size());
+      if (out) std::memcpy(out, v.data(), sizeof(float) * static_cast<size_t>(std::min<long long>(count, cap)));
+    });
+    if (count < 0) throw lc0mi::Error(std::string("no tensor named ") + name);
+  });
+  return rc ? -1 : count;
 }
 
 const int16_t* lc0mi_attn_policy_map(int* count) {

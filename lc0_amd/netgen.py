@@ -222,6 +222,58 @@ def _with_input_format(net, input_format):
     return net
 
 
+def with_batch_norm(net, seed):
+    """Adds batch-norm statistics to every convolution block, the form older nets are stored in
+    (src/neural/network_legacy.cc:62-131 folds them at load). The first residual block's conv1 takes the oldest
+    form: no biases and no gammas/betas; its conv2 has biases but no gammas/betas."""
+    g = _Gen(seed)
+
+    def bn(block, old=0):
+        n = block["biases"].size
+        block["bn_means"] = g.normal((n,), 0.1)
+        block["bn_stddivs"] = (0.5 + g.rng.random(n)).astype(np.float32)
+        if old == 0:
+            block["bn_gammas"] = 1.0 + g.normal((n,), 0.1)
+            block["bn_betas"] = g.normal((n,), 0.1)
+        if old == 2:
+            del block["biases"]
+
+    w = net["weights"]
+    bn(w["input"])
+    for i, r in enumerate(w["residual"]):
+        bn(r["conv1"], old=2 if i == 0 else 0)
+        bn(r["conv2"], old=1 if i == 0 else 0)
+    for key in ("policy1", "policy", "value", "moves_left"):
+        if key in w:
+            bn(w[key])
+    return net
+
+
+def with_classical_value(net, seed):
+    """Scalar tanh value head (VALUE_CLASSICAL, src/neural/backends/blas/network_blas.cc:763-771)."""
+    g = _Gen(seed)
+    w = net["weights"]
+    fan_in = w["ip2_val_w"].shape[1]
+    w["ip2_val_w"] = g.normal((1, fan_in), fan_in ** -0.5)
+    w["ip2_val_b"] = g.normal((1,), 0.02)
+    net["format"]["network_format"]["value"] = 1
+    net["format"]["network_format"]["output"] = 1
+    return net
+
+
+def _old_format(net, network=None, drop=()):
+    """Rewrites the format block the way files written before a format revision look; the loader's
+    FixOlderWeightsFile (src/neural/loader.cc:108-158) has one branch per case."""
+    nf = net["format"]["network_format"]
+    if network is None:
+        del net["format"]["network_format"]
+    else:
+        nf["network"] = network
+        for key in drop:
+            nf.pop(key, None)
+    return net
+
+
 # The benchmark configurations (name -> builder). Seeds are part of the spec.
 CONFIGS = {
     # 6 blocks x 64 filters SE-ResNet, SE ratio 4, classical policy, WDL.
@@ -258,6 +310,31 @@ CONFIGS = {
     "tiny_attn_dense_f8": lambda: attention_body(128, 2, 4, 256, seed=2010, smolgen=(8, 32, 32), perturb_ln=True, std=0.07,
                                                  pe_dense=(16, 128), gating=True, multihead=True),
     "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True, std=0.1),
+    # ---- what real files contain beyond FLOAT32 layers of the current format ----
+    # batch-norm statistics on every convolution block, incl. the bias-less and gamma-less old forms
+    "tiny_resnet_bn": lambda: with_batch_norm(se_resnet(32, 2, 8, seed=2012, moves_left=True), seed=3012),
+    "tiny_resnet_convpolicy_bn": lambda: with_batch_norm(se_resnet(32, 2, 8, seed=2013, conv_policy=True), seed=3013),
+    # scalar tanh value head
+    "tiny_resnet_classical_value": lambda: with_classical_value(se_resnet(32, 2, 8, seed=2014), seed=3014),
+    # no network_format at all: plain residual tower, classical heads (loader.cc:115-121)
+    "old_noformat": lambda: _old_format(with_classical_value(se_resnet(24, 2, 0, seed=2015), seed=3015)),
+    # NETWORK_CLASSICAL (1) and NETWORK_SE (2): head formats are implied (loader.cc:122-132)
+    "old_classical": lambda: _old_format(with_classical_value(se_resnet(24, 2, 0, seed=2016), seed=3016), network=1,
+                                         drop=("policy", "value")),
+    "old_se": lambda: _old_format(with_batch_norm(with_classical_value(se_resnet(24, 2, 8, seed=2017), seed=3017), seed=4017),
+                                  network=2, drop=("policy", "value")),
+    # attention body stored as SE_WITH_HEADFORMAT with smolgen: squared-ReLU FFN and swish are implied (:133-142)
+    "old_attn_as_se": lambda: _old_format(
+        attention_body(64, 2, 2, 96, seed=2018, smolgen=(8, 32, 32), perturb_ln=True, std=0.1), network=4,
+        drop=("smolgen_activation", "ffn_activation", "input_embedding")),
+    # NETWORK_AB_LEGACY_WITH_MULTIHEADFORMAT (134) (:143-145)
+    "old_ab_legacy": lambda: _old_format(
+        attention_body(64, 2, 2, 96, seed=2019, smolgen=(8, 32, 32), perturb_ln=True, pe_dense=(16, 128),
+                       multihead=True, std=0.1), network=134),
+    # format 6 carrying policy_heads and value_heads: becomes format 7 with PE_DENSE (:148-154)
+    "old_format6_with_heads": lambda: _old_format(
+        attention_body(64, 2, 2, 96, seed=2020, smolgen=(8, 32, 32), perturb_ln=True, pe_dense=(16, 128),
+                       multihead=True, std=0.1), network=6, drop=("input_embedding",)),
     # canonical input format with hectoplies: board transforms, en-passant plane, fractional rule-50 plane values
     "tiny_attn_canonical": lambda: _with_input_format(
         attention_body(64, 2, 2, 96, seed=2011, smolgen=(8, 32, 32), perturb_ln=True, std=0.1),
@@ -266,23 +343,29 @@ CONFIGS = {
 
 
 # Part of the cache file name: bump when a generator or a configuration changes.
-CACHE_VERSION = "-g3"
+CACHE_VERSION = "-g4"
 
 
-def write_config(name, path):
-    """Generates config `name` into `path` (a .pb.gz); returns the path."""
+ENCODINGS = {"float32": netproto.FLOAT32, "linear16": netproto.LINEAR16, "float16": netproto.FLOAT16,
+             "bfloat16": netproto.BFLOAT16}
+
+
+def write_config(name, path, encoding="float32"):
+    """Generates config `name` into `path` (a .pb.gz) with every layer stored in `encoding`
+    (Weights.Layer.Encoding, proto/net.proto:42-48; real lc0 files use LINEAR16); returns the path."""
     net = CONFIGS[name]()
-    netproto.write_pb_gz(path, net)
+    netproto.write_pb_gz(path, net, layer_encoding=ENCODINGS[encoding])
     return path
 
 
-def cached_config(name, cache_dir=None):
+def cached_config(name, cache_dir=None, encoding="float32"):
     """Path of the generated file for `name`, generating it on first use."""
     cache_dir = cache_dir or os.environ.get("LC0MI_NET_CACHE", "/tmp/lc0mi_nets")
     os.makedirs(cache_dir, exist_ok=True)
-    path = os.path.join(cache_dir, name + CACHE_VERSION + ".pb.gz")
+    suffix = "" if encoding == "float32" else "-" + encoding
+    path = os.path.join(cache_dir, name + suffix + CACHE_VERSION + ".pb.gz")
     if not os.path.exists(path):
         tmp = path + ".tmp%d" % os.getpid()
-        write_config(name, tmp)
+        write_config(name, tmp, encoding)
         os.replace(tmp, path)
     return path

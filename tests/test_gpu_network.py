@@ -97,6 +97,42 @@ def test_residual_tower_nets_match_oracle(name, batch, options, tol, positions):
     _compare(res, want, positions["legal"][:batch], tol=tol)
 
 
+@pytest.mark.parametrize("name,encoding,options,tol", [
+    # the four Layer encodings (real lc0 files are LINEAR16)
+    ("tiny_attn", "linear16", "", 5e-3), ("tiny_attn", "float16", "", 5e-3), ("tiny_attn", "bfloat16", "", 5e-3),
+    ("tiny_attn_dense", "linear16", "", 5e-3),
+    # batch-norm statistics in the file (folded at load), incl. the bias-less and gamma-less old forms
+    ("tiny_resnet_bn", "linear16", "precision=fp32", 1e-3), ("tiny_resnet_bn", "float32", "precision=fp16", 5e-3),
+    ("tiny_resnet_convpolicy_bn", "float32", "precision=fp32", 1e-3),
+    # scalar tanh value head
+    ("tiny_resnet_classical_value", "float32", "precision=fp32", 1e-3),
+    ("tiny_resnet_classical_value", "linear16", "precision=fp16", 5e-3),
+    # one file per branch of FixOlderWeightsFile
+    ("old_noformat", "linear16", "precision=fp32", 1e-3), ("old_classical", "float32", "precision=fp32", 1e-3),
+    ("old_se", "linear16", "precision=fp32", 1e-3), ("old_attn_as_se", "linear16", "", 5e-3),
+    ("old_ab_legacy", "float32", "", 5e-3), ("old_format6_with_heads", "linear16", "", 5e-3)])
+def test_file_forms_of_real_nets_match_oracle(name, encoding, options, tol, positions):
+    """Layer encodings (src/utils/weights_adapter.cc:38-62), batch-norm fold (src/neural/network_legacy.cc:62-131),
+    classical value head (src/neural/backends/blas/network_blas.cc:763-771) and older file formats
+    (src/neural/loader.cc:108-158): the GPU backend and the oracle read the same file."""
+    batch = 11
+    path = netgen.cached_config(name, encoding=encoding)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    ref_net = nr.load(path)
+    want = onn.BlasNetwork(ref_net).forward(masks, values)
+    net, res = _run_gpu(path, masks, values, options)
+    caps = net.GetCapabilities()
+    assert (caps.input_format, caps.output_format, caps.moves_left) == \
+        (ref_net.format.input, ref_net.format.output, ref_net.format.moves_left)
+    if "wdl" not in want:
+        # GetQVal = tanh value, GetDVal = 0
+        assert float(np.abs(res["q"] - want["q"]).max()) <= tol
+        assert float(np.abs(res["d"]).max()) == 0.0
+        q = want["q"]
+        want["wdl"] = np.stack([(1 + q) / 2, np.zeros_like(q), (1 - q) / 2], axis=1)   # so that _compare sees the same q, d
+    _compare(res, want, positions["legal"][:batch], tol=tol)
+
+
 @pytest.mark.timeout(900)
 def test_bt4_shape_batch_256(positions):
     """configs[2]: oracle comparison on the first 48 positions (seconds of CPU
