@@ -3,7 +3,9 @@
 Metric (BASELINE.json): NN evals/sec at batch 256 on the BT4-shape fp16 net,
 with the dominant kernel's fraction of the MFMA roofline and the CPU oracle's
 evals/sec on the same host next to it. A "step" is one device pass over one
-batch of 256 seeded random-playout positions already resident in HBM.
+batch of 256 seeded random-playout positions already resident in HBM: `value` is
+that rate. The same path with the host copies (H2D of the planes, D2H of the
+outputs) is printed next to it as `with_host_io_evals_per_s`.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--batch B]
 """
@@ -21,14 +23,20 @@ PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA peak
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA peak
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 
-# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration) measured with
-# rocprofv3 --pmc on this same command; counters cannot be read from inside the process, so the figures
-# recorded under profiles/ are repeated here: (workload, batch, kernel) -> bytes.
-MEASURED_TRAFFIC = {
-    ("c2_bt4_15x1024", 256, "gemm_dma_256x256x64"): (72883 + 57204) * 1024,
-    ("c2_bt4_15x1024", 256, "gemm_dma_256x192x64"): (90144 + 54721) * 1024,
-    ("c2_bt4_15x1024", 256, "attention"): (163959 + 32769) * 1024,
-}
+# HBM bytes per launch of a kernel cannot be read from inside the process: they come from two rocprofv3 --pmc
+# runs of this same command (FETCH_SIZE, WRITE_SIZE, scaled by the copy-kernel calibration). The summary of such
+# a run is a small JSON file {"workload", "batch", "source", "kernels": {kernel: bytes per launch}}; when one
+# for this workload and batch is given (or sits under profiles/), roofline.traffic is taken from it, else null.
+def measured_traffic(path, workload, batch, kernel):
+    path = path or os.path.join(ROOT, "profiles", "hbm_traffic_%s_batch%d.txt" % (workload, batch))
+    try:
+        rec = json.load(open(path))
+    except (OSError, ValueError):
+        return None, None
+    if rec.get("workload") != workload or rec.get("batch") != batch:
+        return None, None
+    return rec.get("kernels", {}).get(kernel), rec.get("source")
+
 
 WORKLOADS = {
     "c2_bt4_15x1024": dict(batch=256, desc="BT4-shape attention body: 15 layers, d=1024, 32 heads, dff 1536, "
@@ -46,25 +54,53 @@ WORKLOADS = {
 }
 
 
-def cpu_baseline(path, masks, values, sample, seconds_budget=25.0):
-    """Oracle (numpy/BLAS restatement of the blas backend) timed on this host."""
+def _host_description():
+    model = "unknown CPU"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    blas = "numpy's bundled BLAS"
+    try:
+        from threadpoolctl import threadpool_info
+        libs = ["%s %s (%s threads)" % (i.get("internal_api"), i.get("version"), i.get("num_threads"))
+                for i in threadpool_info() if i.get("user_api") == "blas"]
+        if libs:
+            blas = ", ".join(libs)
+    except ImportError:
+        pass
+    return model, blas
+
+
+def cpu_baseline(path, masks, values, batch, sample=0, seconds_budget=27.0):
+    """Oracle (numpy/BLAS restatement of the blas backend) timed on this host: three timed passes over one
+    sample of the workload's batch (the whole batch when three passes fit the time budget)."""
     from oracle import netread as nr
     from oracle import nn as onn
-    bn = onn.BlasNetwork(nr.load(path))
+    bn = onn.BlasNetwork(nr.load(path), batch_size=max(batch, 1))
+    bn.forward(masks[:2], values[:2])  # warm-up
+    if not sample:
+        probe = min(8, batch)
+        t0 = time.perf_counter()
+        bn.forward(masks[:probe], values[:probe])
+        rate = probe / (time.perf_counter() - t0)
+        sample = int(max(probe, min(batch, rate * seconds_budget / 3.0)))
     m, v = masks[:sample], values[:sample]
-    bn.forward(m[:2], v[:2])  # warm-up
     times = []
-    t_end = time.time() + seconds_budget
-    while len(times) < 3 or (time.time() < t_end and len(times) < 10):
+    for _ in range(3):
         t0 = time.perf_counter()
         bn.forward(m, v)
         times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    model, blas = _host_description()
     out = {"value": sample / med, "unit": "evals/s", "cores": cores, "kind": "port",
-           "sample": "%d positions per pass, %d timed passes, median; numpy float32 + its bundled BLAS sgemm"
-                     % (sample, len(times))}
+           "sample": "%d of the batch's %d positions per pass, 3 timed passes, median; numpy float32, sgemm of %s; %s"
+                     % (sample, batch, blas, model)}
     # The reference blas backend defaults to one thread (network_blas.cc:994): same oracle, BLAS pinned to 1 thread.
     try:
         from threadpoolctl import threadpool_limits
@@ -72,7 +108,7 @@ def cpu_baseline(path, masks, values, sample, seconds_budget=25.0):
         with threadpool_limits(limits=1):
             bn.forward(m[:1], v[:1])
             t1 = []
-            t_end = time.time() + 8.0
+            t_end = time.time() + 6.0
             while len(t1) < 2 or (time.time() < t_end and len(t1) < 5):
                 t0 = time.perf_counter()
                 bn.forward(m[:small], v[:small])
@@ -93,7 +129,10 @@ def main():
     ap.add_argument("--config", default="c2_bt4_15x1024", choices=sorted(WORKLOADS))
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-sample", type=int, default=16)
+    ap.add_argument("--cpu-sample", type=int, default=0, help="positions per CPU pass (0: as many of the batch as "
+                                                              "three passes fit in about 27 s)")
+    ap.add_argument("--traffic-json", default="", help="HBM bytes per launch from a rocprofv3 --pmc run of this command "
+                                                       "(default: profiles/hbm_traffic_<config>_batch<B>.txt if present)")
     ap.add_argument("--sweep", default="", help="comma-separated batch sizes: adds their resident-batch evals/s "
                                                 "as \"batch_sweep\" to the JSON line")
     args = ap.parse_args()
@@ -212,7 +251,7 @@ def main():
                     "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
                     "avg_launch_ms": dom.ms / dom.launches, "launches_per_step": dom.launches // prof_iters}
 
-    roofline["traffic"] = MEASURED_TRAFFIC.get((args.config, batch, dom.name))
+    roofline["traffic"], roofline["traffic_source"] = measured_traffic(args.traffic_json, args.config, batch, dom.name)
     roofline["algorithmic_bytes"] = dom.bytes / dom.launches if dom.bytes else None
 
     result = {
@@ -255,7 +294,7 @@ def main():
             result["batch_sweep"][str(b)] = {"evals_per_s": b / (ms * 1e-3), "ms_per_step": ms}
             c.close()
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(path, masks, values, args.cpu_sample)
+        result["cpu_baseline"] = cpu_baseline(path, masks, values, batch, args.cpu_sample)
     print(json.dumps(result))
 
 

@@ -408,6 +408,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   void AcquireAllLanes();
   void ReleaseAllLanes();
   void EvaluateOnLane(HostSlot* slot, int batch);
+  void DrainStreams();
   void CreateStreams();
   void AllocActivations();
 
@@ -1657,6 +1658,7 @@ void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {
     try {
       EvaluateOnLane(slot, batch);
     } catch (...) {
+      DrainStreams();
       ReleaseAllLanes();
       throw;
     }
@@ -1673,14 +1675,28 @@ void Mi355xNetwork::Evaluate(HostSlot* slot, int batch) {
   try {
     lane->EvaluateOnLane(slot, batch);
   } catch (...) {
+    lane->DrainStreams();
     ReleaseLane(lane);
     throw;
   }
   ReleaseLane(lane);
 }
 
+// After a failed pass work may still be queued on the lane's streams (copies from the pinned slot, kernels on the
+// lane's buffers): wait for it, ignoring errors, before the lane and the slot are reused.
+void Mi355xNetwork::DrainStreams() {
+  (void)hipSetDevice(device_);
+  if (stream_) (void)hipStreamSynchronize(stream_);
+  if (side_stream_) (void)hipStreamSynchronize(side_stream_);
+  (void)hipGetLastError();
+}
+
 void Mi355xNetwork::EvaluateOnLane(HostSlot* slot, int batch) {
   std::lock_guard<std::mutex> lock(eval_mutex_);
+  // Argument errors are reported before anything is enqueued: the lane's streams stay idle.
+  if (slot->legal_samples > 0 && slot->legal_samples != batch) {
+    throw Error("legal moves were given for some inputs of the batch only");
+  }
   HIP_CHECK(hipSetDevice(device_));
   HIP_CHECK(hipMemcpyAsync(d_masks_, slot->masks, sizeof(uint64_t) * kInputPlanes * batch, hipMemcpyHostToDevice,
                            stream_));
@@ -1688,7 +1704,6 @@ void Mi355xNetwork::EvaluateOnLane(HostSlot* slot, int batch) {
                            stream_));
   const bool legal = slot->legal_samples > 0;
   if (legal) {
-    if (slot->legal_samples != batch) throw Error("legal moves were given for some inputs of the batch only");
     const int total = slot->legal_off[batch];
     HIP_CHECK(hipMemcpyAsync(d_legal_off_, slot->legal_off, sizeof(int) * (batch + 1), hipMemcpyHostToDevice, stream_));
     if (total > 0) {
