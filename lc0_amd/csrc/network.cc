@@ -279,6 +279,7 @@ struct ModelState {
   // fp8 configuration: the four large GEMMs of every encoder layer run on e4m3 operands.
   bool fp8_ = false;
   bool q_qkv_ = true, q_dense_ = true, q_ffn1_ = true, q_ffn2_ = true;   // option fp8_gemms
+  int fp8_fp16_layers_ = 0;   // option fp8_fp16_layers: the last that many encoder layers keep fp16 operands
 
   // Residual tower.
   bool fp32_ = false;
@@ -751,6 +752,8 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
       pos = end + 1;
     }
   }
+  fp8_fp16_layers_ = options.GetInt("fp8_fp16_layers", 0);
+  if (fp8_fp16_layers_ < 0) throw Error("fp8_fp16_layers must not be negative.");
   use_graphs_ = options.GetBool("graphs", true);
   // Running the smolgen chain beside the QKV projection costs two cross-queue dependencies per layer; below
   // these batch sizes the chain on the main stream is faster (measured on the 15x1024 net: fp16 batch 1
@@ -1436,11 +1439,13 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       LaunchLayerNorm(t_, x_, x_, emb_ffn_ln_g_, emb_ffn_ln_b_, T, emb_, alpha_, 1e-3f, stream_);
     });
   }
-  // fp8: the large GEMMs read e4m3 operands written by the kernel that produces each tensor.
-  const bool f8 = fp8_ && !calibrating_;
+  // fp8: the large GEMMs read e4m3 operands written by the kernel that produces each tensor. The last
+  // fp8_fp16_layers_ layers (closest to the heads) can be kept in fp16.
+  const bool f8_any = fp8_ && !calibrating_;
+  const size_t n_f8_layers = encoders_.size() - std::min<size_t>(encoders_.size(), static_cast<size_t>(fp8_fp16_layers_));
   const size_t nx = static_cast<size_t>(T) * emb_;
   if (calibrating_) RecordAbsMax(x_, nx, 0);
-  if (f8 && q_qkv_) {
+  if (f8_any && n_f8_layers > 0 && q_qkv_) {
     Timed("quantize_f8", 0.0, 3.0 * nx,
           [&] { LaunchQuantizeF8(x_, xq_, static_cast<long long>(nx), 1.0f / encoders_[0].s_x, stream_); });
   }
@@ -1448,6 +1453,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
   for (size_t li = 0; li < encoders_.size(); li++) {
     const EncoderDev& e = encoders_[li];
     const bool last = li + 1 == encoders_.size();
+    const bool f8 = f8_any && li < n_f8_layers;
     const half_t* bias = nullptr;
     // The smolgen chain depends only on x: it runs on the side stream next to the
     // QKV projection (on the main stream when profiling, for clean per-kernel times).
@@ -1525,7 +1531,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     } else {
       Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, t_, emb_, T, kActNone);
     }
-    const bool ln2_f8 = f8 && q_qkv_ && !last;
+    const bool ln2_f8 = f8_any && li + 1 < n_f8_layers && q_qkv_;   // the next layer reads an e4m3 copy
     Timed("layer_norm_skip", 0.0, (ln2_f8 ? 7.0 : 6.0) * T * emb_, [&] {
       LaunchLayerNorm(t_, x_, x_, e.ln2_g, e.ln2_b, T, emb_, alpha_, eps_, stream_, ln2_f8 ? xq_ : nullptr,
                       last ? 1.0f : 1.0f / encoders_[li + 1].s_x);
