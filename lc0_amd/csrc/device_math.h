@@ -1,0 +1,37 @@
+// Device-side activation functions shared by the kernel sources.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace lc0mi {
+
+// lc0's ActivationFunction numbering (src/neural/tables/activation_function.h:24-35).
+enum : int { kActMish = 1, kActRelu = 2, kActNone = 3, kActTanh = 4, kActSigmoid = 5, kActSelu = 6, kActSwish = 7,
+             kActRelu2 = 8 };
+
+// Activation functions (values as shared/activation.cc:51-100). The GEMM epilogues are bound by
+// vector-ALU issue, so mish and swish use one hardware exponential and one hardware reciprocal
+// (1 ulp each) instead of a correctly rounded division:
+//   mish(v) = v * tanh(log(1 + e^v)) = v * n / (n + 2),  n = e^v * (e^v + 2).
+// The exponent is clamped at 20, where n / (n + 2) already rounds to 1 in float.
+static __device__ __forceinline__ float ActMish(float v) {
+  const float e = __expf(__builtin_fminf(v, 20.0f));
+  const float n = e * (e + 2.0f);
+  return v * n * __builtin_amdgcn_rcpf(n + 2.0f);
+}
+static __device__ __forceinline__ float ActSigmoid(float v) { return __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
+static __device__ __forceinline__ float Activate(float v, int act) {
+  switch (act) {
+    case 1: return ActMish(v);
+    case 2: return v > 0.0f ? v : 0.0f;
+    case 4: return tanhf(v);
+    case 5: return ActSigmoid(v);
+    case 6: return v > 0.0f ? 1.05070098f * v : 1.05070098f * 1.67326324f * (__expf(v) - 1.0f);
+    case 7: return v * ActSigmoid(v);
+    case 8: return v > 0.0f ? v * v : 0.0f;
+    default: return v;
+  }
+}
+
+
+}  // namespace lc0mi

@@ -36,6 +36,10 @@ struct GemmArgs {
   bool latency_first = false;
 };
 void LaunchGemm(const GemmArgs& args, hipStream_t stream);
+// The persistent 256x256 kernel (gemm_persistent.hip) behind LaunchGemm: whether it takes these arguments, and
+// its launch (stream_stores: write the output with streaming stores).
+bool GemmPersistentSupports(const GemmArgs& args);
+void LaunchGemmPersistent(const GemmArgs& args, bool stream_stores, hipStream_t stream);
 // Name of the kernel variant LaunchGemm picks for these arguments (tile shape).
 const char* GemmVariantName(const GemmArgs& args);
 

@@ -11,6 +11,8 @@
 //   attn_policy_gather    promotion offsets + kAttnPolicyMap gather  blas/network_blas.cc:873-914
 #include "kernels.h"
 
+#include "device_math.h"
+
 #include <algorithm>
 #include <type_traits>
 #include <utility>
@@ -25,30 +27,6 @@ typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx8 __attribute__((ext_vector_type(8)));
 
 namespace {
-
-// Activation functions (values as shared/activation.cc:51-100). The GEMM epilogues are bound by
-// vector-ALU issue, so mish and swish use one hardware exponential and one hardware reciprocal
-// (1 ulp each) instead of a correctly rounded division:
-//   mish(v) = v * tanh(log(1 + e^v)) = v * n / (n + 2),  n = e^v * (e^v + 2).
-// The exponent is clamped at 20, where n / (n + 2) already rounds to 1 in float.
-__device__ __forceinline__ float ActMish(float v) {
-  const float e = __expf(__builtin_fminf(v, 20.0f));
-  const float n = e * (e + 2.0f);
-  return v * n * __builtin_amdgcn_rcpf(n + 2.0f);
-}
-__device__ __forceinline__ float ActSigmoid(float v) { return __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
-__device__ __forceinline__ float Activate(float v, int act) {
-  switch (act) {
-    case 1: return ActMish(v);
-    case 2: return v > 0.0f ? v : 0.0f;
-    case 4: return tanhf(v);
-    case 5: return ActSigmoid(v);
-    case 6: return v > 0.0f ? 1.05070098f * v : 1.05070098f * 1.67326324f * (__expf(v) - 1.0f);
-    case 7: return v * ActSigmoid(v);
-    case 8: return v > 0.0f ? v * v : 0.0f;
-    default: return v;
-  }
-}
 
 // Calls f with a branch-free functor for the activation, so that unrolled
 // epilogue loops do not carry a per-element switch.
@@ -627,7 +605,7 @@ void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
 }  // namespace
 
 namespace {
-enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128, kRowPanel, kDma128x64 };
+enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128, kRowPanel, kDma128x64, kPersist256 };
 
 int g_variant_override = -1;
 
@@ -636,7 +614,8 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
     const bool dma_ok = !a.out_f32 && a.split_k == 1 && a.K % 64 == 0;
     const bool is_dma = g_variant_override <= kDma256x128 || g_variant_override == kDma128x128 ||
                         g_variant_override == kDma128x64;
-    const bool ok = is_dma ? dma_ok : (g_variant_override != kRowPanel || a.split_k == 1);
+    bool ok = is_dma ? dma_ok : (g_variant_override != kRowPanel || a.split_k == 1);
+    if (g_variant_override == kPersist256) ok = GemmPersistentSupports(a);
     if (ok) return static_cast<GemmVariant>(g_variant_override);
   }
   const long long tiles128 = (long long)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
@@ -657,6 +636,11 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
     const double cs = rs * 128 * 128 * (rs > 1 ? 0.75 : 0.95) * (a.K <= 256 ? 1.12 : 1.0);
     GemmVariant best = kDma256x256;
     double cost = c256;
+    // (The persistent kernel of gemm_persistent.hip is not part of this choice: alone it is level with the 256x256
+    // kernel on these shapes (16384x3072x1024: 107 against 112 us, single-round shapes equal), but its one
+    // workgroup per CU holds every CU for the whole launch, so the smolgen chain on the second stream no longer
+    // slips in between rounds of tiles: a 15x1024 pass at batch 256 takes 6.66 ms with it against 5.91 ms.
+    // It is reachable through SetGemmVariantOverride(kPersist256).)
     if (c192 < cost) { best = kDma256x192; cost = c192; }
     if (c128 < cost) { best = kDma256x128; cost = c128; }
     if (cs < cost) { best = kDma128x128; cost = cs; }
@@ -688,6 +672,7 @@ void SetGemmVariantOverride(int variant) { g_variant_override = variant; }
 
 const char* GemmVariantName(const GemmArgs& a) {
   switch (PickGemmVariant(a)) {
+    case kPersist256: return "gemm_persistent_256x256x64";
     case kDma256x256: return "gemm_dma_256x256x64";
     case kDma256x192: return "gemm_dma_256x192x64";
     case kDma256x128: return "gemm_dma_256x128x32";
@@ -702,6 +687,7 @@ const char* GemmVariantName(const GemmArgs& a) {
 void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
   switch (PickGemmVariant(a)) {
+    case kPersist256: LaunchGemmPersistent(a, StreamOutput(a.M, a.N, a.batch, 2), stream); break;
     case kDma256x256: LaunchGemmDma<256, 256, 64, 2, 4>(a, stream); break;
     case kDma256x192: LaunchGemmDma<256, 192, 64, 4, 2>(a, stream); break;
     case kDma256x128: LaunchGemmDma<256, 128, 32, 4, 2>(a, stream); break;
