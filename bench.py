@@ -21,6 +21,7 @@ if ROOT not in sys.path:
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA peak
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA peak
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA peak
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 
 # HBM bytes per launch of a kernel cannot be read from inside the process: they come from two rocprofv3 --pmc
@@ -241,7 +242,8 @@ def main():
     dom = max(groups.values(), key=lambda g: g.ms)
     if dom.flops > 0:
         achieved = dom.flops / dom.launches / (dom.ms / dom.launches * 1e-3) / 1e12
-        peak = PEAK_FP8_TFLOPS if dom.name.startswith("gemm_f8") else PEAK_FP16_TFLOPS
+        peak = (PEAK_FP8_TFLOPS if dom.name.startswith("gemm_f8") else
+                PEAK_FP32_TFLOPS if dom.name.startswith("gemm_f32") else PEAK_FP16_TFLOPS)
         roofline = {"bound": "mfma", "kernel": dom.name, "achieved": achieved, "peak": peak,
                     "unit": "TFLOP/s", "frac": achieved / peak, "traffic": None,
                     "avg_launch_ms": dom.ms / dom.launches, "launches_per_step": dom.launches // prof_iters}

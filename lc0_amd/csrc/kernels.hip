@@ -758,52 +758,66 @@ void LaunchGemmF8(const GemmF8Args& a, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------------------
-// float GEMM (fp32 configuration): same contract, LDS-tiled, 64x64 block tile,
-// each thread a 4x4 register tile, plain fp32 FMAs with fp32 accumulation.
+// float GEMM (fp32 configuration): same contract on fp32 operands with the fp32 matrix instruction
+// v_mfma_f32_32x32x2_f32 (fp32 products, fp32 accumulation).
+//
+// Eight waves per workgroup, laid out TILES_M x TILES_N x KSPLIT: every wave owns one 32x32 accumulator tile over
+// its share of the reduction and reads its 32 + 32 operand rows straight from global memory, 16 bytes per lane
+// and k-step (lane half g takes k = 8s + 4g .. 8s + 4g + 3; the four MFMAs of a step pair equal offsets of both
+// operands, so every k is used exactly once). Sixteen such loads are kept in flight per wave. The KSPLIT partial
+// tiles are added through LDS in wave order, then scale, bias and activation are applied.
+//   <1,1,8>: 32x32 tile, the reduction split eight ways -- few output tiles, long K (the heads' dense layers at
+//            small batch: 32x128x2048 used to run on two workgroups);
+//   <2,2,2>: 64x64 tile for launches with many tiles.
 // ---------------------------------------------------------------------------
 namespace {
-__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgsF32 p) {
-  constexpr int BM = 64, BN = 64, BK = 16;
-  __shared__ float As[BK][BM + 4];
-  __shared__ float Ws[BK][BN + 4];
-  const int tid = threadIdx.x;
-  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
-  const float* A = p.A + (long long)blockIdx.z * p.strideA;
-  const float* W = p.W + (long long)blockIdx.z * p.strideW;
+template <int TILES_M, int TILES_N, int KSPLIT>
+__global__ __launch_bounds__(512) void gemm_f32_mfma_kernel(GemmArgsF32 p) {
+  static_assert(TILES_M * TILES_N * KSPLIT == 8, "eight waves");
+  constexpr int UNROLL = 8;   // k-steps (of 8) whose loads are issued together
+  __shared__ float red[8][32][33];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ks = wave % KSPLIT, tile = wave / KSPLIT;
+  const int tm = tile / TILES_N, tn = tile % TILES_N;
+  const int r = lane & 31, g = lane >> 5;
+  const int m0 = (blockIdx.x * TILES_M + tm) * 32, n0 = (blockIdx.y * TILES_N + tn) * 32;
+  const float* A = p.A + (long long)blockIdx.z * p.strideA + (long long)min(m0 + r, p.M - 1) * p.lda + g * 4;
+  const float* W = p.W + (long long)blockIdx.z * p.strideW + (long long)min(n0 + r, p.N - 1) * p.ldw + g * 4;
   float* C = p.C + (long long)blockIdx.z * p.strideC;
-  const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
-  float acc[4][4] = {};
-  const int lrow = tid / 4, lk = (tid % 4) * 4;  // 64 rows x 4 float4 per tile
-  for (int k0 = 0; k0 < p.K; k0 += BK) {
-    floatx4 va = {0, 0, 0, 0}, vw = {0, 0, 0, 0};
-    if (k0 + lk < p.K) {
-      va = *reinterpret_cast<const floatx4*>(A + (long long)min(m0 + lrow, p.M - 1) * p.lda + k0 + lk);
-      vw = *reinterpret_cast<const floatx4*>(W + (long long)min(n0 + lrow, p.N - 1) * p.ldw + k0 + lk);
+  const int K = p.K;
+  floatx16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+  const int steps = (K + 7) / 8;
+  // this wave's k-steps: ks, ks + KSPLIT, ...
+  for (int s0 = ks; s0 < steps; s0 += KSPLIT * UNROLL) {
+    floatx4 va[UNROLL], vw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      const int k = (s0 + u * KSPLIT) * 8;
+      const bool ok = k + g * 4 < K;   // K % 4 == 0: a 16-byte piece is inside or outside as a whole
+      va[u] = ok ? *reinterpret_cast<const floatx4*>(A + k) : floatx4{0, 0, 0, 0};
+      vw[u] = ok ? *reinterpret_cast<const floatx4*>(W + k) : floatx4{0, 0, 0, 0};
     }
 #pragma unroll
-    for (int e = 0; e < 4; e++) { As[lk + e][lrow] = va[e]; Ws[lk + e][lrow] = vw[e]; }
-    __syncthreads();
+    for (int u = 0; u < UNROLL; u++)
 #pragma unroll
-    for (int k = 0; k < BK; k++) {
-      float a[4], w[4];
-#pragma unroll
-      for (int e = 0; e < 4; e++) { a[e] = As[k][tm + e]; w[e] = Ws[k][tn + e]; }
-#pragma unroll
-      for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
-    }
-    __syncthreads();
+      for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(vw[u][e], va[u][e], acc, 0, 0, 0);
   }
+  // accumulator element e: n = 8*(e/4) + 4*g + e%4, m = r
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    int m = m0 + tm + i;
-    if (m >= p.M) continue;
+  for (int e = 0; e < 16; e++) red[wave][r][8 * (e / 4) + 4 * g + (e & 3)] = acc[e];
+  __syncthreads();
+  constexpr int OUT = TILES_M * TILES_N * 1024;
+  for (int idx = tid; idx < OUT; idx += 512) {
+    const int t = idx >> 10, mm = (idx >> 5) & 31, nn = idx & 31;
+    float x = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      int n = n0 + tn + j;
-      if (n >= p.N) continue;
-      float x = acc[i][j] * p.scale;
+    for (int z = 0; z < KSPLIT; z++) x += red[t * KSPLIT + z][mm][nn];
+    const int m = (blockIdx.x * TILES_M + t / TILES_N) * 32 + mm, n = (blockIdx.y * TILES_N + t % TILES_N) * 32 + nn;
+    if (m < p.M && n < p.N) {
+      x *= p.scale;
       if (p.bias != nullptr) x += p.bias[n];
       C[(long long)m * p.ldc + n] = Activate(x, p.act);
     }
@@ -813,8 +827,14 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgsF32 p) {
 
 void LaunchGemmF32(const GemmArgsF32& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
-  dim3 grid((a.M + 63) / 64, (a.N + 63) / 64, a.batch);
-  hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, a);
+  const long long tiles64 = (long long)((a.M + 63) / 64) * ((a.N + 63) / 64) * a.batch;
+  if (tiles64 >= 256) {
+    dim3 grid((a.M + 63) / 64, (a.N + 63) / 64, a.batch);
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<2, 2, 2>), grid, dim3(512), 0, stream, a);
+  } else {
+    dim3 grid((a.M + 31) / 32, (a.N + 31) / 32, a.batch);
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<1, 1, 8>), grid, dim3(512), 0, stream, a);
+  }
 }
 
 // ---------------------------------------------------------------------------

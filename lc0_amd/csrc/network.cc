@@ -1203,7 +1203,7 @@ void Mi355xNetwork::GemmT(const char* name, const void* A, int lda, long long st
     g.W = static_cast<const float*>(W); g.ldw = ldw; g.strideW = strideW;
     g.C = static_cast<float*>(C); g.ldc = ldc; g.strideC = strideC;
     g.bias = bias; g.M = M; g.N = N; g.K = K; g.batch = batch; g.act = act;
-    const std::string label = std::string(name) + "|gemm_f32_64x64x16";
+    const std::string label = std::string(name) + "|gemm_f32_mfma_32x32x2";
     Timed(label.c_str(), flops, bytes, [&] { LaunchGemmF32(g, stream_); });
   }
 }
