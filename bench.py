@@ -134,6 +134,7 @@ def main():
                                                               "three passes fit in about 27 s)")
     ap.add_argument("--traffic-json", default="", help="HBM bytes per launch from a rocprofv3 --pmc run of this command "
                                                        "(default: profiles/hbm_traffic_<config>_batch<B>.txt if present)")
+    ap.add_argument("--options", default="", help="backend options appended to the workload's own (name=value,...)")
     ap.add_argument("--sweep", default="", help="comma-separated batch sizes: adds their resident-batch evals/s "
                                                 "as \"batch_sweep\" to the JSON line")
     args = ap.parse_args()
@@ -156,7 +157,8 @@ def main():
     if max([batch] + sweep) > masks.shape[0]:
         reps = -(-max([batch] + sweep) // masks.shape[0])
         masks, values = np.tile(masks, (reps, 1)), np.tile(values, (reps, 1))
-    net = Network(path, "gpu=0,max_batch=%d" % max([batch, 16] + sweep) + ("," + wl["options"] if wl.get("options") else ""))
+    net = Network(path, "gpu=0,max_batch=%d" % max([batch, 16] + sweep) + ("," + wl["options"] if wl.get("options") else "") +
+                  ("," + args.options if args.options else ""))
     comp = net.NewComputation()
     comp.AddInputs(masks[:batch], values[:batch])
     comp.ComputeBlocking()          # stages the batch into HBM and warms everything up
@@ -264,7 +266,8 @@ def main():
         "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": wl.get("dtype", "fp16"), "data": "synthetic",
         "config": {"workload": args.config, "description": wl["desc"], "batch": batch,
-                   "inputs": "seeded random-playout positions, classical 112 planes"},
+                   "inputs": "seeded random-playout positions, classical 112 planes",
+                   **({"extra_options": args.options} if args.options else {})},
         "roofline": roofline,
         "event_ms_per_step": ev_ms,
         "with_host_io_evals_per_s": batch / (io_ms * 1e-3),

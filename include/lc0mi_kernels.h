@@ -25,6 +25,23 @@ int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* 
  * slice order (bias added once, no activation). C is float [M][N]. */
 int lc0mi_k_gemm_splitk(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,
                         int K, int split_k, float scale, float* C, int ldc);
+/* The two GEMMs around a layer norm with the norm folded into them, so that neither the normalised rows nor the
+ * sum they are computed from travel through memory on their own (LayerNorm2DWithSkipConnection between the dense
+ * layers of an encoder block, src/neural/backends/blas/network_blas.cc:441-470 with encoder.h:29-66).
+ * Producer: U[m][n] = scale * A[m][:] . W[n][:] + bias[n] + s[m][n] as halves, where s = skip, or, when skip_stats
+ * is given, the layer norm of skip's rows with skip_gamma / skip_beta and the statistics in skip_stats
+ * ([M][skip_parts][2] partial (sum, sum of squares) per row). skip is [M][N]. stats_out receives [M][*parts_out][2]
+ * partial sums of the stored U per column tile (at most stats_cap floats). */
+int lc0mi_k_gemm_norm_producer(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,
+                               int K, float scale, const uint16_t* skip, const float* skip_stats, int skip_parts,
+                               const float* skip_gamma, const float* skip_beta, float eps, uint16_t* U,
+                               float* stats_out, int stats_cap, int* parts_out, int time_iters, double* ms);
+/* Consumer: C[m][n] = act(rstd[m] * (U[m][:] . W[n][:] - mean[m] * col_c[n]) + bias[n]), mean and rstd of row m of
+ * U (K columns) from stats [M][parts][2]. With W = w * gamma, col_c[n] = sum_k W[n][k] and bias[n] = b[n] +
+ * sum_k beta[k] w[n][k] this equals act(LN(U) . w^T + b). */
+int lc0mi_k_gemm_norm_consumer(const uint16_t* U, int ldu, const uint16_t* W, int ldw, const float* col_c,
+                               const float* bias, int M, int N, int K, const float* stats, int parts, float eps,
+                               int act, int latency_first, uint16_t* C, int ldc, int time_iters, double* ms);
 /* Forces the GEMM tile variant of subsequent calls (-1 automatic; 0 256x256x64,
  * 1 256x192x64, 2 256x128x32 direct-to-LDS kernels, 3 128x128x64, 4 64x64x64, 5 direct-to-LDS 128x128x64,
  * 6 row-panel 64x32, 7 direct-to-LDS 128x64x64, 8 persistent 256x256x64). */

@@ -109,6 +109,76 @@ int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* 
   });
 }
 
+int lc0mi_k_gemm_norm_producer(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,
+                               int K, float scale, const uint16_t* skip, const float* skip_stats, int skip_parts,
+                               const float* skip_gamma, const float* skip_beta, float eps, uint16_t* U,
+                               float* stats_out, int stats_cap, int* parts_out, int time_iters, double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (K % 8 || lda % 8 || ldw % 8 || N % 8) throw Error("K, lda, ldw and N must be multiples of 8");
+    if (M < 1 || N < 1 || lda < K || ldw < K) throw Error("bad gemm shape");
+    Dev dev;
+    lc0mi::GemmArgs g;
+    g.A = reinterpret_cast<const half_t*>(dev.Put(A, (size_t)(M - 1) * lda + K)); g.lda = lda;
+    g.W = reinterpret_cast<const half_t*>(dev.Put(W, (size_t)(N - 1) * ldw + K)); g.ldw = ldw;
+    // the residual is added in place, as the network does it
+    half_t* u = reinterpret_cast<half_t*>(const_cast<uint16_t*>(dev.Put(skip, (size_t)M * N)));
+    g.C = u; g.ldc = N;
+    g.skip = u; g.ldskip = N;
+    g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
+    g.M = M; g.N = N; g.K = K; g.scale = scale; g.act = 3;
+    if (skip_stats != nullptr) {
+      g.skip_stats = dev.Put(skip_stats, (size_t)M * skip_parts * 2);
+      g.skip_parts = skip_parts;
+      g.skip_gamma = dev.Put(skip_gamma, (size_t)N);
+      g.skip_beta = dev.Put(skip_beta, (size_t)N);
+    }
+    g.norm_n = N; g.norm_eps = eps;
+    if (!lc0mi::GemmSupportsNormFolding(g)) throw Error("no kernel variant with the producer epilogue for this shape");
+    const int parts = lc0mi::GemmStatsParts(g);
+    if (parts < 1 || (size_t)M * parts * 2 > (size_t)stats_cap) throw Error("stats_out is too small");
+    float* d_stats = static_cast<float*>(dev.Alloc((size_t)M * parts * 2 * sizeof(float)));
+    g.stats_out = d_stats;
+    *parts_out = parts;
+    lc0mi::LaunchGemm(g, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(U, u, (size_t)M * N * 2, hipMemcpyDeviceToHost));
+    K_CHECK(hipMemcpy(stats_out, d_stats, (size_t)M * parts * 2 * sizeof(float), hipMemcpyDeviceToHost));
+    if (time_iters > 0 && ms) *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchGemm(g, nullptr); });
+  });
+}
+
+int lc0mi_k_gemm_norm_consumer(const uint16_t* U, int ldu, const uint16_t* W, int ldw, const float* col_c,
+                               const float* bias, int M, int N, int K, const float* stats, int parts, float eps,
+                               int act, int latency_first, uint16_t* C, int ldc, int time_iters, double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (K % 8 || ldu % 8 || ldw % 8) throw Error("K, ldu and ldw must be multiples of 8");
+    if (M < 1 || N < 1 || ldu < K || ldw < K || ldc < N || parts < 1 || col_c == nullptr) throw Error("bad gemm shape");
+    Dev dev;
+    lc0mi::GemmArgs g;
+    g.A = reinterpret_cast<const half_t*>(dev.Put(U, (size_t)(M - 1) * ldu + K)); g.lda = ldu;
+    g.W = reinterpret_cast<const half_t*>(dev.Put(W, (size_t)(N - 1) * ldw + K)); g.ldw = ldw;
+    const size_t c_elems = (size_t)(M - 1) * ldc + N;
+    g.C = dev.Alloc(c_elems * 2); g.ldc = ldc;
+    K_CHECK(hipMemcpy(g.C, C, c_elems * 2, hipMemcpyHostToDevice));
+    g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
+    g.col_c = dev.Put(col_c, (size_t)N);
+    g.row_stats = dev.Put(stats, (size_t)M * parts * 2);
+    g.row_parts = parts;
+    g.norm_n = K; g.norm_eps = eps;
+    g.M = M; g.N = N; g.K = K; g.act = act;
+    g.latency_first = latency_first != 0;
+    if (!lc0mi::GemmSupportsNormFolding(g)) throw Error("no kernel variant with the consumer epilogue for this shape");
+    lc0mi::LaunchGemm(g, nullptr);
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(C, g.C, c_elems * 2, hipMemcpyDeviceToHost));
+    if (time_iters > 0 && ms) *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchGemm(g, nullptr); });
+  });
+}
+
 int lc0mi_k_gemm_splitk(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,
                         int K, int split_k, float scale, float* C, int ldc) {
   return Guard([&] {

@@ -34,8 +34,40 @@ struct GemmArgs {
   // Choose the variant with the shortest latency even if it occupies more of the GPU (for a kernel on the
   // critical path; the default favours the variant that leaves room for a concurrent stream).
   bool latency_first = false;
+
+  // Layer norm folded into the GEMMs on either side of it, so that neither the normalised rows nor the sum they
+  // are computed from make a round trip of their own through memory. A "producer" GEMM adds the residual and
+  // leaves the un-normalised sum u plus per-row partial sums; a "consumer" GEMM multiplies u by weights that
+  // already carry gamma and corrects for mean and deviation per output row:
+  //   LN(u)[m] . w[n] = rstd[m] * (sum_k u[m][k] gamma[k] w[n][k] - mean[m] * c[n]) + sum_k beta[k] w[n][k]
+  // with c[n] = sum_k gamma[k] w[n][k]; the caller passes W = w * gamma, col_c = c and the beta term in bias.
+  // Row statistics travel as partial sums: stats[m][part][2] = (sum, sum of squares) over one column tile of u.
+  //
+  // Consumer (row_stats != nullptr):  C[m][n] = act(rstd[m] * (scale * acc - mean[m] * col_c[n]) + bias[n]),
+  //   mean and rstd of row m from the row_parts partial sums over norm_n columns.
+  const float* row_stats = nullptr;
+  int row_parts = 0;
+  const float* col_c = nullptr;
+  // Producer (skip != nullptr, no activation, half output):  C[m][n] = scale * acc + bias[n] + s[m][n], where
+  //   s = skip (skip_stats == nullptr) or the layer norm of skip's row with skip_gamma / skip_beta and statistics
+  //   from skip_stats (skip_parts partial sums per row over norm_n columns). skip may alias C.
+  //   stats_out (optional) receives the partial sums of the rows of C as stored (rounded to half):
+  //   stats_out[m][tile][2], one part per column tile of the kernel variant (GemmStatsParts()).
+  const half_t* skip = nullptr;
+  int ldskip = 0;
+  const float* skip_stats = nullptr;
+  int skip_parts = 0;
+  const float* skip_gamma = nullptr;
+  const float* skip_beta = nullptr;
+  float* stats_out = nullptr;
+  int norm_n = 0;        // length of the normalised rows (consumer: K of the real problem; producer: N)
+  float norm_eps = 0.0f;
 };
 void LaunchGemm(const GemmArgs& args, hipStream_t stream);
+// Whether LaunchGemm serves the folded layer-norm fields of these arguments (the kernel variant it picks has the
+// epilogue), and the number of partial sums per row a producer launch writes to stats_out.
+bool GemmSupportsNormFolding(const GemmArgs& args);
+int GemmStatsParts(const GemmArgs& args);
 // The persistent 256x256 kernel (gemm_persistent.hip) behind LaunchGemm: whether it takes these arguments, and
 // its launch (stream_stores: write the output with streaming stores).
 bool GemmPersistentSupports(const GemmArgs& args);

@@ -14,6 +14,7 @@
 #include "device_math.h"
 
 #include <algorithm>
+#include <stdexcept>
 #include <type_traits>
 #include <utility>
 
@@ -57,6 +58,28 @@ __device__ __forceinline__ float WaveSum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
+}
+
+// The value of v in the lane that the data-parallel-primitive control CTRL selects (0xB1: lane ^ 1, 0x4E: lane ^ 2
+// within a group of four, 0x141: mirrored within a group of eight).
+template <int CTRL>
+__device__ __forceinline__ float DppMove(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+
+// Mean and 1 / sqrt(variance + eps) of row m from its partial (sum, sum of squares) pairs over n values.
+__device__ __forceinline__ void RowMeanRstd(const float* stats, int parts, long long m, int n, float eps, float& mean,
+                                            float& rstd) {
+  const float2* s = reinterpret_cast<const float2*>(stats) + m * parts;
+  float s1 = 0.0f, s2 = 0.0f;
+  for (int i = 0; i < parts; i++) {
+    const float2 v = s[i];
+    s1 += v.x;
+    s2 += v.y;
+  }
+  const float inv_n = 1.0f / (float)n;
+  mean = s1 * inv_n;
+  rstd = 1.0f / sqrtf(fmaxf(s2 * inv_n - mean * mean, 0.0f) + eps);
 }
 
 // ---------------------------------------------------------------------------
@@ -186,6 +209,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     }
   }
   const bool vec_ok = (p.ldc % 4 == 0);
+  // Consumer side of a folded layer norm (GemmArgs::row_stats): mean and rstd of this lane's rows.
+  float row_mean[TM], row_rstd[TM];
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    row_mean[i] = 0.0f;
+    row_rstd[i] = 1.0f;
+    if (p.row_stats != nullptr) {
+      RowMeanRstd(p.row_stats, p.row_parts, min(m0 + wm * WM + i * 32 + frag_row, M - 1), p.norm_n, p.norm_eps,
+                  row_mean[i], row_rstd[i]);
+    }
+  }
   DispatchAct(p.act, [&](auto act_fn) {
 #pragma unroll
     for (int j = 0; j < TN; j++) {
@@ -193,15 +227,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
       for (int blk = 0; blk < 4; blk++) {
         const int n = n0 + wn * WN + j * 32 + blk * 8 + (lane >> 5) * 4;
         if (n >= N) continue;
-        float b4[4];
+        float b4[4], c4[4];
         LoadBias4(p.bias, n, N, b4);
+        LoadBias4(p.row_stats != nullptr ? p.col_c : nullptr, n, N, c4);
 #pragma unroll
         for (int i = 0; i < TM; i++) {
           const int m = m0 + wm * WM + i * 32 + frag_row;
           if (m >= M) continue;
           float v[4];
 #pragma unroll
-          for (int r = 0; r < 4; r++) v[r] = act_fn(acc[i][j][blk * 4 + r] * p.scale + b4[r]);
+          for (int r = 0; r < 4; r++)
+            v[r] = act_fn(row_rstd[i] * (acc[i][j][blk * 4 + r] * p.scale - row_mean[i] * c4[r]) + b4[r]);
           OutT* dst = C + (long long)m * p.ldc + n;
           if (vec_ok && n + 3 < N) {
             if constexpr (sizeof(OutT) == 2) {
@@ -303,7 +339,13 @@ __global__ __launch_bounds__(512) void gemm_rowpanel_kernel(GemmArgs p) {
         float sum = part[0][row * 33 + col];
 #pragma unroll
         for (int w = 1; w < NW; w++) sum += part[w][row * 33 + col];
-        const float v = act_fn(sum * p.scale + (p.bias ? p.bias[n] : 0.0f));
+        sum *= p.scale;
+        if (p.row_stats != nullptr) {   // consumer side of a folded layer norm
+          float mean, rstd;
+          RowMeanRstd(p.row_stats, p.row_parts, m, p.norm_n, p.norm_eps, mean, rstd);
+          sum = rstd * (sum - mean * p.col_c[n]);
+        }
+        const float v = act_fn(sum + (p.bias ? p.bias[n] : 0.0f));
         C[(long long)m * p.ldc + n] = (OutT)v;
       }
     }
@@ -350,7 +392,10 @@ __device__ __forceinline__ unsigned PackFp8x4(float a, float b, float c, float d
 // GemmF8Args: 128 bytes = 128 values per row, v_mfma_f32_32x32x64_f8f6f4);
 // BKB is the k-tile in bytes. OutT is half_t or uint8_t (e4m3, fp8 operands only).
 // STREAM: the output is written with streaming (non-temporal) stores.
-template <int BM, int BN, int BKB, int WAVES_M, int WAVES_N, typename Args, typename OutT, bool STREAM = false>
+// EPI (fp16 operands only): 0 the plain epilogue, 1 the consumer and 2 the producer side of a folded layer norm
+// (GemmArgs::row_stats / GemmArgs::skip).
+template <int BM, int BN, int BKB, int WAVES_M, int WAVES_N, typename Args, typename OutT, bool STREAM = false,
+          int EPI = 0>
 // Second launch bound = waves per SIMD: with small wave tiles two workgroups share a CU
 // (4 waves per SIMD, at most 128 VGPRs) and overlap each other's prologue and epilogue.
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
@@ -374,7 +419,12 @@ void gemm_dma_kernel(Args p) {
   constexpr int OV = 16 / sizeof(OutT);           // output elements per 16-byte vector
   constexpr int EPI_STRIDE = WN + OV;             // elements
   constexpr int EPI_BYTES = NWAVES * 32 * EPI_STRIDE * (int)sizeof(OutT);
-  constexpr int SMEM = (2 * STAGE > EPI_BYTES) ? 2 * STAGE : EPI_BYTES;
+  // Folded layer norm: (mean, rstd) of the tile's rows, and the producer's per-wave-column partial sums.
+  constexpr int STAT_BYTES = (EPI != 0) ? BM * 8 : 0;
+  constexpr int PART_BYTES = (EPI == 2) ? WAVES_N * BM * 8 : 0;
+  constexpr int EPI_TOTAL = EPI_BYTES + STAT_BYTES + PART_BYTES;
+  constexpr int SMEM = (2 * STAGE > EPI_TOTAL) ? 2 * STAGE : EPI_TOTAL;
+  static_assert(EPI == 0 || (!F8 && sizeof(OutT) == 2), "folded layer norm: fp16 operands and output");
   __shared__ __attribute__((aligned(1024))) char smem[SMEM];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -424,6 +474,21 @@ void gemm_dma_kernel(Args p) {
 
   const int nk = K * ES / BKB;
   issue(smem, smem + BM * BKB, 0);
+  // Folded layer norm: (mean, rstd) of tile row `tid` (of the A operand for a consumer, of the residual for a
+  // producer), fetched while the first k-tile is on its way and kept in two registers until the epilogue.
+  [[maybe_unused]] float2 my_ms = make_float2(0.0f, 1.0f);
+  [[maybe_unused]] bool norm_skip = false;
+  if constexpr (EPI != 0) {
+    const float* st = (EPI == 1) ? p.row_stats : p.skip_stats;
+    norm_skip = st != nullptr;
+    if (st != nullptr && tid < BM) {
+      RowMeanRstd(st, (EPI == 1) ? p.row_parts : p.skip_parts, min(m0 + tid, M - 1), p.norm_n, p.norm_eps, my_ms.x,
+                  my_ms.y);
+    }
+  }
+  // Producer: the residual tile is touched early (one dword per 128-byte line, values unused), so that the
+  // epilogue finds it in cache instead of reading memory in the same burst in which every workgroup writes.
+  [[maybe_unused]] int touch[(BM * BN * 2 / 128 + NWAVES * 64 - 1) / (NWAVES * 64)] = {};
   for (int kt = 0; kt < nk; kt++) {
     const char* As = smem + (kt & 1) * STAGE;
     const char* Ws = As + BM * BKB;
@@ -431,6 +496,19 @@ void gemm_dma_kernel(Args p) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of k-tile kt have landed
     __syncthreads();                     // ... and everybody's; everybody is done reading the other stage
     if (kt + 1 < nk) issue(nxt, nxt + BM * BKB, (kt + 1) * BKB);
+    if constexpr (EPI == 2) {
+      if (kt == 1) {
+        constexpr int LINES_PER_ROW = BN * 2 / 128;
+        constexpr int LINES = BM * LINES_PER_ROW;
+#pragma unroll
+        for (int q = 0; q < (LINES + NWAVES * 64 - 1) / (NWAVES * 64); q++) {
+          const int line = q * NWAVES * 64 + tid;
+          const int row = line / LINES_PER_ROW, seg = line % LINES_PER_ROW;
+          const half_t* src = p.skip + (long long)min(m0 + row, M - 1) * p.ldskip + min(n0 + seg * 64, N - 2);
+          if (line < LINES) asm volatile("global_load_dword %0, %1, off" : "=v"(touch[q]) : "v"(src) : "memory");
+        }
+      }
+    }
     if constexpr (F8) {
       // One MFMA consumes 64 k-values: lane half g holds 32 consecutive bytes = 2 chunks.
 #pragma unroll
@@ -475,20 +553,79 @@ void gemm_dma_kernel(Args p) {
 
   // Epilogue through LDS (the stage buffers are free after the barrier).
   __syncthreads();
+  if constexpr (EPI == 2) {
+    // (the registers of the early touches stay reserved up to here: every wait of the loop has covered them)
+#pragma unroll
+    for (int q = 0; q < (int)(sizeof(touch) / sizeof(touch[0])); q++) asm volatile("" ::"v"(touch[q]));
+  }
   OutT* C = reinterpret_cast<OutT*>(p.C);
   if constexpr (!F8) C += (long long)blockIdx.z * p.strideC;
   OutT* strip = reinterpret_cast<OutT*>(smem) + wave * 32 * EPI_STRIDE;
   constexpr int CHUNKS_PER_ROW = WN / OV;
   constexpr int STRIP_CHUNKS = 32 * CHUNKS_PER_ROW;
+  constexpr int NPASS = (STRIP_CHUNKS + 63) / 64;
   const bool vec_ok = (p.ldc % OV == 0);
   float bias_v[TN][4][4];
 #pragma unroll
   for (int j = 0; j < TN; j++)
 #pragma unroll
     for (int blk = 0; blk < 4; blk++) LoadBias4(p.bias, n0 + wn * WN + j * 32 + blk * 8 + g * 4, N, bias_v[j][blk]);
+  // Folded layer norm: statistics of this tile's rows (of the A operand for a consumer, of the residual for a
+  // producer), one row per thread, shared through LDS.
+  [[maybe_unused]] float2* row_ms = reinterpret_cast<float2*>(smem + EPI_BYTES);                 // [BM] (mean, rstd)
+  [[maybe_unused]] float2* part_lds = reinterpret_cast<float2*>(smem + EPI_BYTES + STAT_BYTES);  // [WAVES_N][BM]
+  [[maybe_unused]] float col_c[TN][4][4];
+  auto load_skip = [&](int i, intx4 (&sk)[NPASS]) {
+#pragma unroll
+    for (int pass = 0; pass < NPASS; pass++) {
+      const int idx = pass * 64 + lane;
+      const int row = idx / CHUNKS_PER_ROW;
+      const int ch = idx - row * CHUNKS_PER_ROW;
+      const int m = m0 + wm * WM + i * 32 + row;
+      const int n = n0 + wn * WN + ch * OV;
+      if constexpr (EPI == 2) {
+        sk[pass] = (idx < STRIP_CHUNKS && m < M && n + OV - 1 < N)
+                       ? *reinterpret_cast<const intx4*>(p.skip + (long long)m * p.ldskip + n)
+                       : intx4{0, 0, 0, 0};
+      }
+    }
+  };
+  // Producer: the residual chunks of a strip are fetched one strip ahead.
+  [[maybe_unused]] intx4 sk_cur[NPASS], sk_nxt[NPASS];
+  if constexpr (EPI == 2) load_skip(0, sk_cur);
+  if constexpr (EPI != 0) {
+    if (norm_skip) {
+      if (tid < BM) row_ms[tid] = my_ms;
+      __syncthreads();
+    }
+    if constexpr (EPI == 1) {
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int blk = 0; blk < 4; blk++) LoadBias4(p.col_c, n0 + wn * WN + j * 32 + blk * 8 + g * 4, N, col_c[j][blk]);
+    }
+  }
+  // Producer: gamma and beta of the residual's layer norm for this lane's eight columns (the same in every pass).
+  [[maybe_unused]] float sk_gamma[8], sk_beta[8];
+  if constexpr (EPI == 2) {
+    static_assert(64 % CHUNKS_PER_ROW == 0, "a lane must keep its columns over the passes of a strip");
+    const int n = n0 + wn * WN + (lane % CHUNKS_PER_ROW) * OV;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      sk_gamma[e] = (norm_skip && n + e < N) ? p.skip_gamma[n + e] : 1.0f;
+      sk_beta[e] = (norm_skip && n + e < N) ? p.skip_beta[n + e] : 0.0f;
+    }
+  }
   DispatchAct(p.act, [&](auto act_fn) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
+      // Consumer: v = rstd * (scale * acc - mean * c) + bias = acc * (rstd * scale) + (bias - (rstd * mean) * c)
+      [[maybe_unused]] float rs_scale = 1.0f, rs_mean = 0.0f;
+      if constexpr (EPI == 1) {
+        const float2 ms = row_ms[wm * WM + i * 32 + r];
+        rs_scale = ms.y * p.scale;
+        rs_mean = -ms.y * ms.x;
+      }
 #pragma unroll
       for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -500,6 +637,10 @@ void gemm_dma_kernel(Args p) {
             LoadBias4(p.col_scale, n0 + wn * WN + j * 32 + blk * 8 + g * 4, N, cs);
 #pragma unroll
             for (int rr = 0; rr < 4; rr++) v[rr] = act_fn(acc[i][j][blk * 4 + rr] * cs[rr] + bias_v[j][blk][rr]);
+          } else if constexpr (EPI == 1) {
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++)
+              v[rr] = act_fn(fmaf(acc[i][j][blk * 4 + rr], rs_scale, fmaf(rs_mean, col_c[j][blk][rr], bias_v[j][blk][rr])));
           } else {
 #pragma unroll
             for (int rr = 0; rr < 4; rr++) v[rr] = act_fn(acc[i][j][blk * 4 + rr] * p.scale + bias_v[j][blk][rr]);
@@ -518,13 +659,60 @@ void gemm_dma_kernel(Args p) {
       }
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0); the strip is private to this wave
       __builtin_amdgcn_wave_barrier();
+      if constexpr (EPI == 2) {
+        if (i + 1 < TM) load_skip(i + 1, sk_nxt);
+      }
 #pragma unroll
-      for (int pass = 0; pass < (STRIP_CHUNKS + 63) / 64; pass++) {
+      for (int pass = 0; pass < NPASS; pass++) {
         const int idx = pass * 64 + lane;
         const int row = idx / CHUNKS_PER_ROW;
         const int ch = idx - row * CHUNKS_PER_ROW;
         const int m = m0 + wm * WM + i * 32 + row;
         const int n = n0 + wn * WN + ch * OV;
+        if constexpr (EPI == 2) {
+          // C = (scale * acc + bias, already rounded to half) + residual, the residual normalised on the way when
+          // it is itself an un-normalised sum; then the partial sums of the stored values over this wave's columns.
+          const bool ok = idx < STRIP_CHUNKS && m < M && n + OV - 1 < N;
+          const half8 hv = *reinterpret_cast<const half8*>(&strip[row * EPI_STRIDE + ch * OV]);
+          const half8 hs = __builtin_bit_cast(half8, sk_cur[pass]);
+          float2 rm = make_float2(0.0f, 1.0f);
+          if (norm_skip) rm = row_ms[wm * WM + i * 32 + min(row, 31)];
+          const float neg_mean_rstd = -rm.x * rm.y;
+          half8 o;
+          float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const float t = fmaf((float)hs[e], rm.y, neg_mean_rstd);
+            const float u = fmaf(t, sk_gamma[e], sk_beta[e]) + (float)hv[e];
+            o[e] = (half_t)u;
+            s1 += u;            // (of the sums before rounding to half: the difference is far below the rounding
+            s2 = fmaf(u, u, s2);   //  of the normalised values themselves)
+          }
+          if (ok) {
+            half_t* dst = reinterpret_cast<half_t*>(C) + (long long)m * p.ldc + n;
+            if constexpr (STREAM) {
+              __builtin_nontemporal_store(__builtin_bit_cast(intx4, o), reinterpret_cast<intx4*>(dst));
+            } else {
+              *reinterpret_cast<half8*>(dst) = o;
+            }
+          }
+          // Sum over the CHUNKS_PER_ROW (4 or 8) neighbouring lanes of a row, with data-parallel-primitive moves.
+          static_assert(CHUNKS_PER_ROW == 4 || CHUNKS_PER_ROW == 8, "row reduction written for 4 or 8 lanes per row");
+          s1 += DppMove<0xB1>(s1);   // lane ^ 1
+          s2 += DppMove<0xB1>(s2);
+          s1 += DppMove<0x4E>(s1);   // lane ^ 2
+          s2 += DppMove<0x4E>(s2);
+          if constexpr (CHUNKS_PER_ROW == 8) {
+            s1 += DppMove<0x141>(s1);   // mirror within 8 lanes: the other quad's sum
+            s2 += DppMove<0x141>(s2);
+          }
+          if (ch == 0 && idx < STRIP_CHUNKS) part_lds[wn * BM + wm * WM + i * 32 + row] = make_float2(s1, s2);
+          if (pass + 1 == NPASS && i + 1 < TM) {
+#pragma unroll
+            for (int q = 0; q < NPASS; q++) sk_cur[q] = sk_nxt[q];
+          }
+          continue;
+        }
         if (idx < STRIP_CHUNKS && m < M && n < N) {
           OutT* dst = C + (long long)m * p.ldc + n;
           if (vec_ok && n + OV - 1 < N) {
@@ -543,6 +731,21 @@ void gemm_dma_kernel(Args p) {
       __builtin_amdgcn_wave_barrier();
     }
   });
+  if constexpr (EPI == 2) {
+    // Partial sums of this column tile: the WAVES_N wave columns added in a fixed order.
+    if (p.stats_out != nullptr) {
+      __syncthreads();
+      if (tid < BM && m0 + tid < M) {
+        float2 t = part_lds[tid];
+#pragma unroll
+        for (int w = 1; w < WAVES_N; w++) {
+          t.x += part_lds[w * BM + tid].x;
+          t.y += part_lds[w * BM + tid].y;
+        }
+        reinterpret_cast<float2*>(p.stats_out)[(long long)(m0 + tid) * gridDim.y + blockIdx.y] = t;
+      }
+    }
+  }
 }
 
 // Outputs of at least 64 MiB, or of 32 MiB (the size of L2) from at least 16384 rows, are written with streaming stores:
@@ -558,15 +761,29 @@ inline bool StreamOutput(long long m, long long n, long long batch, int elem_byt
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
   dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch);
+  const dim3 block(WAVES_M * WAVES_N * 64);
+  auto launch = [&](auto stream_tag) {
+    constexpr bool S = decltype(stream_tag)::value;
+    if (a.skip != nullptr) {
+      if constexpr ((BN / WAVES_N) % 64 == 0 || BN / WAVES_N == 32) {
+        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 2>), grid, block, 0,
+                           stream, a);
+      }
+    } else if (a.row_stats != nullptr) {
+      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 1>), grid, block, 0,
+                         stream, a);
+    } else {
+      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 0>), grid, block, 0,
+                         stream, a);
+    }
+  };
   if constexpr (BM == 256) {
     if (StreamOutput(a.M, a.N, a.batch, 2)) {
-      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, true>), grid,
-                         dim3(WAVES_M * WAVES_N * 64), 0, stream, a);
+      launch(std::true_type{});
       return;
     }
   }
-  hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t>), grid,
-                     dim3(WAVES_M * WAVES_N * 64), 0, stream, a);
+  launch(std::false_type{});
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BKB = 128>
@@ -641,7 +858,8 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
     // workgroup per CU holds every CU for the whole launch, so the smolgen chain on the second stream no longer
     // slips in between rounds of tiles: a 15x1024 pass at batch 256 takes 6.66 ms with it against 5.91 ms.
     // It is reachable through SetGemmVariantOverride(kPersist256).)
-    if (c192 < cost) { best = kDma256x192; cost = c192; }
+    // (a producer of a folded layer norm needs a power-of-two column count per wave: not the 192-wide tile)
+    if (c192 < cost && a.skip == nullptr) { best = kDma256x192; cost = c192; }
     if (c128 < cost) { best = kDma256x128; cost = c128; }
     if (cs < cost) { best = kDma128x128; cost = cs; }
     // 128x64 tiles (three workgroups per CU, so partial rounds are counted as fractions) move more operand
@@ -670,6 +888,37 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
 
 void SetGemmVariantOverride(int variant) { g_variant_override = variant; }
 
+namespace {
+// Column-tile width of the direct-to-LDS variants (0 for the others).
+int DmaTileN(GemmVariant v) {
+  switch (v) {
+    case kDma256x256: return 256;
+    case kDma256x192: return 192;
+    case kDma256x128: case kDma128x128: return 128;
+    case kDma128x64: return 64;
+    default: return 0;
+  }
+}
+}  // namespace
+
+bool GemmSupportsNormFolding(const GemmArgs& a) {
+  const GemmVariant v = PickGemmVariant(a);
+  if (a.skip != nullptr) {
+    return DmaTileN(v) != 0 && v != kDma256x192 && !a.out_f32 && a.act == 3 && a.batch == 1 && a.N % 8 == 0 &&
+           a.ldc % 8 == 0 && a.ldskip % 8 == 0 && a.row_stats == nullptr;
+  }
+  if (a.row_stats != nullptr) {
+    if (a.split_k != 1 || a.batch != 1 || a.col_c == nullptr) return false;
+    return DmaTileN(v) != 0 || v == kTile128 || v == kTile64 || v == kRowPanel;
+  }
+  return true;
+}
+
+int GemmStatsParts(const GemmArgs& a) {
+  const int bn = DmaTileN(PickGemmVariant(a));
+  return bn == 0 ? 0 : (a.N + bn - 1) / bn;
+}
+
 const char* GemmVariantName(const GemmArgs& a) {
   switch (PickGemmVariant(a)) {
     case kPersist256: return "gemm_persistent_256x256x64";
@@ -686,6 +935,9 @@ const char* GemmVariantName(const GemmArgs& a) {
 
 void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
+  if ((a.skip != nullptr || a.row_stats != nullptr) && !GemmSupportsNormFolding(a)) {
+    throw std::runtime_error("LaunchGemm: no kernel variant with the folded layer-norm epilogue for this shape");
+  }
   switch (PickGemmVariant(a)) {
     case kPersist256: LaunchGemmPersistent(a, StreamOutput(a.M, a.N, a.batch, 2), stream); break;
     case kDma256x256: LaunchGemmDma<256, 256, 64, 2, 4>(a, stream); break;

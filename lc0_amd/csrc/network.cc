@@ -118,6 +118,26 @@ struct Linear {
   half_t* w = nullptr;   // [out][ld] halves, K zero-padded to ld
   float* b = nullptr;    // [out] or null
   int out = 0, in = 0, ld = 0;
+  float* c = nullptr;    // [out] row sums of w, for a layer whose input layer norm is folded into it (GemmArgs::col_c)
+};
+
+// The layer-norm side of one GEMM launch (see GemmArgs in kernels.h): the statistics of the rows the GEMM reads
+// (consumer), or the residual it adds and the statistics it leaves (producer).
+struct NormFold {
+  const float* row_stats = nullptr;
+  int row_parts = 0;
+  const half_t* skip = nullptr;
+  int ldskip = 0;
+  const float* skip_stats = nullptr;
+  int skip_parts = 0;
+  const float* skip_gamma = nullptr;
+  const float* skip_beta = nullptr;
+  float* stats_out = nullptr;
+  int* parts_out = nullptr;      // receives the number of partial sums per row written to stats_out
+  const float* bias = nullptr;   // replaces the layer's bias (producer: bias x scale)
+  float scale = 1.0f;
+  int norm_n = 0;
+  float eps = 0.0f;
 };
 
 int RoundUp(int v, int m) { return (v + m - 1) / m * m; }
@@ -159,6 +179,11 @@ struct EncoderDev {
   bool has_smolgen = false;
   Linear sg_compress, sg_dense1, sg_dense2;
   float *sg_ln1_g = nullptr, *sg_ln1_b = nullptr, *sg_ln2_g = nullptr, *sg_ln2_b = nullptr;
+  // Folded layer norms: the three layers that read normalised rows, with the gamma / beta of the norm before them
+  // multiplied in (qkv and sg_compress: the second norm of the previous encoder layer, absent in the first layer;
+  // ffn1: this layer's first norm), and the biases of the two layers before a norm times the DeepNorm alpha.
+  Linear qkv_n, sg_compress_n, ffn1_n;
+  float *dense_ab = nullptr, *ffn2_ab = nullptr;
 };
 
 // Pinned host staging of one batch (inputs and outputs).
@@ -255,6 +280,7 @@ struct ModelState {
   int sg_hc_ = 0, sg_hs_ = 0, sg_gen_ = 0;
   int pol_emb_ = 0, pol_d_ = 0, val_ch_ = 0, val_fc_ = 0, val_out_ = 0, mov_ch_ = 0, mov_fc_ = 0;
   float alpha_ = 1.0f, eps_ = 1e-6f;
+  bool fold_layer_norm_ = false;
   bool any_smolgen_ = false;
   // Dense position encoding (PE_DENSE nets): preprocessing layer, embedding layer norm and
   // embedding FFN; optional input gating.
@@ -342,6 +368,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   template <typename T>
   struct LinearT MakeLinearT(const Vec& w, const Vec& b, int out, int in);
   Linear MakeLinear(const Vec& w, const Vec& b, int out, int in, int pad_to = 8);
+  Linear MakeLinearNormFolded(const Vec& w, const Vec& b, const Vec& gamma, const Vec& beta, int out, int in);
   LinearF8 MakeLinearF8(const Vec& w, int out, int in);
   void GemmF8(const char* name, const uint8_t* A, const Linear& lin, const LinearF8& q, void* C, int M, int act,
               bool out_f8, float out_mul);
@@ -364,7 +391,11 @@ class Mi355xNetwork : public Network, protected ModelState {
   template <typename F>
   void Timed(const char* name, double flops, double bytes, F&& launch, hipStream_t st = nullptr);
   void Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act,
-            bool out_f32 = false, hipStream_t st = nullptr, int split_k = 1, bool latency_first = false);
+            bool out_f32 = false, hipStream_t st = nullptr, int split_k = 1, bool latency_first = false,
+            const NormFold* fold = nullptr);
+  GemmArgs MakeGemmArgs(const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act, bool out_f32,
+                        int split_k, bool latency_first, const NormFold* fold) const;
+  bool CanFoldLayerNorms(int B) const;
 
   // ---- per-lane state: streams, activations, recorded graphs ----
   hipStream_t stream_ = nullptr;
@@ -381,6 +412,8 @@ class Mi355xNetwork : public Network, protected ModelState {
   half_t *in0_ = nullptr, *x_ = nullptr, *t_ = nullptr, *qkv_ = nullptr, *att_ = nullptr, *ffn_ = nullptr;
   half_t *sg1_ = nullptr, *sg2_ = nullptr, *sg3_ = nullptr, *sbias_ = nullptr;
   float* sg2f_ = nullptr;  // split-K accumulator of smolgen dense1
+  // Partial row sums of the two un-normalised sums of an encoder layer (folded layer norms): [rows][parts][2].
+  float *ln_stats_a_ = nullptr, *ln_stats_b_ = nullptr;
   half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
   half_t *pe_qkv_ = nullptr, *pe_att_ = nullptr, *pe_t_ = nullptr, *pe_ffn_ = nullptr;   // policy encoder scratch
   float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
@@ -501,9 +534,40 @@ Linear Mi355xNetwork::MakeLinear(const Vec& w, const Vec& b, int out, int in, in
   return l;
 }
 
-void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M,
-                         int act, bool out_f32, hipStream_t st, int split_k, bool latency_first) {
-  if (st == nullptr) st = stream_;
+// A layer that reads layer-normalised rows, prepared for reading the un-normalised rows instead (the consumer
+// side of GemmArgs): weights w[o][i] * gamma[i], their row sums as stored (after rounding to half, so that the
+// mean cancels exactly), and the bias plus sum_i beta[i] w[o][i].
+Linear Mi355xNetwork::MakeLinearNormFolded(const Vec& w, const Vec& b, const Vec& gamma, const Vec& beta, int out,
+                                           int in) {
+  if (w.size() != static_cast<size_t>(out) * in || gamma.size() != static_cast<size_t>(in) ||
+      beta.size() != static_cast<size_t>(in) || (!b.empty() && b.size() != static_cast<size_t>(out))) {
+    throw Error("A dense layer has a wrong number of weights.");
+  }
+  Linear l;
+  l.out = out; l.in = in;
+  l.ld = RoundUp(in, 8);
+  std::vector<half_t> h(static_cast<size_t>(out) * l.ld, (half_t)0.0f);
+  std::vector<float> c(out), d(out);
+  for (int o = 0; o < out; o++) {
+    double csum = 0.0, dsum = b.empty() ? 0.0 : b[o];
+    for (int i = 0; i < in; i++) {
+      const double wv = w[static_cast<size_t>(o) * in + i];
+      const half_t hv = (half_t)static_cast<float>(wv * gamma[i]);
+      h[static_cast<size_t>(o) * l.ld + i] = hv;
+      csum += static_cast<double>(static_cast<float>(hv));
+      dsum += wv * beta[i];
+    }
+    c[o] = static_cast<float>(csum);
+    d[o] = static_cast<float>(dsum);
+  }
+  l.w = arena_.Upload(h);
+  l.b = arena_.Upload(d);
+  l.c = arena_.Upload(c);
+  return l;
+}
+
+GemmArgs Mi355xNetwork::MakeGemmArgs(const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act,
+                                     bool out_f32, int split_k, bool latency_first, const NormFold* fold) const {
   GemmArgs g;
   g.latency_first = latency_first;
   g.split_k = split_k;
@@ -515,11 +579,59 @@ void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linea
   g.M = M; g.N = lin.out; g.K = lin.ld;
   g.act = act;
   g.out_f32 = out_f32;
+  if (fold != nullptr) {
+    g.row_stats = fold->row_stats; g.row_parts = fold->row_parts; g.col_c = lin.c;
+    g.skip = fold->skip; g.ldskip = fold->ldskip;
+    g.skip_stats = fold->skip_stats; g.skip_parts = fold->skip_parts;
+    g.skip_gamma = fold->skip_gamma; g.skip_beta = fold->skip_beta;
+    g.stats_out = fold->stats_out;
+    g.norm_n = fold->norm_n; g.norm_eps = fold->eps;
+    g.scale = fold->scale;
+    if (fold->bias != nullptr) g.bias = fold->bias;
+  }
+  return g;
+}
+
+void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M,
+                         int act, bool out_f32, hipStream_t st, int split_k, bool latency_first,
+                         const NormFold* fold) {
+  if (st == nullptr) st = stream_;
+  const GemmArgs g = MakeGemmArgs(A, lda, lin, C, ldc, M, act, out_f32, split_k, latency_first, fold);
+  if (fold != nullptr && fold->parts_out != nullptr) *fold->parts_out = GemmStatsParts(g);
   const double flops = 2.0 * M * lin.out * lin.in;
   const double bytes = 2.0 * (static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in) +
-                       static_cast<double>(M) * lin.out * (out_f32 ? 4 : 2);
-  const std::string label = std::string(name) + "|" + GemmVariantName(g);
+                       static_cast<double>(M) * lin.out * (out_f32 ? 4 : 2) +
+                       (fold != nullptr && fold->skip != nullptr ? 2.0 * M * lin.out : 0.0);
+  std::string label = std::string(name) + "|" + GemmVariantName(g);
+  if (fold != nullptr) label += fold->skip != nullptr ? "+skip_stats" : "+row_norm";
   Timed(label.c_str(), flops, bytes, [&] { LaunchGemm(g, st); }, st);
+}
+
+// Whether a pass over B positions can run the encoder stack with its layer norms folded into the GEMMs around
+// them: every one of the five launches per layer must get a kernel variant that has the epilogue.
+bool Mi355xNetwork::CanFoldLayerNorms(int B) const {
+  if (!fold_layer_norm_ || encoders_.empty() || encoders_[0].ffn1_n.w == nullptr) return false;
+  const int T = B * 64;
+  const half_t* any_h = x_;
+  const float* any_f = ln_stats_a_;
+  const EncoderDev& e = encoders_.back();
+  NormFold cons;
+  cons.row_stats = any_f; cons.row_parts = 1; cons.norm_n = emb_;
+  NormFold prod;
+  prod.skip = any_h; prod.ldskip = emb_; prod.stats_out = ln_stats_a_; prod.norm_n = emb_;
+  const bool chain_first = B <= 128;
+  if (!GemmSupportsNormFolding(MakeGemmArgs(x_, emb_, e.qkv_n, qkv_, 3 * d_model_, T, kActNone, false, 1, false, &cons)) ||
+      !GemmSupportsNormFolding(MakeGemmArgs(x_, emb_, e.ffn1_n, ffn_, dff_, T, ffn_act_, false, 1, false, &cons)) ||
+      !GemmSupportsNormFolding(MakeGemmArgs(att_, d_model_, e.dense, x_, emb_, T, kActNone, false, 1, false, &prod)) ||
+      !GemmSupportsNormFolding(MakeGemmArgs(ffn_, dff_, e.ffn2, x_, emb_, T, kActNone, false, 1, false, &prod))) {
+    return false;
+  }
+  if (e.has_smolgen &&
+      !GemmSupportsNormFolding(
+          MakeGemmArgs(x_, emb_, e.sg_compress_n, sg1_, sg_hc_, T, kActNone, false, 1, chain_first, &cons))) {
+    return false;
+  }
+  return true;
 }
 
 // ------------------------------------------------------------------- fp8 --
@@ -752,6 +864,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
       pos = end + 1;
     }
   }
+  fold_layer_norm_ = options.GetBool("fold_layer_norm", false);
   fp8_fp16_layers_ = options.GetInt("fp8_fp16_layers", 0);
   if (fp8_fp16_layers_ < 0) throw Error("fp8_fp16_layers must not be negative.");
   use_graphs_ = options.GetBool("graphs", true);
@@ -891,6 +1004,12 @@ void Mi355xNetwork::AllocActivations() {
   if (pe_dense_) {
     pre_in_ = AllocH(static_cast<size_t>(max_batch_) * 768);
     pre_out_ = AllocH(T * enc_ch_);
+  }
+  if (!encoders_.empty() && encoders_[0].ffn1_n.w != nullptr) {
+    // at most one part per 64 columns (the narrowest column tile of the GEMM variants that write them)
+    const size_t n = T * static_cast<size_t>((emb_ + 63) / 64) * 2;
+    ln_stats_a_ = AllocF(n);
+    ln_stats_b_ = AllocF(n);
   }
   if (any_smolgen_) {
     sg1_ = AllocH(T * sg_hc_);
@@ -1124,6 +1243,26 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
       e.sg_dense2 = MakeLinear(s.dense2_w, s.dense2_b, gen, hs);
       e.sg_ln1_g = UploadN(s.ln1_gammas, hs, "Smolgen layer norm gamma"); e.sg_ln1_b = UploadN(s.ln1_betas, hs, "Smolgen layer norm beta");
       e.sg_ln2_g = UploadN(s.ln2_gammas, gen, "Smolgen layer norm gamma"); e.sg_ln2_b = UploadN(s.ln2_betas, gen, "Smolgen layer norm beta");
+    }
+    if (fold_layer_norm_ && !fp8_ && emb_ % 8 == 0) {
+      // Folded layer norms (fp16 path): the layers after a norm get its gamma and beta multiplied in, the layers
+      // before one get alpha multiplied into their bias (the GEMM scales the sum by alpha).
+      const size_t li = encoders_.size();
+      e.ffn1_n = MakeLinearNormFolded(l.ffn.dense1_w, l.ffn.dense1_b, l.ln1_gammas, l.ln1_betas, dff_, emb_);
+      if (li > 0) {
+        const EncoderLayer& prev = w.encoder[li - 1];
+        e.qkv_n = MakeLinearNormFolded(qkv_w, qkv_b, prev.ln2_gammas, prev.ln2_betas, 3 * d_model_, emb_);
+        if (e.has_smolgen) {
+          e.sg_compress_n = MakeLinearNormFolded(l.mha.smolgen.compress, Vec(), prev.ln2_gammas, prev.ln2_betas,
+                                                 sg_hc_, emb_);
+        }
+      }
+      Vec ab(l.mha.dense_b);
+      for (float& v : ab) v *= alpha_;
+      e.dense_ab = UploadF(ab);
+      ab = l.ffn.dense2_b;
+      for (float& v : ab) v *= alpha_;
+      e.ffn2_ab = UploadF(ab);
     }
     encoders_.push_back(e);
   }
@@ -1450,11 +1589,29 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
           [&] { LaunchQuantizeF8(x_, xq_, static_cast<long long>(nx), 1.0f / encoders_[0].s_x, stream_); });
   }
 
+  // Folded layer norms (fp16 arithmetic, batches whose GEMMs all run on the direct-to-LDS kernels): the two
+  // norms of a layer run inside the GEMM before them (residual + row sums) and the GEMMs after them (row
+  // normalisation of the product), and x_ carries the un-normalised sums from layer to layer.
+  const bool fold = !fp8_ && !calibrating_ && CanFoldLayerNorms(B);
+  const float* pend_stats = nullptr;   // row sums of x_ when it holds an un-normalised sum
+  const float *pend_gamma = nullptr, *pend_beta = nullptr;
+  int pend_parts = 0, mid_parts = 0;
   for (size_t li = 0; li < encoders_.size(); li++) {
     const EncoderDev& e = encoders_[li];
     const bool last = li + 1 == encoders_.size();
     const bool f8 = f8_any && li < n_f8_layers;
     const half_t* bias = nullptr;
+    // Folded layer norms: x_ holds the un-normalised sum u when `pending` is set; the layers that read it take
+    // the consumer epilogue, the two layers before a norm add the residual in place and leave the row sums.
+    NormFold cons_in, cons_mid, prod_mid, prod_out;
+    if (fold) {
+      cons_in.row_stats = pend_stats; cons_in.row_parts = pend_parts; cons_in.norm_n = emb_; cons_in.eps = eps_;
+      prod_mid.skip = x_; prod_mid.ldskip = emb_; prod_mid.skip_stats = pend_stats; prod_mid.skip_parts = pend_parts;
+      prod_mid.skip_gamma = pend_gamma; prod_mid.skip_beta = pend_beta;
+      prod_mid.stats_out = ln_stats_b_; prod_mid.parts_out = &mid_parts;
+      prod_mid.bias = e.dense_ab; prod_mid.scale = alpha_; prod_mid.norm_n = emb_; prod_mid.eps = eps_;
+    }
+    const bool norm_in = fold && pend_stats != nullptr;   // this layer reads an un-normalised x_
     // The smolgen chain depends only on x: it runs on the side stream next to the
     // QKV projection (on the main stream when profiling, for clean per-kernel times).
     hipStream_t ss = (profiling_ || single_stream_ || B < overlap_min_batch_) ? stream_ : side_stream_;
@@ -1468,7 +1625,8 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       // or at most 128 positions): its kernels then take the variants with the shortest latency. At larger fp16
       // batches the two are balanced and the leaner variants disturb the projection less (batch 256: 1.5 %).
       const bool chain_first = f8 || B <= 128;
-      Gemm("gemm_smolgen_compress", x_, emb_, e.sg_compress, sg1_, sg_hc_, T, kActNone, false, ss, 1, chain_first);
+      Gemm("gemm_smolgen_compress", x_, emb_, norm_in ? e.sg_compress_n : e.sg_compress, sg1_, sg_hc_, T, kActNone,
+           false, ss, 1, chain_first, norm_in ? &cons_in : nullptr);
       // dense1 has a long reduction and few outputs: split K, accumulate in float,
       // and let the layer norm kernel apply the activation.
       const int split = std::max(1, std::min(16, (64 * sg_hc_) / 256));
@@ -1489,7 +1647,8 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     if (f8 && q_qkv_) {
       GemmF8("gemm_qkv", xq_, e.qkv, e.qkv8, qkv_, T, kActNone, false, 1.0f);
     } else {
-      Gemm("gemm_qkv", x_, emb_, e.qkv, qkv_, 3 * d_model_, T, kActNone);
+      Gemm("gemm_qkv", x_, emb_, norm_in ? e.qkv_n : e.qkv, qkv_, 3 * d_model_, T, kActNone, false, nullptr, 1, false,
+           norm_in ? &cons_in : nullptr);
     }
     if (e.has_smolgen && ss != stream_) HIP_CHECK(hipStreamWaitEvent(stream_, join_events_[li], 0));
     const double att_flops = 4.0 * 64 * 64 * depth_ * B * heads_;
@@ -1505,6 +1664,24 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       Timed("attention", att_flops, att_bytes,
             [&] { LaunchAttention(qkv_, bias, att_, B, heads_, att_scale, stream_, depth_); });
       if (calibrating_) RecordAbsMax(att_, static_cast<size_t>(T) * d_model_, static_cast<int>(4 * li + 1));
+      if (fold) {
+        // x_ <- alpha * (att . dense + b) + LN2_prev(x_), with the row sums of the new x_
+        Gemm("gemm_mha_dense", att_, d_model_, e.dense, x_, emb_, T, kActNone, false, nullptr, 1, false, &prod_mid);
+        cons_mid.row_stats = ln_stats_b_; cons_mid.row_parts = mid_parts; cons_mid.norm_n = emb_; cons_mid.eps = eps_;
+        Gemm("gemm_ffn1", x_, emb_, e.ffn1_n, ffn_, dff_, T, ffn_act_, false, nullptr, 1, false, &cons_mid);
+        prod_out.skip = x_; prod_out.ldskip = emb_; prod_out.skip_stats = ln_stats_b_; prod_out.skip_parts = mid_parts;
+        prod_out.skip_gamma = e.ln1_g; prod_out.skip_beta = e.ln1_b;
+        prod_out.stats_out = ln_stats_a_; prod_out.parts_out = &pend_parts;
+        prod_out.bias = e.ffn2_ab; prod_out.scale = alpha_; prod_out.norm_n = emb_; prod_out.eps = eps_;
+        Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, x_, emb_, T, kActNone, false, nullptr, 1, false, &prod_out);
+        pend_stats = ln_stats_a_; pend_gamma = e.ln2_g; pend_beta = e.ln2_b;
+        if (last) {   // the heads read normalised rows
+          Timed("layer_norm", 0.0, 4.0 * T * emb_, [&] {
+            LaunchLayerNorm(x_, nullptr, x_, pend_gamma, pend_beta, T, emb_, 1.0f, eps_, stream_, nullptr, 1.0f);
+          });
+        }
+        continue;
+      }
       Gemm("gemm_mha_dense", att_, d_model_, e.dense, t_, emb_, T, kActNone);
     }
     const bool ln1_f8 = f8 && q_ffn1_;

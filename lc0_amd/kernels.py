@@ -18,6 +18,9 @@ def _lib():
         vp, ci, ll, cf, cd = C.c_void_p, C.c_int, C.c_longlong, C.c_float, C.POINTER(C.c_double)
         lib.lc0mi_k_gemm.argtypes = [vp, ci, ll, vp, ci, ll, vp, ci, ci, ci, ci, cf, ci, ci, vp, ci, ll, ci, cd]
         lib.lc0mi_k_gemm_splitk.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, ci, cf, vp, ci]
+        lib.lc0mi_k_gemm_norm_producer.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, vp, vp, ci, vp, vp, cf, vp, vp, ci,
+                                                   C.POINTER(C.c_int), ci, cd]
+        lib.lc0mi_k_gemm_norm_consumer.argtypes = [vp, ci, vp, ci, vp, vp, ci, ci, ci, vp, ci, cf, ci, ci, vp, ci, ci, cd]
         lib.lc0mi_k_layer_norm_rows.argtypes = [vp, vp, ci, vp, vp, vp, ci, ci, cf, cf, vp]
         lib.lc0mi_k_winograd_conv.argtypes = [vp] * 8 + [ci] * 6 + [vp] * 3
         lib.lc0mi_k_expand_planes_nhwc.argtypes = [vp, vp, ci, vp]
@@ -72,6 +75,47 @@ def set_gemm_variant(variant):
     6 row-panel 64x32, 7 direct-to-LDS 128x64, 8 persistent 256x256 (one workgroup per CU walks over the tiles;
     M, N multiples of 256, K of 128; other shapes fall back to the automatic choice)."""
     _lib().lc0mi_k_set_gemm_variant(int(variant))
+
+
+def gemm_norm_producer(a, w, bias, skip, scale=1.0, skip_stats=None, skip_gamma=None, skip_beta=None, eps=1e-6,
+                       time_iters=0):
+    """U = scale * a @ w^T + bias + s (halves) and the partial row sums of U, [M, parts, 2]; s = skip, or the layer
+    norm of skip's rows when skip_stats [M, parts, 2] (with skip_gamma, skip_beta) is given.
+    Returns (U, stats) or (U, stats, ms)."""
+    a, w, skip = _h(a), _h(w), _h(skip)
+    m, k = a.shape
+    n = w.shape[0]
+    b = np.ascontiguousarray(bias, np.float32) if bias is not None else None
+    st = np.ascontiguousarray(skip_stats, np.float32) if skip_stats is not None else None
+    g = np.ascontiguousarray(skip_gamma, np.float32) if skip_stats is not None else None
+    be = np.ascontiguousarray(skip_beta, np.float32) if skip_stats is not None else None
+    u = np.zeros((m, n), np.float16)
+    cap_parts = (n + 63) // 64
+    stats = np.zeros((m, cap_parts, 2), np.float32)
+    parts = C.c_int(0)
+    ms = C.c_double(0.0)
+    _check(_lib().lc0mi_k_gemm_norm_producer(
+        _ptr(a), k, _ptr(w), k, _ptr(b), m, n, k, scale, _ptr(skip), _ptr(st),
+        0 if st is None else st.shape[1], _ptr(g), _ptr(be), eps, _ptr(u), _ptr(stats), stats.size,
+        C.byref(parts), time_iters, C.byref(ms)))
+    stats = stats.reshape(-1)[:m * parts.value * 2].reshape(m, parts.value, 2).copy()
+    return (u, stats, ms.value) if time_iters else (u, stats)
+
+
+def gemm_norm_consumer(u, w, col_c, bias, stats, eps=1e-6, act=ACT_NONE, latency_first=False, time_iters=0):
+    """act(rstd * (u @ w^T - mean x col_c) + bias) with the row statistics of u from stats [M, parts, 2]."""
+    u, w = _h(u), _h(w)
+    m, k = u.shape
+    n = w.shape[0]
+    c = np.ascontiguousarray(col_c, np.float32)
+    b = np.ascontiguousarray(bias, np.float32) if bias is not None else None
+    st = np.ascontiguousarray(stats, np.float32)
+    out = np.zeros((m, n), np.float16)
+    ms = C.c_double(0.0)
+    _check(_lib().lc0mi_k_gemm_norm_consumer(
+        _ptr(u), k, _ptr(w), k, _ptr(c), _ptr(b), m, n, k, _ptr(st), st.shape[1], eps, act,
+        int(latency_first), _ptr(out), n, time_iters, C.byref(ms)))
+    return (out, ms.value) if time_iters else out
 
 
 def gemm_splitk(a, w, bias=None, split_k=4, scale=1.0):

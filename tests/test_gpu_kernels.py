@@ -385,3 +385,101 @@ def test_legal_softmax_bit_exact_vs_oracle():
         for i, ids in enumerate(lists):
             want = onn.softmax_policy_legal(policy[i], ids, t)
             np.testing.assert_array_equal(got[i].view(np.uint32), want.view(np.uint32), err_msg="row %d T %g" % (i, t))
+
+
+def _fold_norm_into_layer(w, b, gamma, beta):
+    """Host-side preparation of a layer that follows a layer norm: weights times gamma (as halves), their row sums
+    as stored, and the bias plus the beta term."""
+    wg = np.asarray(w.astype(np.float64) * gamma[None, :], np.float16)
+    c = wg.astype(np.float64).sum(axis=1).astype(f32)
+    d = (b.astype(np.float64) + w.astype(np.float64) @ beta.astype(np.float64)).astype(f32)
+    return wg, c, d
+
+
+@pytest.mark.parametrize("m,n,k,n2,act,skip_is_sum", [
+    (16384, 1024, 1024, 1536, nr.ACT_MISH, True),    # 256x256 producer, 256x192 consumer (the BT4 shapes)
+    (2048, 1024, 1536, 3072, nr.ACT_NONE, True),
+    (2100, 512, 256, 32, nr.ACT_NONE, False),        # ragged rows; the consumer is a single 32-column panel
+    (4096, 256, 128, 256, nr.ACT_RELU, True),        # 128x64 tiles: four lanes per row in the producer
+    (4096, 768, 768, 64, nr.ACT_SWISH, False),
+])
+def test_layer_norm_folded_into_the_gemms_around_it(m, n, k, n2, act, skip_is_sum):
+    """x1 = LN(alpha * (a . w1 + b1) + s) followed by act(x1 . w2 + b2), against the oracle's dense layer and
+    layer norm (LayerNorm2DWithSkipConnection), with the norm computed inside the two GEMMs: the first leaves the
+    un-normalised sum and its row sums, the second normalises its product. s is either given, or itself the layer
+    norm of an un-normalised sum s0 whose statistics and gamma / beta the first GEMM receives."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(m + 3 * n + 5 * k + n2)
+    eps, alpha = 1e-6, 0.43
+    a = _h(rng.standard_normal((m, k)) * 0.5)
+    w1 = _h(rng.standard_normal((n, k)) * (1.0 / np.sqrt(k)))
+    b1 = (rng.standard_normal(n) * 0.1).astype(f32)
+    g1 = (1.0 + 0.2 * rng.standard_normal(n)).astype(f32)
+    be1 = (0.1 * rng.standard_normal(n)).astype(f32)
+    w2 = _h(rng.standard_normal((n2, n)) * (1.0 / np.sqrt(n)))
+    b2 = (rng.standard_normal(n2) * 0.1).astype(f32)
+    s0 = _h(rng.standard_normal((m, n)) * 1.5 + 0.7 * rng.standard_normal((m, 1)))   # rows with a mean of their own
+    g0 = (1.0 + 0.2 * rng.standard_normal(n)).astype(f32)
+    be0 = (0.1 * rng.standard_normal(n)).astype(f32)
+    if skip_is_sum:
+        s0_stats = np.stack([s0.sum(axis=1), (s0.astype(np.float64) ** 2).sum(axis=1)], axis=1).astype(f32)
+        # as three partial sums per row, the last two empty, to exercise the addition of parts
+        s0_stats = np.concatenate([s0_stats[:, None, :], np.zeros((m, 2, 2), f32)], axis=1)
+        s = onn.layer_norm_skip(s0, 1.0, None, g0, be0, eps)
+        u, stats = K.gemm_norm_producer(a, w1, b1 * alpha, s0, scale=alpha, skip_stats=s0_stats, skip_gamma=g0,
+                                        skip_beta=be0, eps=eps)
+    else:
+        s = s0
+        u, stats = K.gemm_norm_producer(a, w1, b1 * alpha, s0, scale=alpha, eps=eps)
+    t = onn.fc(a, w1.reshape(-1), b1, nr.ACT_NONE)
+    want_u = alpha * t + s
+    u32 = u.astype(f32)
+    # two roundings to half on the way (the product, then the sum)
+    np.testing.assert_allclose(u32, want_u, rtol=3e-3, atol=3e-3)
+    # the row sums describe U as stored, up to the rounding of its n elements to half (2^-11 relative each, taken
+    # before the rounding: six standard deviations of the accumulated rounding errors are about 0.1 for the sums)
+    np.testing.assert_allclose(stats[:, :, 0].sum(axis=1), u32.astype(np.float64).sum(axis=1), rtol=1e-4, atol=0.1)
+    np.testing.assert_allclose(stats[:, :, 1].sum(axis=1), (u32.astype(np.float64) ** 2).sum(axis=1), rtol=1e-3)
+    # consumer: against the oracle's layer norm of the stored U followed by its dense layer
+    wg, c, d = _fold_norm_into_layer(w2, b2, g1, be1)
+    got = K.gemm_norm_consumer(u, wg, c, d, stats, eps=eps, act=act, latency_first=(n2 <= 32)).astype(f32)
+    x1 = onn.layer_norm_skip(u32, 1.0, None, g1, be1, eps)
+    want = onn.fc(x1, w2.reshape(-1), b2, act)
+    # fp16 output, gamma-scaled weights rounded to half once more: 3e-3 of the output scale (about 1)
+    np.testing.assert_allclose(got, want, rtol=4e-3, atol=4e-3)
+    # and the pair against the unfused pair of kernels on the same inputs
+    t16 = K.gemm(a, w1, b1)
+    x1_k = K.layer_norm(t16, s.astype(np.float16), g1, be1, alpha, eps)
+    ref_pair = K.gemm(x1_k, w2, b2, act=act).astype(f32)
+    assert np.abs(got - want).max() <= 2.0 * np.abs(ref_pair - want).max() + 2e-3
+
+
+@pytest.mark.parametrize("producer_variant,consumer_variant", [(0, 1), (2, 2), (5, 5), (7, 7), (0, 3), (7, 4), (2, 0)])
+def test_layer_norm_folding_in_every_gemm_variant_that_has_it(producer_variant, consumer_variant):
+    """The same pair as above on one shape with the kernel variants forced: every direct-to-LDS tile shape as
+    producer (except 256x192, which the choice never takes for one) and every variant as consumer."""
+    from lc0_amd import kernels as K
+    m, n, k, n2 = 2100, 512, 256, 384
+    rng = np.random.default_rng(producer_variant * 16 + consumer_variant)
+    eps, alpha = 1e-6, 0.5
+    a = _h(rng.standard_normal((m, k)) * 0.5)
+    w1 = _h(rng.standard_normal((n, k)) * (1.0 / np.sqrt(k)))
+    b1 = (rng.standard_normal(n) * 0.1).astype(f32)
+    g1 = (1.0 + 0.2 * rng.standard_normal(n)).astype(f32)
+    be1 = (0.1 * rng.standard_normal(n)).astype(f32)
+    w2 = _h(rng.standard_normal((n2, n)) * (1.0 / np.sqrt(n)))
+    b2 = (rng.standard_normal(n2) * 0.1).astype(f32)
+    s = _h(rng.standard_normal((m, n)) + 0.5 * rng.standard_normal((m, 1)))
+    wg, c, d = _fold_norm_into_layer(w2, b2, g1, be1)
+    try:
+        K.set_gemm_variant(producer_variant)
+        u, stats = K.gemm_norm_producer(a, w1, b1 * alpha, s, scale=alpha, eps=eps)
+        K.set_gemm_variant(consumer_variant)
+        got = K.gemm_norm_consumer(u, wg, c, d, stats, eps=eps, act=nr.ACT_MISH).astype(f32)
+    finally:
+        K.set_gemm_variant(-1)
+    assert stats.shape[1] == -(-n // {0: 256, 2: 128, 5: 128, 7: 64}[producer_variant])
+    u32 = u.astype(f32)
+    np.testing.assert_allclose(u32, alpha * onn.fc(a, w1.reshape(-1), b1, nr.ACT_NONE) + s, rtol=3e-3, atol=3e-3)
+    want = onn.fc(onn.layer_norm_skip(u32, 1.0, None, g1, be1, eps), w2.reshape(-1), b2, nr.ACT_MISH)
+    np.testing.assert_allclose(got, want, rtol=4e-3, atol=4e-3)

@@ -82,6 +82,26 @@ def test_attention_nets_match_oracle(name, batch, positions):
     np.testing.assert_allclose(comp.GetDVal(0) + 0 * comp.GetMVal(0), res["d"][3], atol=2e-3)
 
 
+@pytest.mark.parametrize("name,batch", [("c1_attn_10x256", 64), ("c2_bt4_15x1024", 32)])
+def test_layer_norms_folded_into_the_gemms_match_oracle(name, batch, positions):
+    """Option fold_layer_norm=true: LayerNorm2DWithSkipConnection (src/neural/backends/blas/encoder.h:29-66) runs
+    inside the GEMMs on either side of it. Same bar as the default path; the profile must name the folded
+    variants, so that a silent return to the separate kernels cannot pass."""
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    net, res = _run_gpu(path, masks, values, "fold_layer_norm=true")
+    _compare(res, want, positions["legal"][:batch])
+    net.SetProfiling(True)
+    comp = net.NewComputation()
+    comp.AddInputs(masks, values)
+    comp.ComputeBlocking()
+    names = [k.name for k in net.TakeProfile()]
+    net.SetProfiling(False)
+    assert any(n.endswith("+skip_stats") for n in names) and any(n.endswith("+row_norm") for n in names), names
+    assert not any(n == "layer_norm_skip" for n in names), names
+
+
 @pytest.mark.parametrize("name,batch,options,tol", [
     ("tiny_resnet", 19, "precision=fp32", 1e-3), ("tiny_resnet", 19, "precision=fp16", 5e-3),
     ("tiny_resnet_convpolicy", 8, "precision=fp32", 1e-3), ("tiny_resnet_nose", 8, "precision=fp32", 1e-3),
