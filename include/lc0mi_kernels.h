@@ -107,6 +107,13 @@ int lc0mi_k_quantize_f8(const uint16_t* x, long long n, float mul, uint8_t* y);
 /* lc0mi_k_layer_norm with a second, e4m3 output y_f8 = e4m3(y * f8_mul). */
 int lc0mi_k_layer_norm_f8(const uint16_t* x, const uint16_t* skip, const float* gamma, const float* beta, int rows,
                           int C, float alpha, float eps, float f8_mul, uint16_t* y, uint8_t* y_f8);
+/* The shared smolgen generator layer and the attention in one kernel (network_blas.cc:332-347 followed by :352-439):
+ * logits[b][h][q][k] = scale * Q.K^T + sum_j w[q*64+k][j] * gen[b][h][j], out = softmax_k(logits) . V.
+ * qkv [B*64][3*heads*32] halves, gen [B][heads][gen_sz] halves, w [4096][gen_sz] halves (row q*64+k); head depth 32,
+ * heads <= 32, gen_sz 32, 128 or 256. out [B*64][heads*32]: halves, or e4m3(out * out_mul) bytes when f8_out. */
+int lc0mi_k_smolgen_attention(const uint16_t* qkv, const uint16_t* gen, const uint16_t* w, int batch, int heads,
+                              int gen_sz, float scale, int f8_out, float out_mul, void* out, int time_iters,
+                              double* ms);
 /* lc0mi_k_attention with e4m3 output e4m3(out * out_mul). */
 int lc0mi_k_attention_f8(const uint16_t* qkv, const uint16_t* bias, int batch, int heads, float scale, float out_mul,
                          uint8_t* out);

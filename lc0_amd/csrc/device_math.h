@@ -1,4 +1,4 @@
-// Device-side activation functions shared by the kernel sources.
+// Device-side activation functions and the e4m3 pack shared by the kernel sources.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -33,5 +33,16 @@ static __device__ __forceinline__ float Activate(float v, int act) {
   }
 }
 
+// 4 floats -> 4 e4m3 bytes (round to nearest even, saturating at +-448; the
+// hardware conversion alone would turn |v| > 464 into NaN).
+static __device__ __forceinline__ unsigned PackFp8x4(float a, float b, float c, float d) {
+  a = __builtin_amdgcn_fmed3f(a, -448.0f, 448.0f);  // median of three = clamp, one instruction
+  b = __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f);
+  c = __builtin_amdgcn_fmed3f(c, -448.0f, 448.0f);
+  d = __builtin_amdgcn_fmed3f(d, -448.0f, 448.0f);
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return (unsigned)v;
+}
 
 }  // namespace lc0mi

@@ -575,6 +575,39 @@ int lc0mi_k_attention_f8(const uint16_t* qkv, const uint16_t* bias, int batch, i
   });
 }
 
+int lc0mi_k_smolgen_attention(const uint16_t* qkv, const uint16_t* gen, const uint16_t* w, int batch, int heads,
+                              int gen_sz, float scale, int f8_out, float out_mul, void* out, int time_iters,
+                              double* ms) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1 || !lc0mi::SmolgenAttentionSupported(heads, 32, gen_sz)) throw Error("bad smolgen attention shape");
+    Dev dev;
+    const int d = heads * 32;
+    auto* dq = reinterpret_cast<half_t*>(dev.Put(qkv, (size_t)batch * 64 * 3 * d));
+    auto* dg = reinterpret_cast<half_t*>(dev.Put(gen, (size_t)batch * heads * gen_sz));
+    std::vector<uint16_t> frag((size_t)4096 * gen_sz);
+    for (int row = 0; row < 4096; row++)
+      for (int col = 0; col < gen_sz; col++)
+        frag[lc0mi::SmolgenFragmentIndex(row, col, gen_sz)] = w[(size_t)row * gen_sz + col];
+    auto* dw = reinterpret_cast<half_t*>(dev.Put(frag.data(), frag.size()));
+    const size_t out_bytes = (size_t)batch * 64 * d * (f8_out ? 1 : 2);
+    void* dout = dev.Alloc(out_bytes);
+    auto launch = [&] {
+      if (f8_out) {
+        lc0mi::LaunchSmolgenAttentionF8Out(dq, dg, dw, static_cast<uint8_t*>(dout), out_mul, batch, heads, 32, gen_sz,
+                                           scale, nullptr);
+      } else {
+        lc0mi::LaunchSmolgenAttention(dq, dg, dw, static_cast<half_t*>(dout), batch, heads, 32, gen_sz, scale, nullptr);
+      }
+    };
+    launch();
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(out, dout, out_bytes, hipMemcpyDeviceToHost));
+    if (time_iters > 0 && ms) *ms = TimeLaunches(time_iters, launch);
+  });
+}
+
 int lc0mi_k_copy(long long bytes, int iters, double* ms) {
   return Guard([&] {
     RequireDevice();

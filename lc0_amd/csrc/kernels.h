@@ -167,6 +167,19 @@ void LaunchAttentionF8Out(const half_t* qkv, const half_t* bias, uint8_t* out, f
 // Position inside one head's 4096-entry bias block of logit (query q, key k).
 int SmolgenBiasIndex(int q, int k);
 
+// Smolgen generator layer and attention in one kernel (smolgen_attention.hip): the logits
+//   sum_j W[q*64+k][j] * gen[b][h][j]   (W: the shared smolgen_w layer [4096][gen_sz], gen: [B][heads][gen_sz])
+// are computed per workgroup and added to scale * Q.K^T without passing through memory. wfrag is W converted to
+// halves and reordered with SmolgenFragmentIndex (element (row, col) of W at that position). Head depth 32, at most
+// 32 heads, gen_sz 32, 128 or 256 (SmolgenAttentionSupported); qkv and out as for LaunchAttention.
+bool SmolgenAttentionSupported(int heads, int depth, int gen_sz);
+long long SmolgenFragmentIndex(int row, int col, int gen_sz);
+void LaunchSmolgenAttention(const half_t* qkv, const half_t* gen, const half_t* wfrag, half_t* out, int batch,
+                            int heads, int depth, int gen_sz, float scale, hipStream_t stream);
+void LaunchSmolgenAttentionF8Out(const half_t* qkv, const half_t* gen, const half_t* wfrag, uint8_t* out,
+                                 float out_mul, int batch, int heads, int depth, int gen_sz, float scale,
+                                 hipStream_t stream);
+
 // Attention policy tail: promotion offsets + gather to 1858 moves.
 // logits: [B][64*64] float (already scaled), kq: [B*64][ld_kq] with keys at column
 // offset key_off, ppo: [4][pd] float, inv_map: [1858] source index into the

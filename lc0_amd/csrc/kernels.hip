@@ -375,18 +375,6 @@ __device__ __forceinline__ void DmaToLds16(const void* gptr, void* lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory", "m0");
 }
 
-// 4 floats -> 4 e4m3 bytes (round to nearest even, saturating at +-448; the
-// hardware conversion alone would turn |v| > 464 into NaN).
-__device__ __forceinline__ unsigned PackFp8x4(float a, float b, float c, float d) {
-  a = __builtin_amdgcn_fmed3f(a, -448.0f, 448.0f);  // median of three = clamp, one instruction
-  b = __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f);
-  c = __builtin_amdgcn_fmed3f(c, -448.0f, 448.0f);
-  d = __builtin_amdgcn_fmed3f(d, -448.0f, 448.0f);
-  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
-  v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
-  return (unsigned)v;
-}
-
 // The same kernel serves fp16 operands (Args = GemmArgs: BKB = 128 bytes = 64
 // halves per tile row, v_mfma_f32_32x32x16_f16) and e4m3 operands (Args =
 // GemmF8Args: 128 bytes = 128 values per row, v_mfma_f32_32x32x64_f8f6f4);
@@ -505,7 +493,7 @@ void gemm_dma_kernel(Args p) {
           const int line = q * NWAVES * 64 + tid;
           const int row = line / LINES_PER_ROW, seg = line % LINES_PER_ROW;
           const half_t* src = p.skip + (long long)min(m0 + row, M - 1) * p.ldskip + min(n0 + seg * 64, N - 2);
-          if (line < LINES) asm volatile("global_load_dword %0, %1, off" : "=v"(touch[q]) : "v"(src) : "memory");
+          if (line < LINES) touch[q] = *reinterpret_cast<const volatile int*>(src);
         }
       }
     }
@@ -554,7 +542,7 @@ void gemm_dma_kernel(Args p) {
   // Epilogue through LDS (the stage buffers are free after the barrier).
   __syncthreads();
   if constexpr (EPI == 2) {
-    // (the registers of the early touches stay reserved up to here: every wait of the loop has covered them)
+    // (the early touches are consumed here: every wait of the loop has covered them)
 #pragma unroll
     for (int q = 0; q < (int)(sizeof(touch) / sizeof(touch[0])); q++) asm volatile("" ::"v"(touch[q]));
   }

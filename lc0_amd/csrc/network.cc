@@ -281,6 +281,9 @@ struct ModelState {
   int pol_emb_ = 0, pol_d_ = 0, val_ch_ = 0, val_fc_ = 0, val_out_ = 0, mov_ch_ = 0, mov_fc_ = 0;
   float alpha_ = 1.0f, eps_ = 1e-6f;
   bool fold_layer_norm_ = false;
+  bool fused_smolgen_attention_ = true;
+  int fused_smolgen_min_batch_ = 96;
+  half_t* smolgen_wfrag_ = nullptr;   // smolgen_w in the fragment order of smolgen_attention_kernel (null: not fused)
   bool any_smolgen_ = false;
   // Dense position encoding (PE_DENSE nets): preprocessing layer, embedding layer norm and
   // embedding FFN; optional input gating.
@@ -865,6 +868,11 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
     }
   }
   fold_layer_norm_ = options.GetBool("fold_layer_norm", false);
+  // The generator layer of smolgen inside the attention kernel: ahead from 128 positions up (one workgroup serves two
+  // samples and a quarter of the queries, and its two phases do not overlap: at fewer positions than fill the CUs the
+  // separate GEMM and attention kernels are faster; 15x1024 net: batch 128 +4 %, 256 +1.5 %, 1024 +2 %, 64 -1 %, 16 -6 %).
+  fused_smolgen_attention_ = options.GetBool("fused_smolgen_attention", true);
+  fused_smolgen_min_batch_ = options.GetInt("fused_smolgen_min_batch", 96);
   fp8_fp16_layers_ = options.GetInt("fp8_fp16_layers", 0);
   if (fp8_fp16_layers_ < 0) throw Error("fp8_fp16_layers must not be negative.");
   use_graphs_ = options.GetBool("graphs", true);
@@ -1277,6 +1285,14 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
         std::memcpy(&perm[static_cast<size_t>(SmolgenBiasIndex(q, k)) * g], &w.smolgen_w[static_cast<size_t>(q * 64 + k) * g],
                     sizeof(float) * g);
     smolgen_w_ = MakeLinear(perm, Vec(), 4096, g);
+    if (fused_smolgen_attention_ && SmolgenAttentionSupported(heads_, depth_, g)) {
+      // The same weights in the fragment order of the kernel that generates the logits inside the attention.
+      std::vector<half_t> frag(w.smolgen_w.size());
+      for (int row = 0; row < 4096; row++)
+        for (int col = 0; col < g; col++)
+          frag[SmolgenFragmentIndex(row, col, g)] = (half_t)w.smolgen_w[static_cast<size_t>(row) * g + col];
+      smolgen_wfrag_ = arena_.Upload(frag);
+    }
   }
 
   // Heads.
@@ -1615,6 +1631,8 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     // The smolgen chain depends only on x: it runs on the side stream next to the
     // QKV projection (on the main stream when profiling, for clean per-kernel times).
     hipStream_t ss = (profiling_ || single_stream_ || B < overlap_min_batch_) ? stream_ : side_stream_;
+    // The generator layer (smolgen_w) runs inside the attention kernel where that kernel serves the shape.
+    const bool fused_gen = e.has_smolgen && smolgen_wfrag_ != nullptr && B >= fused_smolgen_min_batch_;
     if (e.has_smolgen) {
       const int g = sg_gen_ / heads_;
       if (ss != stream_) {
@@ -1640,7 +1658,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
         LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f, 1e-3f,
                             ss);
       }, ss);
-      Gemm("gemm_smolgen_global", sg3_, g, smolgen_w_, sbias_, 4096, B * heads_, kActNone, false, ss);
+      if (!fused_gen) Gemm("gemm_smolgen_global", sg3_, g, smolgen_w_, sbias_, 4096, B * heads_, kActNone, false, ss);
       if (ss != stream_) HIP_CHECK(hipEventRecord(join_events_[li], ss));
       bias = sbias_;
     }
@@ -1651,18 +1669,32 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
            norm_in ? &cons_in : nullptr);
     }
     if (e.has_smolgen && ss != stream_) HIP_CHECK(hipStreamWaitEvent(stream_, join_events_[li], 0));
-    const double att_flops = 4.0 * 64 * 64 * depth_ * B * heads_;
+    const int gen_sz = e.has_smolgen ? sg_gen_ / heads_ : 0;
+    const double att_flops = 4.0 * 64 * 64 * depth_ * B * heads_ + (fused_gen ? 2.0 * 4096 * gen_sz * B * heads_ : 0.0);
     const bool att_f8 = f8 && q_dense_;
     const double att_bytes =
-        B * heads_ * (2.0 * 3 * 64 * depth_ + (att_f8 ? 1.0 : 2.0) * 64 * depth_ + (bias ? 2.0 * 4096 : 0.0));
+        B * heads_ * (2.0 * 3 * 64 * depth_ + (att_f8 ? 1.0 : 2.0) * 64 * depth_ +
+                      (fused_gen ? 2.0 * gen_sz : bias ? 2.0 * 4096 : 0.0));
     const float att_scale = 1.0f / std::sqrt(static_cast<float>(depth_));
-    if (att_f8) {
+    if (att_f8 && fused_gen) {
+      Timed("smolgen_attention", att_flops, att_bytes, [&] {
+        LaunchSmolgenAttentionF8Out(qkv_, sg3_, smolgen_wfrag_, attq_, 1.0f / e.s_att, B, heads_, depth_, gen_sz,
+                                    att_scale, stream_);
+      });
+      GemmF8("gemm_mha_dense", attq_, e.dense, e.dense8, t_, T, kActNone, false, 1.0f);
+    } else if (att_f8) {
       Timed("attention", att_flops, att_bytes,
             [&] { LaunchAttentionF8Out(qkv_, bias, attq_, 1.0f / e.s_att, B, heads_, att_scale, stream_, depth_); });
       GemmF8("gemm_mha_dense", attq_, e.dense, e.dense8, t_, T, kActNone, false, 1.0f);
     } else {
-      Timed("attention", att_flops, att_bytes,
-            [&] { LaunchAttention(qkv_, bias, att_, B, heads_, att_scale, stream_, depth_); });
+      if (fused_gen) {
+        Timed("smolgen_attention", att_flops, att_bytes, [&] {
+          LaunchSmolgenAttention(qkv_, sg3_, smolgen_wfrag_, att_, B, heads_, depth_, gen_sz, att_scale, stream_);
+        });
+      } else {
+        Timed("attention", att_flops, att_bytes,
+              [&] { LaunchAttention(qkv_, bias, att_, B, heads_, att_scale, stream_, depth_); });
+      }
       if (calibrating_) RecordAbsMax(att_, static_cast<size_t>(T) * d_model_, static_cast<int>(4 * li + 1));
       if (fold) {
         // x_ <- alpha * (att . dense + b) + LN2_prev(x_), with the row sums of the new x_

@@ -34,6 +34,7 @@ def _lib():
         lib.lc0mi_k_quantize_f8.argtypes = [vp, ll, cf, vp]
         lib.lc0mi_k_layer_norm_f8.argtypes = [vp, vp, vp, vp, ci, ci, cf, cf, cf, vp, vp]
         lib.lc0mi_k_attention_f8.argtypes = [vp, vp, ci, ci, cf, cf, vp]
+        lib.lc0mi_k_smolgen_attention.argtypes = [vp, vp, vp, ci, ci, ci, cf, ci, cf, vp, ci, cd]
         lib.lc0mi_k_legal_softmax.argtypes = [vp, vp, vp, cf, ci, vp]
         lib._k_ready = True
     return lib
@@ -218,6 +219,16 @@ def attention_f8(qkv, bias, batch, heads, scale, out_mul):
     _check(_lib().lc0mi_k_attention_f8(_ptr(qkv), _ptr(b), batch, heads, C.c_float(scale), C.c_float(out_mul),
                                        _ptr(out)))
     return out
+
+
+def smolgen_attention(qkv, gen, w, batch, heads, scale, f8_out=False, out_mul=1.0, time_iters=0):
+    """qkv [B*64, 3*heads*32], gen [B, heads, gen_sz], w [4096, gen_sz] -> [B*64, heads*32] (halves, or e4m3 bytes)."""
+    qkv, gen, w = _h(qkv), _h(gen), _h(w)
+    out = np.zeros((batch * 64, heads * 32), np.uint8 if f8_out else np.float16)
+    ms = C.c_double(0)
+    _check(_lib().lc0mi_k_smolgen_attention(_ptr(qkv), _ptr(gen), _ptr(w), batch, heads, w.shape[1], scale,
+                                            int(f8_out), out_mul, _ptr(out), time_iters, C.byref(ms)))
+    return (out, ms.value) if time_iters else out
 
 
 def expand_planes_attn(masks, values, ld=176, time_iters=0):

@@ -5,6 +5,7 @@ counters to it. Meant to be launched under the profiler:
   rocprofv3 --pmc WRITE_SIZE -- python3 -m lc0_amd.profile_kernels gemm --m 16384 --n 3072 --k 1024
   rocprofv3 --kernel-trace --stats -- python3 -m lc0_amd.profile_kernels gemm_f8 --m 16384 --n 3072 --k 1024
   rocprofv3 --kernel-trace --stats -- python3 -m lc0_amd.profile_kernels attention --batch 256 --heads 32
+  rocprofv3 --kernel-trace --stats -- python3 -m lc0_amd.profile_kernels smolgen_attention --batch 256 --heads 32
 
 `copy` moves a known number of bytes (reads N, writes N) and calibrates the HBM byte counters.
 """
@@ -19,7 +20,7 @@ from .backend import load_library
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("kernel", choices=["copy", "gemm", "gemm_f8", "attention", "layer_norm", "expand"])
+    ap.add_argument("kernel", choices=["copy", "gemm", "gemm_f8", "attention", "smolgen_attention", "layer_norm", "expand"])
     ap.add_argument("--mib", type=int, default=256)
     ap.add_argument("--m", type=int, default=16384)
     ap.add_argument("--n", type=int, default=3072)
@@ -71,6 +72,16 @@ def main():
         nbytes = args.batch * args.heads * (4 * 64 * 32 * 2 + 8192)
         print("attention B=%d H=%d: %.1f us, %.0f GB/s algorithmic" % (args.batch, args.heads, ms * 1e3,
                                                                       nbytes / (ms * 1e-3) / 1e9))
+    elif args.kernel == "smolgen_attention":
+        d = args.heads * 32
+        qkv = rng.standard_normal((args.batch * 64, 3 * d), dtype=np.float32).astype(np.float16)
+        gen = rng.standard_normal((args.batch, args.heads, 256), dtype=np.float32).astype(np.float16)
+        w = (rng.standard_normal((4096, 256), dtype=np.float32) * 0.1).astype(np.float16)
+        _, ms = K.smolgen_attention(qkv, gen, w, args.batch, args.heads, 32 ** -0.5, time_iters=args.iters)
+        nbytes = args.batch * args.heads * (4 * 64 * 32 * 2 + 512)
+        print("smolgen_attention B=%d H=%d: %.1f us, %.0f GB/s algorithmic, %.0f TFLOP/s" % (
+            args.batch, args.heads, ms * 1e3, nbytes / (ms * 1e-3) / 1e9,
+            args.batch * args.heads * (2.0 * 4096 * 256 + 4.0 * 64 * 64 * 32) / (ms * 1e-3) / 1e12))
     elif args.kernel == "layer_norm":
         x = rng.standard_normal((args.m, args.k), dtype=np.float32).astype(np.float16)
         _, ms = K.layer_norm(x, x, np.ones(args.k, np.float32), np.zeros(args.k, np.float32), 0.5, 1e-6,

@@ -322,6 +322,50 @@ def test_attention_f8_output_matches_half_output():
     _f8_close(got, half_out, 100.0)   # same fp32 result, rounded to e4m3 instead of fp16 (fp16 error << e4m3 step)
 
 
+def _smolgen_attention_reference(qkv, gen, w, batch, heads, scale):
+    """float32 numpy: the generator layer (logits as halves, as the separate GEMM stores them), then the attention."""
+    d = heads * 32
+    logits = (gen.astype(f32).reshape(batch * heads, -1) @ w.astype(f32).T).astype(np.float16).astype(f32)
+    logits = logits.reshape(batch, heads, 64, 64)
+    q = qkv[:, :d].astype(f32).reshape(batch, 64, heads, 32).transpose(0, 2, 1, 3)
+    k = qkv[:, d:2 * d].astype(f32).reshape(batch, 64, heads, 32).transpose(0, 2, 1, 3)
+    v = qkv[:, 2 * d:].astype(f32).reshape(batch, 64, heads, 32).transpose(0, 2, 1, 3)
+    p = onn.softmax_rows(np.matmul(q, k.transpose(0, 1, 3, 2)) * f32(scale) + logits)
+    return np.matmul(p, v).transpose(0, 2, 1, 3).reshape(batch * 64, d), logits
+
+
+@pytest.mark.parametrize("batch,heads,gen_sz", [(1, 2, 32), (2, 4, 32), (5, 8, 128), (4, 32, 256), (7, 32, 256),
+                                                (19, 24, 256)])
+def test_smolgen_attention_vs_oracle(batch, heads, gen_sz):
+    """The generator layer inside the attention kernel (network_blas.cc:332-347 + :352-439): odd batches (a sample
+    pair with one sample), fewer than 32 heads (unused matrix columns) and every generator width; also against the
+    two separate kernels, whose logits make the same round trip through halves."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(batch * 1000 + heads * 10 + gen_sz)
+    d = heads * 32
+    qkv = _h(rng.standard_normal((batch * 64, 3 * d)))
+    gen = _h(rng.standard_normal((batch, heads, gen_sz)))
+    w = _h(rng.standard_normal((4096, gen_sz)) * (2.0 / np.sqrt(gen_sz)))
+    scale = 1.0 / np.sqrt(32.0)
+    want, logits = _smolgen_attention_reference(qkv, gen, w, batch, heads, scale)
+    got = K.smolgen_attention(qkv, gen, w, batch, heads, scale).astype(f32)
+    np.testing.assert_allclose(got, want, rtol=4e-3, atol=4e-3)   # probabilities and output are rounded to fp16
+    separate = K.attention(qkv, _h(logits), batch, heads, scale).astype(f32)
+    np.testing.assert_allclose(got, separate, rtol=0, atol=4e-3)
+
+
+def test_smolgen_attention_f8_output():
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(79)
+    batch, heads, gen_sz = 3, 4, 32
+    qkv = _h(rng.standard_normal((batch * 64, 3 * heads * 32)))
+    gen = _h(rng.standard_normal((batch, heads, gen_sz)))
+    w = _h(rng.standard_normal((4096, gen_sz)) * 0.3)
+    half_out = K.smolgen_attention(qkv, gen, w, batch, heads, 32 ** -0.5).astype(f32)
+    got = K.smolgen_attention(qkv, gen, w, batch, heads, 32 ** -0.5, f8_out=True, out_mul=100.0)
+    _f8_close(got, half_out, 100.0)
+
+
 @pytest.mark.parametrize("depth", [64, 128])
 def test_attention_head_depths(depth):
     from lc0_amd import kernels as K

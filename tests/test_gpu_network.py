@@ -82,6 +82,37 @@ def test_attention_nets_match_oracle(name, batch, positions):
     np.testing.assert_allclose(comp.GetDVal(0) + 0 * comp.GetMVal(0), res["d"][3], atol=2e-3)
 
 
+@pytest.mark.parametrize("name,batch,options", [("tiny_attn", 37, ""), ("c2_bt4_15x1024", 33, ""),
+                                                ("tiny_attn_f8", 21, "precision=fp8,")])
+def test_smolgen_generator_inside_attention_and_as_a_gemm_of_its_own(name, batch, options, positions):
+    """The shared smolgen_w layer (network_blas.cc:332-347) runs inside the attention kernel (by default from 96
+    positions up, here forced) and as a separate GEMM with fused_smolgen_attention=false: both against the oracle,
+    and the profile names which ran."""
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    results = {}
+    for fused in (True, False):
+        net, res = _run_gpu(path, masks, values,
+                            options + "fused_smolgen_min_batch=1,fused_smolgen_attention=%s" % str(fused).lower())
+        if "fp8" in options:
+            st = _fp8_report(res, want, positions["legal"][:batch])
+            assert st["logit_rms"] <= 0.08 * st["logit_std"] and st["kl_max"] <= 5e-4
+        else:
+            _compare(res, want, positions["legal"][:batch])
+        net.SetProfiling(True)
+        comp = net.NewComputation()
+        comp.AddInputs(masks, values)
+        comp.ComputeBlocking()
+        names = [k.name for k in net.TakeProfile()]
+        net.SetProfiling(False)
+        assert ("smolgen_attention" in names) == fused and ("attention" in names) != fused, names
+        assert any(n.startswith("gemm_smolgen_global") for n in names) != fused, names
+        results[fused] = res
+    np.testing.assert_allclose(results[True]["policy"], results[False]["policy"], rtol=0,
+                               atol=5e-2 if "fp8" in options else 5e-3)
+
+
 @pytest.mark.parametrize("name,batch", [("c1_attn_10x256", 64), ("c2_bt4_15x1024", 32)])
 def test_layer_norms_folded_into_the_gemms_match_oracle(name, batch, positions):
     """Option fold_layer_norm=true: LayerNorm2DWithSkipConnection (src/neural/backends/blas/encoder.h:29-66) runs
