@@ -283,6 +283,7 @@ struct ModelState {
   bool fold_layer_norm_ = false;
   bool fused_smolgen_attention_ = true;
   int fused_smolgen_min_batch_ = 96;
+  bool qkv_first_ = true;
   half_t* smolgen_wfrag_ = nullptr;   // smolgen_w in the fragment order of smolgen_attention_kernel (null: not fused)
   bool any_smolgen_ = false;
   // Dense position encoding (PE_DENSE nets): preprocessing layer, embedding layer norm and
@@ -873,6 +874,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   // separate GEMM and attention kernels are faster; 15x1024 net: batch 128 +4 %, 256 +1.5 %, 1024 +2 %, 64 -1 %, 16 -6 %).
   fused_smolgen_attention_ = options.GetBool("fused_smolgen_attention", true);
   fused_smolgen_min_batch_ = options.GetInt("fused_smolgen_min_batch", 96);
+  qkv_first_ = options.GetBool("qkv_first", true);
   fp8_fp16_layers_ = options.GetInt("fp8_fp16_layers", 0);
   if (fp8_fp16_layers_ < 0) throw Error("fp8_fp16_layers must not be negative.");
   use_graphs_ = options.GetBool("graphs", true);
@@ -1633,10 +1635,23 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     hipStream_t ss = (profiling_ || single_stream_ || B < overlap_min_batch_) ? stream_ : side_stream_;
     // The generator layer (smolgen_w) runs inside the attention kernel where that kernel serves the shape.
     const bool fused_gen = e.has_smolgen && smolgen_wfrag_ != nullptr && B >= fused_smolgen_min_batch_;
+    auto launch_qkv = [&] {
+      if (f8 && q_qkv_) {
+        GemmF8("gemm_qkv", xq_, e.qkv, e.qkv8, qkv_, T, kActNone, false, 1.0f);
+      } else {
+        Gemm("gemm_qkv", x_, emb_, norm_in ? e.qkv_n : e.qkv, qkv_, 3 * d_model_, T, kActNone, false, nullptr, 1, false,
+             norm_in ? &cons_in : nullptr);
+      }
+    };
+    // With two streams the projection is recorded before the chain: a replayed graph then keeps it on the hardware
+    // queue of the layer norm before it and of the attention after it, and only the chain, which has slack, pays the
+    // dependencies between queues.
+    const bool qkv_before_chain = e.has_smolgen && ss != stream_ && qkv_first_;
     if (e.has_smolgen) {
       const int g = sg_gen_ / heads_;
       if (ss != stream_) {
         HIP_CHECK(hipEventRecord(fork_events_[li], stream_));
+        if (qkv_before_chain) launch_qkv();
         HIP_CHECK(hipStreamWaitEvent(ss, fork_events_[li], 0));
       }
       // The chain is the critical path of this phase when the QKV projection beside it is short (e4m3 operands,
@@ -1662,12 +1677,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       if (ss != stream_) HIP_CHECK(hipEventRecord(join_events_[li], ss));
       bias = sbias_;
     }
-    if (f8 && q_qkv_) {
-      GemmF8("gemm_qkv", xq_, e.qkv, e.qkv8, qkv_, T, kActNone, false, 1.0f);
-    } else {
-      Gemm("gemm_qkv", x_, emb_, norm_in ? e.qkv_n : e.qkv, qkv_, 3 * d_model_, T, kActNone, false, nullptr, 1, false,
-           norm_in ? &cons_in : nullptr);
-    }
+    if (!qkv_before_chain) launch_qkv();
     if (e.has_smolgen && ss != stream_) HIP_CHECK(hipStreamWaitEvent(stream_, join_events_[li], 0));
     const int gen_sz = e.has_smolgen ? sg_gen_ / heads_ : 0;
     const double att_flops = 4.0 * 64 * 64 * depth_ * B * heads_ + (fused_gen ? 2.0 * 4096 * gen_sz * B * heads_ : 0.0);
