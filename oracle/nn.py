@@ -20,15 +20,20 @@ Follows (reference file:line):
   legal-move softmax of the caller      src/neural/wrapper.cc:135-156, src/utils/fastmath.h:59-86
   check-backend comparison              src/neural/backends/network_check.cc:121-186
 
-Pins (tests/test_oracle_nn.py): activations, softmax, LayerNorm and the
-winograd filter transform against the compiled reference translation units
-(oracle/_ref) and against torch/scipy library routines; winograd convolution
-against direct zero-padded 3x3 correlation; the policy tables against SHA-256
-of the reference's tables and against oracle/_ref; one encoder layer against
-torch's scaled_dot_product_attention + layer_norm; whole-net invariants.
-The whole-net float results themselves have no reference-held vectors
-(the reference ships none): whole-net parity is pinned only through the
-per-function pins above.
+Pins: activations, softmax, LayerNorm and the winograd filter transform against
+the compiled reference translation units (oracle/_ref) and against torch/scipy
+library routines; winograd convolution against direct zero-padded 3x3
+correlation; the policy tables against SHA-256 of the reference's tables and
+against oracle/_ref; one encoder layer against torch's
+scaled_dot_product_attention + layer_norm; promotion offsets and the SE
+gamma/beta split by closed-form special cases (tests/test_oracle_nn.py).
+The whole-net wiring (flatten orders of the heads, policy Q.K^T, PE_DENSE
+preprocessing, gating layout, smolgen flatten, residual-tower order, SE split)
+is pinned against an independent float64 model written from the reference's
+C++ (tests/blas_model_f64.py, tests/test_oracle_wholenet.py), which also shows
+that each of these layout decisions, perturbed, fails the comparison.
+The reference ships no whole-net output vectors and its backend cannot be
+built here, so no reference-produced number enters these checks.
 """
 import numpy as np
 
