@@ -12,11 +12,11 @@
 //     operand and stay in registers. A lane ends up with the logits of one (sample, head) column: they go to LDS as
 //     halves in the layout phase 2 reads (128 KiB for the workgroup, XOR-swizzled so that both sides are free of
 //     bank conflicts).
-//   Phase 2 (memory and vector ALU): every wave takes 8 of the 64 (sample, head) columns, two at a time: S^T = K.Q^T for
-//     the 16 queries of both heads (the 32-wide MFMA tile carries head A's queries in its lower and head B's in its
-//     upper half), adds the logits from LDS, softmax over keys in registers plus one exchange with lane^32, then
-//     O^T = V^T.P^T with V transposed on the matrix cores (no LDS staging) and 8-byte output stores straight from the
-//     accumulators. K, Q and V of the next two heads are fetched while these are computed.
+//   Phase 2 (memory and vector ALU): every wave takes 8 of the 64 (sample, head) columns. With 16-wide MFMA tiles the 16
+//     queries are one tile: S^T = K.Q^T, plus the logits from LDS, softmax in registers with two lane exchanges,
+//     O^T = V^T.P^T with V transposed on the matrix cores (no LDS gather) and 8-byte output stores straight from the
+//     accumulators. K and V come in by full 128-byte rows of two neighbouring heads; the next pair's are in flight
+//     while this one is computed.
 // Per workgroup 0.5 MiB of weights, 0.5 MiB of K and V and 64 KiB of Q come from L2; nothing but the output is written.
 #include <hip/hip_runtime.h>
 
@@ -30,19 +30,20 @@ namespace lc0mi {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
 constexpr int kQueriesPerGroup = 16;               // queries of one workgroup
-constexpr int kLogitBytes = 2 * 2 * 16 * 2 * 64 * 16;   // [key half][8-key half][query][lane half][column slot] x 16 B
+constexpr int kLogitBytes = 64 * 16 * 4 * 32;   // [column][query][key group of the lane][16-key tile] x 8 B
 constexpr int kVBytesPerWave = 64 * 32 * 2;
 
-// Byte offset of the 16-byte slot that holds eight logits (keys 32*mt + 8*(e/4) + 4*g + e%4 for e = 8*hf .. 8*hf+7)
-// of query qq (0..15) in column c (0..63). Columns of one (mt, hf, qq, g) row are contiguous and rotated by qq, so that
-// the 32 lanes that write one row (neighbouring columns) and the 16 x 2 lanes that read one column (all queries) each
-// touch every bank group once.
-__device__ __forceinline__ int LogitSlot(int c, int qq, int g, int mt, int hf) {
-  return (((((mt * 2 + hf) * 16 + qq) * 2 + g) * 64) + (c ^ qq)) * 16;
+// Byte offset of the four logits of query qq (0..15) and column c (0..63) for keys 16*t + 4*g4 + (0..3). The 32 bytes
+// of one (c, qq, g4) are what a lane of phase 2 reads; the position of that block inside the column's 2 KiB is
+// XOR-ed with the low bits of c, which leaves the readers of one column (all qq, g4) on a contiguous 2 KiB and spreads
+// the 32 columns that phase 1 writes with one instruction over eight bank groups.
+__device__ __forceinline__ int LogitSlot(int c, int qq, int g4, int t) {
+  return (((c * 16 + (qq ^ ((c >> 2) & 1))) * 4 + (g4 ^ (c & 3))) * 32) + t * 8;
 }
 
 template <int NKS, typename OutT>
@@ -114,40 +115,41 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
       if (ks == NKS - 1) {
         const int rt = wave * 4 + f / NKS;   // row tile within the query group
         const int qq = rt >> 1, mt = rt & 1;
+        // register 4 q4 + e of lane (column r, g): key 32 mt + 8 q4 + 4 g + e = 4 u + e with u = 8 mt + 2 q4 + g
 #pragma unroll
         for (int ct = 0; ct < 2; ct++)
 #pragma unroll
-          for (int hf = 0; hf < 2; hf++) {
-            half8 hv;
+          for (int q4 = 0; q4 < 4; q4++) {
+            half4 hv;
 #pragma unroll
-            for (int e = 0; e < 8; e++) hv[e] = (half_t)acc[ct][hf * 8 + e];
-            *reinterpret_cast<half8*>(smem + LogitSlot(ct * 32 + r, qq, g, mt, hf)) = hv;
+            for (int e = 0; e < 4; e++) hv[e] = (half_t)acc[ct][q4 * 4 + e];
+            const int u = 8 * mt + 2 * q4 + g;
+            *reinterpret_cast<half4*>(smem + LogitSlot(ct * 32 + r, qq, u & 3, u >> 2)) = hv;
           }
       }
     }
   }
   __syncthreads();
 
-  // ---- phase 2: attention of the 16 queries, eight (sample, head) columns per wave, two at a time ----
-  // Lanes r < 16 of each half work on head A (an even column), lanes r >= 16 on head B (the next column), both for
-  // queries 0..15, so that the softmax arithmetic is spent on 32 distinct (head, query) pairs per half:
-  //   S^T:  one MFMA chain over the concatenated depth of both heads, [K_A | K_B] against query columns that carry
-  //         [q_A ; 0] in lanes r < 16 and [0 ; q_B] in lanes r >= 16;
-  //   V:    loaded by rows like K and transposed on the matrix cores (V_tile . I leaves, in the accumulator layout, a
-  //         lane per depth index holding keys, which is the operand layout of the product below);
-  //   O^T = V^T . P^T per head, so that a lane ends up with 16 depth values of its own query and stores them directly;
-  //         each lane keeps the product with its own head's V.
-  const int qq = r & 15;
-  const bool is_b = r >= 16;
-  // K and V of a head pair are fetched by 128-byte rows (both heads' 32 halves side by side), eight lanes per row, so
-  // that every load instruction touches eight full cache lines instead of 32 partial ones; a tile of 32 rows then
-  // passes through this wave's 4 KiB of LDS (16-byte chunk c of row w at chunk c ^ ((w >> 1) & 7): both directions
-  // free of bank conflicts) to reach the lanes in operand layout.
+  // ---- phase 2: attention of the 16 queries, eight (sample, head) columns per wave ----
+  // 16-wide MFMA tiles (v_mfma_f32_16x16x32_f16): the 16 queries are the columns of one tile, and lane (j, g4) = (query,
+  // group of four keys per 16-key tile) holds 16 of the 64 logits of its query, so that all 64 lanes carry distinct
+  // softmax elements:
+  //   S^T tiles (16 keys x 16 queries, the whole head depth in one MFMA), plus the logits of phase 1 from LDS;
+  //   softmax over the 16 values of a lane and the lanes 16, 32 and 48 away;
+  //   V transposed on the matrix cores (V_tile . I leaves a lane per depth index holding keys in the order of P);
+  //   O^T = V^T . P^T, so that a lane ends up with depth values of its own query, scales them by 1 / sum and stores.
+  // K and V are fetched for two neighbouring heads at once by 128-byte rows (both heads' 32 halves side by side), eight
+  // lanes per row, so that every load instruction touches eight full cache lines instead of 32 partial ones; a tile
+  // of 32 rows then passes through this wave's 4 KiB of LDS (16-byte chunk c of row w at chunk c ^ ((w >> 1) & 7):
+  // both directions free of bank conflicts) to reach the lanes in operand layout. The loads of the next pair of heads
+  // are in flight while this one is computed.
+  const int j = lane & 15, g4 = lane >> 4;
   const int lr = lane >> 3, ch = lane & 7;
   unsigned char* stg = smem + kLogitBytes + wave * kVBytesPerWave;
   struct PairData {
     half8 k[2][4], v[2][4];   // [32-row tile][8-row group]
-    half8 qf[2];              // this lane's head
+    half8 q[2];               // [head]: query j, depth 8 g4 .. 8 g4 + 7
   };
   auto load_pair = [&](int pi, PairData& d) {
     const int ca = wave * 8 + 2 * pi;
@@ -167,12 +169,11 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
         d.k[t][i] = *reinterpret_cast<const half8*>(Kp + off);
         d.v[t][i] = *reinterpret_cast<const half8*>(Vp + off);
       }
-    const half_t* Q = base + (is_b && has_b ? ha_c + 1 : ha_c) * DEPTH +
-                      (unsigned)(kQueriesPerGroup * qt + qq) * (unsigned)ld + 8u * g;
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) d.qf[ks] = *reinterpret_cast<const half8*>(Q + 16 * ks);
+    const half_t* Q = base + ha_c * DEPTH + (unsigned)(kQueriesPerGroup * qt + j) * (unsigned)ld + 8u * g4;
+    d.q[0] = *reinterpret_cast<const half8*>(Q);
+    d.q[1] = *reinterpret_cast<const half8*>(Q + (has_b ? DEPTH : 0));
   };
-  // fr[head][k-step]: rows of the tile in MFMA operand layout (lane r = row, g = 8-half group of the k-step)
+  // fr[head][16-row half]: rows of the staged tile in operand layout (lane j = row of the half, g4 = 8-half group)
   auto stage_tile = [&](const half8 (&raw)[4], half8 (&fr)[2][2]) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -182,18 +183,18 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
 #pragma unroll
     for (int hb = 0; hb < 2; hb++)
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-        const int c = hb * 4 + ks * 2 + g;
-        fr[hb][ks] = *reinterpret_cast<const half8*>(stg + r * 128 + ((c ^ ((r >> 1) & 7)) * 16));
+      for (int th = 0; th < 2; th++) {
+        const int row = 16 * th + j, c = hb * 4 + g4;
+        fr[hb][th] = *reinterpret_cast<const half8*>(stg + row * 128 + ((c ^ ((row >> 1) & 7)) * 16));
       }
   };
-  // Identity fragments: B operand of the transposing product, element (k, j) = [k == j].
+  // Identity fragments: B operand of the transposing product, element (k, column) = [k == 16 dt + column].
   half8 ident[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ks++)
+  for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-    for (int e = 0; e < 8; e++) ident[ks][e] = (16 * ks + 8 * g + e == r) ? (half_t)1.0f : (half_t)0.0f;
-  const half8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int e = 0; e < 8; e++) ident[dt][e] = (8 * g4 + e == 16 * dt + j) ? (half_t)1.0f : (half_t)0.0f;
+  const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
   PairData cur, nxt;
   load_pair(0, cur);
@@ -206,102 +207,85 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
     if (pi + 1 < 4) load_pair(pi + 1, nxt);
     if (live_a) {
       const int b = ca >= 32 ? b1 : b0;
-      // S^T[key][lane's (head, query)]
-      half8 qcat[4];
+      // S^T[key][query] of both heads: st[head][16-key tile], register e = key 16 t + 4 g4 + e
+      floatx4 st[2][4];
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-        qcat[ks] = is_b ? zero8 : cur.qf[ks];
-        qcat[2 + ks] = is_b ? cur.qf[ks] : zero8;
-      }
-      floatx16 st[2];
-#pragma unroll
-      for (int mt = 0; mt < 2; mt++) {
+      for (int tt = 0; tt < 2; tt++) {
         half8 kf[2][2];
-        stage_tile(cur.k[mt], kf);
+        stage_tile(cur.k[tt], kf);
 #pragma unroll
-        for (int e = 0; e < 16; e++) st[mt][e] = 0.0f;
+        for (int hb = 0; hb < 2; hb++)
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++)
-          st[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks >> 1][ks & 1], qcat[ks], st[mt], 0, 0, 0);
+          for (int th = 0; th < 2; th++)
+            st[hb][2 * tt + th] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[hb][th], cur.q[hb], zero4, 0, 0, 0);
       }
-      // V^T of both heads as halves in operand layout: vt[head][s] covers keys 16 s .. 16 s + 15
-      half8 vt[2][4];
+      // V^T of both heads as halves in operand layout: vt[head][depth half][32-key step], lane (depth index, g4),
+      // elements = keys 32 s + 4 g4 + (0..3) and 32 s + 16 + 4 g4 + (0..3), the order of the P operand below
+      half8 vt[2][2][2];
 #pragma unroll
-      for (int mt = 0; mt < 2; mt++) {
+      for (int tt = 0; tt < 2; tt++) {
         half8 vr[2][2];
-        stage_tile(cur.v[mt], vr);
+        stage_tile(cur.v[tt], vr);
 #pragma unroll
-        for (int hb = 0; hb < 2; hb++) {
-          floatx16 tr;
+        for (int hb = 0; hb < 2; hb++)
 #pragma unroll
-          for (int e = 0; e < 16; e++) tr[e] = 0.0f;
+          for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-          for (int ks = 0; ks < 2; ks++)
-            tr = __builtin_amdgcn_mfma_f32_32x32x16_f16(vr[hb][ks], ident[ks], tr, 0, 0, 0);
+            for (int th = 0; th < 2; th++) {
+              const floatx4 tr = __builtin_amdgcn_mfma_f32_16x16x32_f16(vr[hb][th], ident[dt], zero4, 0, 0, 0);
 #pragma unroll
-          for (int e = 0; e < 8; e++) {
-            vt[hb][2 * mt][e] = (half_t)tr[e];
-            vt[hb][2 * mt + 1][e] = (half_t)tr[8 + e];
-          }
-        }
+              for (int e = 0; e < 4; e++) vt[hb][dt][tt][4 * th + e] = (half_t)tr[e];
+            }
       }
-      // scale, add the logits, softmax over the 64 keys of this lane's (head, query): 32 here, 32 in lane^32
-      const int myc = ca + (is_b && live_b ? 1 : 0);
-      float mx = -3.0e38f;
 #pragma unroll
-      for (int mt = 0; mt < 2; mt++)
+      for (int hb = 0; hb < 2; hb++) {
+        if (hb == 1 && !live_b) break;
+        const int c = ca + hb;
+        // scale, add the logits, softmax over the 64 keys of this lane's query: 16 here, 48 in the lanes 16, 32, 48 away
+        const half8 lg0 = *reinterpret_cast<const half8*>(smem + LogitSlot(c, j, g4, 0));
+        const half8 lg1 = *reinterpret_cast<const half8*>(smem + LogitSlot(c, j, g4, 2));
+        float sv[16];
+        float mx = -3.0e38f;
 #pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-          const half8 bv = *reinterpret_cast<const half8*>(smem + LogitSlot(myc, qq, g, mt, hf));
+        for (int t = 0; t < 4; t++)
 #pragma unroll
-          for (int e = 0; e < 8; e++) {
-            const float sv = st[mt][hf * 8 + e] * scale + (float)bv[e];
-            st[mt][hf * 8 + e] = sv;
-            mx = fmaxf(mx, sv);
+          for (int e = 0; e < 4; e++) {
+            const float lgv = (float)(t < 2 ? lg0[4 * t + e] : lg1[4 * (t - 2) + e]);
+            sv[4 * t + e] = st[hb][t][e] * scale + lgv;
+            mx = fmaxf(mx, sv[4 * t + e]);
           }
-        }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      float sum = 0.0f;
-      const float kLog2e = 1.44269504f, neg_mx = -mx * kLog2e;
-#pragma unroll
-      for (int mt = 0; mt < 2; mt++)
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float sum = 0.0f;
+        const float kLog2e = 1.44269504f, neg_mx = -mx * kLog2e;
 #pragma unroll
         for (int e = 0; e < 16; e++) {
-          const float ev = __builtin_amdgcn_exp2f(__builtin_fmaf(st[mt][e], kLog2e, neg_mx));   // e^(s - mx)
-          st[mt][e] = ev;
-          sum += ev;
+          sv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[e], kLog2e, neg_mx));   // e^(s - mx) <= 1
+          sum += sv[e];
         }
-      sum += __shfl_xor(sum, 32, 64);
-      const float inv = 1.0f / sum;
-      half8 pf[4];
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        const float inv = __builtin_amdgcn_rcpf(sum);   // 1 ulp
+        half8 pf[2];
 #pragma unroll
-      for (int s4 = 0; s4 < 4; s4++)
+        for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) pf[s4][e] = (half_t)st[s4 / 2][8 * (s4 % 2) + e];   // e^(s - mx) <= 1
-      // O^T = V^T . P^T: lane (its head and query, g), register e = depth index 8*(e/4) + 4*g + e%4
-      floatx16 oa, ob;
+          for (int e = 0; e < 8; e++) pf[s2][e] = (half_t)sv[8 * s2 + e];
+        // O^T = V^T . P^T: lane (query j, g4), register e = depth index 16 dt + 4 g4 + e
+        OutT* O = out + (long long)(b * 64 + kQueriesPerGroup * qt + j) * d_model + (ha + hb) * DEPTH + 4 * g4;
 #pragma unroll
-      for (int e = 0; e < 16; e++) { oa[e] = 0.0f; ob[e] = 0.0f; }
+        for (int dt = 0; dt < 2; dt++) {
+          floatx4 o = zero4;
 #pragma unroll
-      for (int s4 = 0; s4 < 4; s4++) {
-        oa = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt[0][s4], pf[s4], oa, 0, 0, 0);
-        ob = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt[1][s4], pf[s4], ob, 0, 0, 0);
-      }
-      if (!is_b || live_b) {
-        OutT* O = out + (long long)(b * 64 + kQueriesPerGroup * qt + qq) * d_model + (ha + (is_b ? 1 : 0)) * DEPTH + 4 * g;
-#pragma unroll
-        for (int j4 = 0; j4 < 4; j4++) {
-          float v4[4];
-#pragma unroll
-          for (int e = 0; e < 4; e++) v4[e] = (is_b ? ob[4 * j4 + e] : oa[4 * j4 + e]) * inv;   // this lane's own query
+          for (int s2 = 0; s2 < 2; s2++) o = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt[hb][dt][s2], pf[s2], o, 0, 0, 0);
           if constexpr (sizeof(OutT) == 1) {
-            *reinterpret_cast<unsigned*>(O + 8 * j4) =
-                PackFp8x4(v4[0] * out_mul, v4[1] * out_mul, v4[2] * out_mul, v4[3] * out_mul);
+            const float m = inv * out_mul;
+            *reinterpret_cast<unsigned*>(O + 16 * dt) = PackFp8x4(o[0] * m, o[1] * m, o[2] * m, o[3] * m);
           } else {
             half4 h4;
 #pragma unroll
-            for (int e = 0; e < 4; e++) h4[e] = (half_t)v4[e];
-            *reinterpret_cast<half4*>(O + 8 * j4) = h4;
+            for (int e = 0; e < 4; e++) h4[e] = (half_t)(o[e] * inv);
+            *reinterpret_cast<half4*>(O + 16 * dt) = h4;
           }
         }
       }
