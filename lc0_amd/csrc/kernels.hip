@@ -413,13 +413,23 @@ void gemm_dma_kernel(Args p) {
   constexpr int EPI_TOTAL = EPI_BYTES + STAT_BYTES + PART_BYTES;
   constexpr int SMEM = (2 * STAGE > EPI_TOTAL) ? 2 * STAGE : EPI_TOTAL;
   static_assert(EPI == 0 || (!F8 && sizeof(OutT) == 2), "folded layer norm: fp16 operands and output");
-  __shared__ __attribute__((aligned(1024))) char smem[SMEM];
+  // The tile's bias (and per-column scale, fp8 operands) waits in LDS behind the stages: fetched with the first k-tile,
+  // so that the epilogue does not start with a round trip to memory.
+  constexpr int COLV_BYTES = (F8 ? 2 : 1) * BN * 4;
+  __shared__ __attribute__((aligned(1024))) char smem[SMEM + COLV_BYTES];
+  float* colv = reinterpret_cast<float*>(smem + SMEM);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
   const int M = p.M, N = p.N, K = p.K;
+  float my_bias = 0.0f;
+  [[maybe_unused]] float my_cscale = 0.0f;
+  if (tid < BN && n0 + tid < N) {
+    if (p.bias != nullptr) my_bias = p.bias[n0 + tid];
+    if constexpr (F8) my_cscale = p.col_scale[n0 + tid];
+  }
   const char* A = reinterpret_cast<const char*>(p.A);
   const char* W = reinterpret_cast<const char*>(p.W);
   if constexpr (!F8) {
@@ -462,6 +472,10 @@ void gemm_dma_kernel(Args p) {
 
   const int nk = K * ES / BKB;
   issue(smem, smem + BM * BKB, 0);
+  if (tid < BN) {
+    colv[tid] = my_bias;
+    if constexpr (F8) colv[BN + tid] = my_cscale;
+  }
   // Folded layer norm: (mean, rstd) of tile row `tid` (of the A operand for a consumer, of the residual for a
   // producer), fetched while the first k-tile is on its way and kept in two registers until the epilogue.
   [[maybe_unused]] float2 my_ms = make_float2(0.0f, 1.0f);
@@ -557,7 +571,11 @@ void gemm_dma_kernel(Args p) {
 #pragma unroll
   for (int j = 0; j < TN; j++)
 #pragma unroll
-    for (int blk = 0; blk < 4; blk++) LoadBias4(p.bias, n0 + wn * WN + j * 32 + blk * 8 + g * 4, N, bias_v[j][blk]);
+    for (int blk = 0; blk < 4; blk++) {
+      const floatx4 b4 = *reinterpret_cast<const floatx4*>(colv + wn * WN + j * 32 + blk * 8 + g * 4);
+#pragma unroll
+      for (int rr = 0; rr < 4; rr++) bias_v[j][blk][rr] = b4[rr];
+    }
   // Folded layer norm: statistics of this tile's rows (of the A operand for a consumer, of the residual for a
   // producer), one row per thread, shared through LDS.
   [[maybe_unused]] float2* row_ms = reinterpret_cast<float2*>(smem + EPI_BYTES);                 // [BM] (mean, rstd)
@@ -622,7 +640,9 @@ void gemm_dma_kernel(Args p) {
           if constexpr (F8) {
             // Per-column dequantisation factor (activation scale x weight-row scale).
             float cs[4];
-            LoadBias4(p.col_scale, n0 + wn * WN + j * 32 + blk * 8 + g * 4, N, cs);
+            const floatx4 c4 = *reinterpret_cast<const floatx4*>(colv + BN + wn * WN + j * 32 + blk * 8 + g * 4);
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) cs[rr] = c4[rr];
 #pragma unroll
             for (int rr = 0; rr < 4; rr++) v[rr] = act_fn(acc[i][j][blk * 4 + rr] * cs[rr] + bias_v[j][blk][rr]);
           } else if constexpr (EPI == 1) {
