@@ -228,6 +228,9 @@ def test_resnet_20x256_batch_512():
     assert np.isfinite(full["policy"]).all()
     np.testing.assert_allclose(onn.softmax_rows(full["policy"][:24]), onn.softmax_rows(res24["policy"]), rtol=0, atol=5e-3)
     np.testing.assert_allclose(full["q"][:24], res24["q"], rtol=0, atol=5e-3)
+    # the last rows of the full batch against the oracle as well (other tiles of every launch than the first rows)
+    want_tail = onn.BlasNetwork(nr.load(path)).forward(masks[-24:], values[-24:])
+    _compare({k: v[-24:] for k, v in full.items()}, want_tail, pos["legal"][-24:])
 
 
 def test_ragged_and_oversized_batches(positions):
@@ -441,7 +444,9 @@ def test_bt4_dense_multihead_batch_256(positions):
     np.testing.assert_allclose(full["policy"][:32], res32["policy"], rtol=0, atol=5e-3)
 
 
-@pytest.mark.parametrize("name,options", [("tiny_attn", ""), ("tiny_attn_f8", "precision=fp8"), ("tiny_resnet", "")])
+@pytest.mark.parametrize("name,options", [("tiny_attn", ""), ("tiny_attn_f8", "precision=fp8"), ("tiny_resnet", ""),
+                                          ("tiny_attn", "fused_smolgen_min_batch=1"),
+                                          ("tiny_attn", "fused_smolgen_min_batch=1,fold_layer_norm=true")])
 def test_graph_replays_equal_eager_launches(name, options, positions):
     """The device pass is recorded once per batch size and replayed; every replay, with other
     batch sizes and eager work of a second network in between, must give exactly what plain
@@ -462,7 +467,7 @@ def test_graph_replays_equal_eager_launches(name, options, positions):
             outs.append(comp.results())
         for key in ("policy", "q", "d", "m"):
             np.testing.assert_array_equal(outs[0][key], outs[1][key])
-    if options:   # re-calibration drops the recorded graphs: the next replay must use the new scales
+    if "fp8" in options:   # re-calibration drops the recorded graphs: the next replay must use the new scales
         for net in (replay, eager):
             net.CalibrateFp8(positions["masks"][100:164], positions["values"][100:164])
         outs = []
@@ -475,6 +480,7 @@ def test_graph_replays_equal_eager_launches(name, options, positions):
 
 
 @pytest.mark.parametrize("name,options", [("tiny_attn", "lanes=1"), ("tiny_attn", "lanes=3"), ("tiny_resnet", "lanes=2"),
+                                          ("tiny_attn", "lanes=3,fused_smolgen_min_batch=1"),
                                           ("tiny_attn_f8", "precision=fp8,lanes=2")])
 def test_concurrent_computations_from_several_threads(name, options, positions):
     """Search threads share one network (backendbench.cc:177-184 does the same): computations
