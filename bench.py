@@ -230,8 +230,9 @@ def main():
     net.SetProfiling(False)
     total_kernel_ms = sum(k.ms for k in prof) / prof_iters
     kernels = sorted(prof, key=lambda k: -k.ms)
-    gemm_ms = sum(k.ms for k in prof if k.name.startswith("gemm") or k.name == "attention") / prof_iters
-    gemm_flops = sum(k.flops for k in prof if k.name.startswith("gemm") or k.name == "attention") / prof_iters
+    matrix = [k for k in prof if k.name.startswith("gemm") or k.name in ("attention", "smolgen_attention")]
+    gemm_ms = sum(k.ms for k in matrix) / prof_iters
+    gemm_flops = sum(k.flops for k in matrix) / prof_iters
     # Group call sites by the kernel that ran them ("call_site|kernel_variant"): the
     # roofline is quoted for the kernel (as rocprofv3 sees it), not for one call site.
     from collections import namedtuple
