@@ -10,8 +10,8 @@
 //     stored at load in fragment order (each wave streams 1 KiB per load, fully coalesced, a ring of loads ahead of the
 //     MFMAs) and used for both column tiles; the generator vectors of the 64 (sample, head) columns are the "B"
 //     operand and stay in registers. A lane ends up with the logits of one (sample, head) column: they go to LDS as
-//     halves in the layout phase 2 reads (128 KiB for the workgroup, XOR-swizzled so that both sides are free of
-//     bank conflicts).
+//     halves in the layout phase 2 reads (128 KiB for the workgroup: 32 contiguous bytes per reading lane, the
+//     positions XOR-ed with the column so that the writers of one instruction spread over eight bank groups).
 //   Phase 2 (memory and vector ALU): every wave takes 8 of the 64 (sample, head) columns. With 16-wide MFMA tiles the 16
 //     queries are one tile: S^T = K.Q^T, plus the logits from LDS, softmax in registers with two lane exchanges,
 //     O^T = V^T.P^T with V transposed on the matrix cores (no LDS gather) and 8-byte output stores straight from the
@@ -36,7 +36,7 @@ namespace {
 
 constexpr int kQueriesPerGroup = 16;               // queries of one workgroup
 constexpr int kLogitBytes = 64 * 16 * 4 * 32;   // [column][query][key group of the lane][16-key tile] x 8 B
-constexpr int kVBytesPerWave = 64 * 32 * 2;
+constexpr int kVBytesPerWave = 64 * 32 * 2;   // staging area of one wave: a tile of 32 rows x 128 bytes
 
 // Byte offset of the four logits of query qq (0..15) and column c (0..63) for keys 16*t + 4*g4 + (0..3). The 32 bytes
 // of one (c, qq, g4) are what a lane of phase 2 reads; the position of that block inside the column's 2 KiB is
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
     half8 ring[PF];
 #pragma unroll
     for (int f = 0; f < PF; f++) ring[f] = wp[f * 64];
-    // The generator vectors of the 64 columns: once per workgroup through LDS (the region phase 2 uses for V), 16-byte
+    // The generator vectors of the 64 columns: once per workgroup through LDS (the region phase 2 stages K and V in), 16-byte
     // slot s of column c at slot s ^ (c & 31) of its row, then into the registers of every wave as MFMA "B" operands.
     unsigned char* gl = smem + kLogitBytes;
     constexpr int kSlotsPerCol = G / 8;
