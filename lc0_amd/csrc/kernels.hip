@@ -500,7 +500,7 @@ void gemm_dma_kernel(Args p) {
     if (kt + 1 < nk) issue(nxt, nxt + BM * BKB, (kt + 1) * BKB);
     if constexpr (EPI == 2) {
       if (kt == 1) {
-        constexpr int LINES_PER_ROW = BN * 2 / 128;
+        constexpr int LINES_PER_ROW = (BN * 2 + 127) / 128;
         constexpr int LINES = BM * LINES_PER_ROW;
 #pragma unroll
         for (int q = 0; q < (LINES + NWAVES * 64 - 1) / (NWAVES * 64); q++) {
@@ -830,7 +830,8 @@ void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
 }  // namespace
 
 namespace {
-enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128, kRowPanel, kDma128x64, kPersist256 };
+enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128, kRowPanel, kDma128x64, kPersist256,
+                   kDma128x32 };
 
 int g_variant_override = -1;
 
@@ -838,7 +839,7 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
   if (g_variant_override >= 0) {
     const bool dma_ok = !a.out_f32 && a.split_k == 1 && a.K % 64 == 0;
     const bool is_dma = g_variant_override <= kDma256x128 || g_variant_override == kDma128x128 ||
-                        g_variant_override == kDma128x64;
+                        g_variant_override == kDma128x64 || g_variant_override == kDma128x32;
     bool ok = is_dma ? dma_ok : (g_variant_override != kRowPanel || a.split_k == 1);
     if (g_variant_override == kPersist256) ok = GemmPersistentSupports(a);
     if (ok) return static_cast<GemmVariant>(g_variant_override);
@@ -880,6 +881,12 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
     }
     return best;
   }
+  // Very many rows, at most 32 columns (the smolgen compression at 512 positions and more): a memory-bound stream of
+  // the activation rows. 128x32 direct-to-LDS tiles (four workgroups per CU) read them once at full line width
+  // (65536x32x1024: 34 us against 96 for the row-panel kernel).
+  if (!a.out_f32 && a.split_k == 1 && a.batch == 1 && a.N <= 32 && a.K % 64 == 0 && a.K >= 128 && a.M >= 32768) {
+    return kDma128x32;
+  }
   // Small problems with a long reduction: the 64x64 kernel walks K serially in one workgroup;
   // when it would start at most 64 workgroups, the row-panel kernel (8-way K split inside the
   // workgroup, 64x32 panels) is faster (64x3072x1024: 8.5 vs 9.7 us; 8192x32x1024: 9.2 vs 11.9 us).
@@ -904,6 +911,7 @@ int DmaTileN(GemmVariant v) {
     case kDma256x192: return 192;
     case kDma256x128: case kDma128x128: return 128;
     case kDma128x64: return 64;
+    case kDma128x32: return 32;
     default: return 0;
   }
 }
@@ -935,6 +943,7 @@ const char* GemmVariantName(const GemmArgs& a) {
     case kDma256x128: return "gemm_dma_256x128x32";
     case kDma128x128: return "gemm_dma_128x128x64";
     case kDma128x64: return "gemm_dma_128x64x64";
+    case kDma128x32: return "gemm_dma_128x32x64";
     case kRowPanel: return "gemm_rowpanel_64x32";
     case kTile128: return "gemm_128x128x64";
     default: return a.split_k > 1 ? "gemm_64x64x64_splitk" : "gemm_64x64x64";
@@ -953,6 +962,7 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
     case kDma256x128: LaunchGemmDma<256, 128, 32, 4, 2>(a, stream); break;
     case kDma128x128: LaunchGemmDma<128, 128, 64, 2, 2>(a, stream); break;
     case kDma128x64: LaunchGemmDma<128, 64, 64, 2, 2>(a, stream); break;
+    case kDma128x32: LaunchGemmDma<128, 32, 64, 4, 1>(a, stream); break;
     case kRowPanel: {
       dim3 grid((a.M + 63) / 64, (a.N + 31) / 32, a.batch);
       if (a.out_f32) {
