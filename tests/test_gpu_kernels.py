@@ -335,11 +335,12 @@ def _smolgen_attention_reference(qkv, gen, w, batch, heads, scale):
 
 
 @pytest.mark.parametrize("batch,heads,gen_sz", [(1, 2, 32), (2, 4, 32), (5, 8, 128), (4, 32, 256), (7, 32, 256),
-                                                (19, 24, 256)])
+                                                (19, 24, 256), (3, 1, 32), (6, 3, 128), (9, 31, 256)])
 def test_smolgen_attention_vs_oracle(batch, heads, gen_sz):
     """The generator layer inside the attention kernel (network_blas.cc:332-347 + :352-439): odd batches (a sample
-    pair with one sample), fewer than 32 heads (unused matrix columns) and every generator width; also against the
-    two separate kernels, whose logits make the same round trip through halves."""
+    pair with one sample), fewer than 32 heads (unused matrix columns), odd head counts (a last head without a
+    neighbour in its 128-byte rows) and every generator width; also against the two separate kernels, whose logits
+    make the same round trip through halves."""
     from lc0_amd import kernels as K
     rng = np.random.default_rng(batch * 1000 + heads * 10 + gen_sz)
     d = heads * 32
