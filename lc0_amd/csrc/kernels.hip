@@ -260,85 +260,98 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 
 // ---------------------------------------------------------------------------
 // Row-panel GEMM for small problems (few rows, or few columns): a workgroup owns a
-// 64 x 32 output panel and its eight waves split the reduction dimension, so even
-// a 64 x 32 x K problem keeps eight waves busy, the serial chain is K / 128 MFMA
-// steps instead of K / 16, and up to eight steps of operand loads are in flight per
-// wave (these problems are bound by memory latency, not by arithmetic). Fragments go
-// from global memory straight into registers; the eight partial sums are added in
-// wave order through LDS, so results do not depend on timing.
+// (16 RT) x (16 CT) output panel and its eight waves split the reduction dimension, so
+// even a 16 x 16 x K problem keeps eight waves busy, the serial chain is K / 256 MFMA
+// steps instead of K / 32, and U steps of operand loads are in flight per wave (these
+// problems are bound by memory latency and by the 64 bytes per cycle at which a CU's
+// address path takes loads, not by arithmetic: the time of a launch grows with the
+// RT + CT operand rows a workgroup reads, so the launcher picks the smallest panel that
+// still fits the problem into one workgroup per CU). Fragments of 16x16x32 tiles go from
+// global memory straight into registers, 64 bytes of a row per load instruction; the
+// eight partial sums are added in wave order through LDS, so results do not depend on
+// timing.
 // ---------------------------------------------------------------------------
-template <typename OutT>
+template <int RT, int CT, int U, typename OutT>
 __global__ __launch_bounds__(512) void gemm_rowpanel_kernel(GemmArgs p) {
-  constexpr int NW = 8;
-  __shared__ float part[NW][64 * 33];
+  constexpr int NW = 8, ROWS = 16 * RT, COLS = 16 * CT, LD = COLS + 1;
+  __shared__ float part[NW][ROWS * LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 31, g = lane >> 5;
-  const int m0 = blockIdx.x * 64, n0 = blockIdx.y * 32;
+  const int r = lane & 15, g = lane >> 4;
+  const int m0 = blockIdx.x * ROWS, n0 = blockIdx.y * COLS;
   const int M = p.M, N = p.N, K = p.K;
   const half_t* A = p.A + (long long)blockIdx.z * p.strideA;
   const half_t* W = p.W + (long long)blockIdx.z * p.strideW;
-  // K range of this wave, in steps of 16.
-  const int steps = (K + 15) / 16;
+  // K range of this wave, in steps of 32. A last step of 8, 16 or 24 values goes to the last wave.
+  const int steps = K / 32;
   const int per_wave = (steps + NW - 1) / NW;
-  const int s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
-  const half_t* a0 = A + (long long)min(m0 + r, M - 1) * p.lda + 8 * g;
-  const half_t* a1 = A + (long long)min(m0 + 32 + r, M - 1) * p.lda + 8 * g;
-  const half_t* w0 = W + (long long)min(n0 + r, N - 1) * p.ldw + 8 * g;
-  floatx16 acc0, acc1;
+  const int s_begin = min(steps, wave * per_wave), s_end = min(steps, s_begin + per_wave);
+  const half_t* a_row[RT];
+  const half_t* w_row[CT];
 #pragma unroll
-  for (int e = 0; e < 16; e++) acc0[e] = acc1[e] = 0.0f;
-  // All steps but a possible half-step at the very end of K are loaded without a
-  // predicate, so that the compiler can put the loads of eight steps in flight at once.
-  const int full_end = (K % 16 == 0) ? s_end : min(s_end, steps - 1);
-  for (int st = s_begin; st < full_end; st += 8) {
-    half8 fa0[8], fa1[8], fw[8];
+  for (int t = 0; t < RT; t++) a_row[t] = A + (long long)min(m0 + 16 * t + r, M - 1) * p.lda + 8 * g;
 #pragma unroll
-    for (int u = 0; u < 8; u++) {   // steps past the end re-read the last one (never used)
-      const int k = min(st + u, full_end - 1) * 16;
-      fa0[u] = *reinterpret_cast<const half8*>(a0 + k);
-      fa1[u] = *reinterpret_cast<const half8*>(a1 + k);
-      fw[u] = *reinterpret_cast<const half8*>(w0 + k);
+  for (int c = 0; c < CT; c++) w_row[c] = W + (long long)min(n0 + 16 * c + r, N - 1) * p.ldw + 8 * g;
+  floatx4 acc[RT][CT];
+#pragma unroll
+  for (int t = 0; t < RT; t++)
+#pragma unroll
+    for (int c = 0; c < CT; c++) acc[t][c] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+  // Loads carry no predicate, so that the compiler can put the loads of U steps in flight at once.
+  for (int st = s_begin; st < s_end; st += U) {
+    half8 fa[RT][U], fw[CT][U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {   // steps past the end re-read the last one (never used)
+      const int k = min(st + u, s_end - 1) * 32;
+#pragma unroll
+      for (int t = 0; t < RT; t++) fa[t][u] = *reinterpret_cast<const half8*>(a_row[t] + k);
+#pragma unroll
+      for (int c = 0; c < CT; c++) fw[c][u] = *reinterpret_cast<const half8*>(w_row[c] + k);
     }
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-      if (st + u < full_end) {
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[u], fa0[u], acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[u], fa1[u], acc1, 0, 0, 0);
+    for (int u = 0; u < U; u++) {
+      if (st + u < s_end) {
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+          for (int c = 0; c < CT; c++)
+            acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[c][u], fa[t][u], acc[t][c], 0, 0, 0);
       }
     }
   }
-  if (s_end > full_end && s_end > s_begin) {   // K is a multiple of 8: the upper half of the last step is zero-filled
-    const int k = (steps - 1) * 16;
+  if (wave == NW - 1 && K % 32 != 0) {   // K is a multiple of 8: the missing part of the last step is zero-filled
+    const int k = steps * 32;
     const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    const bool in = g == 0;
-    const half8 fa0 = in ? *reinterpret_cast<const half8*>(a0 + k) : zero;
-    const half8 fa1 = in ? *reinterpret_cast<const half8*>(a1 + k) : zero;
-    const half8 fw = in ? *reinterpret_cast<const half8*>(w0 + k) : zero;
-    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw, fa0, acc0, 0, 0, 0);
-    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw, fa1, acc1, 0, 0, 0);
+    const bool in = k + 8 * g < K;
+    half8 fa[RT], fw[CT];
+#pragma unroll
+    for (int t = 0; t < RT; t++) fa[t] = in ? *reinterpret_cast<const half8*>(a_row[t] + k) : zero;
+#pragma unroll
+    for (int c = 0; c < CT; c++) fw[c] = in ? *reinterpret_cast<const half8*>(w_row[c] + k) : zero;
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+      for (int c = 0; c < CT; c++) acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[c], fa[t], acc[t][c], 0, 0, 0);
   }
-  // Accumulator lane (r, g) holds rows m = r (+32), columns n = 8 blk + 4 g + j.
+  // Accumulator lane (r, g) of tile (t, c) holds row m = 16 t + r, columns n = 16 c + 4 g + e.
   float* mine = part[wave];
 #pragma unroll
-  for (int blk = 0; blk < 4; blk++)
+  for (int t = 0; t < RT; t++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int n = 8 * blk + 4 * g + j;
-      mine[r * 33 + n] = acc0[blk * 4 + j];
-      mine[(32 + r) * 33 + n] = acc1[blk * 4 + j];
-    }
+    for (int c = 0; c < CT; c++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) mine[(16 * t + r) * LD + 16 * c + 4 * g + e] = acc[t][c][e];
   __syncthreads();
   OutT* C = reinterpret_cast<OutT*>(p.C) + (long long)blockIdx.z * p.strideC;
   DispatchAct(p.act, [&](auto act_fn) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int idx = tid + 512 * i;        // 64 x 32 outputs, consecutive threads along n
-      const int row = idx >> 5, col = idx & 31;
+    for (int i = 0; i < (ROWS * COLS + 511) / 512; i++) {
+      const int idx = tid + 512 * i;        // consecutive threads along n
+      const int row = idx / COLS, col = idx % COLS;
       const int m = m0 + row, n = n0 + col;
-      if (m < M && n < N) {
-        float sum = part[0][row * 33 + col];
+      if (row < ROWS && m < M && n < N) {
+        float sum = part[0][row * LD + col];
 #pragma unroll
-        for (int w = 1; w < NW; w++) sum += part[w][row * 33 + col];
+        for (int w = 1; w < NW; w++) sum += part[w][row * LD + col];
         sum *= p.scale;
         if (p.row_stats != nullptr) {   // consumer side of a folded layer norm
           float mean, rstd;
@@ -830,6 +843,67 @@ void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
 }  // namespace
 
 namespace {
+// The smallest panel (in operand rows a workgroup reads) with which the problem still fits into one workgroup per
+// CU; the largest one otherwise. 64x1024xK runs as 256 panels of 16x16 (64x1024x1536: 4.6 us against 14.3 with 64x32
+// panels), 64x3072xK as 192 panels of 32x32.
+struct RowPanelShape { int rt, ct; };
+constexpr RowPanelShape kRowPanelShapes[] = {{1, 1}, {2, 1}, {1, 2}, {2, 2}, {4, 2}};
+constexpr long long kRowPanelWorkgroups = 256;   // one per CU
+inline long long RowPanelWorkgroups(const GemmArgs& a, const RowPanelShape& c) {
+  return (long long)((a.M + 16 * c.rt - 1) / (16 * c.rt)) * ((a.N + 16 * c.ct - 1) / (16 * c.ct)) * a.batch;
+}
+inline RowPanelShape PickRowPanelShape(const GemmArgs& a) {
+  for (const RowPanelShape& c : kRowPanelShapes) {
+    if (RowPanelWorkgroups(a, c) <= kRowPanelWorkgroups) return c;
+  }
+  return kRowPanelShapes[4];
+}
+
+template <int RT, int CT, int U>
+void LaunchGemmRowPanelShape(const GemmArgs& a, hipStream_t stream) {
+  dim3 grid((a.M + 16 * RT - 1) / (16 * RT), (a.N + 16 * CT - 1) / (16 * CT), a.batch);
+  if (a.out_f32) {
+    hipLaunchKernelGGL((gemm_rowpanel_kernel<RT, CT, U, float>), grid, dim3(512), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((gemm_rowpanel_kernel<RT, CT, U, half_t>), grid, dim3(512), 0, stream, a);
+  }
+}
+
+template <int RT, int CT>
+void LaunchGemmRowPanelSteps(const GemmArgs& a, hipStream_t stream) {
+  // Steps of 32 per wave; U of them are loaded at once (registers: 4 (RT + CT) U), in as few rounds as possible
+  // with as few steps loaded in vain as possible.
+  constexpr int kMaxU = (RT + CT >= 6) ? 6 : 8;
+  const int per_wave = (a.K / 32 + 7) / 8;
+  int u = 2;
+  if (per_wave > 2) {
+    int best_waste = 1 << 30;
+    for (int cand = kMaxU; cand >= 4; cand -= 2) {
+      const int rounds = (per_wave + cand - 1) / cand;
+      const int waste = rounds * cand - per_wave + 4 * (rounds - 1);   // a further round costs about four steps
+      if (waste < best_waste) { best_waste = waste; u = cand; }
+    }
+  }
+  switch (u) {
+    case 2: LaunchGemmRowPanelShape<RT, CT, 2>(a, stream); break;
+    case 4: LaunchGemmRowPanelShape<RT, CT, 4>(a, stream); break;
+    case 6: LaunchGemmRowPanelShape<RT, CT, 6>(a, stream); break;
+    default:
+      if constexpr (kMaxU >= 8) LaunchGemmRowPanelShape<RT, CT, 8>(a, stream);
+      else LaunchGemmRowPanelShape<RT, CT, 6>(a, stream);
+      break;
+  }
+}
+
+inline void LaunchGemmRowPanel(const GemmArgs& a, hipStream_t stream) {
+  const RowPanelShape c = PickRowPanelShape(a);
+  if (c.rt == 1 && c.ct == 1) LaunchGemmRowPanelSteps<1, 1>(a, stream);
+  else if (c.rt == 2 && c.ct == 1) LaunchGemmRowPanelSteps<2, 1>(a, stream);
+  else if (c.rt == 1 && c.ct == 2) LaunchGemmRowPanelSteps<1, 2>(a, stream);
+  else if (c.rt == 2 && c.ct == 2) LaunchGemmRowPanelSteps<2, 2>(a, stream);
+  else LaunchGemmRowPanelSteps<4, 2>(a, stream);
+}
+
 enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128, kRowPanel, kDma128x64, kPersist256,
                    kDma128x32 };
 
@@ -887,12 +961,16 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
   if (!a.out_f32 && a.split_k == 1 && a.batch == 1 && a.N <= 32 && a.K % 64 == 0 && a.K >= 128 && a.M >= 32768) {
     return kDma128x32;
   }
-  // Small problems with a long reduction: the 64x64 kernel walks K serially in one workgroup;
-  // when it would start at most 64 workgroups, the row-panel kernel (8-way K split inside the
-  // workgroup, 64x32 panels) is faster (64x3072x1024: 8.5 vs 9.7 us; 8192x32x1024: 9.2 vs 11.9 us).
-  // With a short K and many columns it loses (128x8192x256: 15.8 vs 5.6 us).
+  // Small problems: the 64x64 kernel walks K serially in one workgroup; when it would start at most 64 workgroups,
+  // the row-panel kernel (8-way K split inside the workgroup, panels sized to give every CU one) is faster
+  // (64x3072x1024: 6.4 vs 9.7 us; 32x4096x256: 3.1 vs 5.1 us). With a short K and more panels than CUs it loses
+  // (128x8192x256 in 64x32 panels: 15.8 vs 5.6 us).
+  // The same holds for a handful of rows with thousands of columns, as long as panels of at most 32x32 cover them
+  // with one workgroup per CU (1x8192x256: 2.9 vs 5.0 us).
   const long long tiles64 = (long long)((a.M + 63) / 64) * ((a.N + 63) / 64) * a.batch;
-  if (a.split_k == 1 && tiles64 <= 64 && a.K >= 512) return kRowPanel;
+  if (a.split_k == 1 && a.K >= 256 && (tiles64 <= 64 || RowPanelWorkgroups(a, kRowPanelShapes[3]) <= kRowPanelWorkgroups)) {
+    return kRowPanel;
+  }
   // A single 32-column panel (the smolgen compression): one workgroup per 64 rows, K split over its waves
   // (16384x32x1024: 9.5 us against 12.3 for the 64x64 tiles, but with twice the threads on every CU).
   if (a.latency_first && a.split_k == 1 && a.N <= 32 && a.K >= 512) return kRowPanel;
@@ -944,7 +1022,7 @@ const char* GemmVariantName(const GemmArgs& a) {
     case kDma128x128: return "gemm_dma_128x128x64";
     case kDma128x64: return "gemm_dma_128x64x64";
     case kDma128x32: return "gemm_dma_128x32x64";
-    case kRowPanel: return "gemm_rowpanel_64x32";
+    case kRowPanel: return "gemm_rowpanel";
     case kTile128: return "gemm_128x128x64";
     default: return a.split_k > 1 ? "gemm_64x64x64_splitk" : "gemm_64x64x64";
   }
@@ -963,15 +1041,7 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
     case kDma128x128: LaunchGemmDma<128, 128, 64, 2, 2>(a, stream); break;
     case kDma128x64: LaunchGemmDma<128, 64, 64, 2, 2>(a, stream); break;
     case kDma128x32: LaunchGemmDma<128, 32, 64, 4, 1>(a, stream); break;
-    case kRowPanel: {
-      dim3 grid((a.M + 63) / 64, (a.N + 31) / 32, a.batch);
-      if (a.out_f32) {
-        hipLaunchKernelGGL(gemm_rowpanel_kernel<float>, grid, dim3(512), 0, stream, a);
-      } else {
-        hipLaunchKernelGGL(gemm_rowpanel_kernel<half_t>, grid, dim3(512), 0, stream, a);
-      }
-      break;
-    }
+    case kRowPanel: LaunchGemmRowPanel(a, stream); break;
     case kTile128: LaunchGemmTile<128, 128, 64, 2, 2>(a, stream); break;
     default: LaunchGemmTile<64, 64, 64, 2, 2>(a, stream); break;
   }
@@ -1330,6 +1400,10 @@ __global__ __launch_bounds__(256) void zero_kernel(float* p, long long n) {
 }
 
 // One workgroup per row; every thread keeps up to 4 vectors of 8 elements.
+// EARLY (few rows, where the kernel's latency is the pass's): gamma and beta, which nobody has touched since the
+// previous pass, are asked for first and arrive while the row is reduced; otherwise they are read where they are
+// used, which leaves more of the CU to a GEMM on the other stream.
+template <bool EARLY>
 __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __restrict__ xf, int n_partials,
                                                               long long partial_stride, const half_t* xh,
                                                               int pre_act, const half_t* skip, half_t* y,
@@ -1339,38 +1413,52 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __res
   __shared__ float red[4];
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int nvec = C / 8;
-  float t[4][8];
-  float sum = 0.0f;
+  [[maybe_unused]] floatx4 gm[4][2], bt[4][2];
+  if constexpr (EARLY) {
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int v = tid + i * 256;
-#pragma unroll
-    for (int e = 0; e < 8; e++) t[i][e] = 0.0f;
-    if (v < nvec) {
-      const long long off = (long long)row * C + v * 8;
-      if (xf != nullptr) {
-        for (int part = 0; part < n_partials; part++) {
-          floatx4 a = *reinterpret_cast<const floatx4*>(xf + part * partial_stride + off);
-          floatx4 b = *reinterpret_cast<const floatx4*>(xf + part * partial_stride + off + 4);
-#pragma unroll
-          for (int e = 0; e < 4; e++) { t[i][e] += a[e]; t[i][4 + e] += b[e]; }
-        }
-      } else {
-        half8 h = *reinterpret_cast<const half8*>(xh + off);
-#pragma unroll
-        for (int e = 0; e < 8; e++) t[i][e] = (float)h[e];
-      }
-#pragma unroll
-      for (int e = 0; e < 8; e++) t[i][e] = Activate(t[i][e], pre_act) * alpha;
-      if (skip != nullptr) {
-        half8 hs = *reinterpret_cast<const half8*>(skip + off);
-#pragma unroll
-        for (int e = 0; e < 8; e++) t[i][e] += (float)hs[e];
-      }
-#pragma unroll
-      for (int e = 0; e < 8; e++) sum += t[i][e];
+    for (int i = 0; i < 4; i++) {
+      const int v = min(tid + i * 256, nvec - 1);
+      gm[i][0] = *reinterpret_cast<const floatx4*>(gamma + v * 8);
+      gm[i][1] = *reinterpret_cast<const floatx4*>(gamma + v * 8 + 4);
+      bt[i][0] = *reinterpret_cast<const floatx4*>(beta + v * 8);
+      bt[i][1] = *reinterpret_cast<const floatx4*>(beta + v * 8 + 4);
     }
   }
+  float t[4][8];
+  float sum = 0.0f;
+  // One switch over the activation for the kernel, not one per element.
+  DispatchAct(pre_act, [&](auto act_fn) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int v = tid + i * 256;
+#pragma unroll
+      for (int e = 0; e < 8; e++) t[i][e] = 0.0f;
+      if (v < nvec) {
+        const long long off = (long long)row * C + v * 8;
+        if (xf != nullptr) {
+          for (int part = 0; part < n_partials; part++) {
+            floatx4 a = *reinterpret_cast<const floatx4*>(xf + part * partial_stride + off);
+            floatx4 b = *reinterpret_cast<const floatx4*>(xf + part * partial_stride + off + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) { t[i][e] += a[e]; t[i][4 + e] += b[e]; }
+          }
+        } else {
+          half8 h = *reinterpret_cast<const half8*>(xh + off);
+#pragma unroll
+          for (int e = 0; e < 8; e++) t[i][e] = (float)h[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) t[i][e] = act_fn(t[i][e]) * alpha;
+        if (skip != nullptr) {
+          half8 hs = *reinterpret_cast<const half8*>(skip + off);
+#pragma unroll
+          for (int e = 0; e < 8; e++) t[i][e] += (float)hs[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) sum += t[i][e];
+      }
+    }
+  });
   sum = WaveSum(sum);
   if (lane == 0) red[wave] = sum;
   __syncthreads();
@@ -1391,9 +1479,15 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __res
   for (int i = 0; i < 4; i++) {
     const int v = tid + i * 256;
     if (v < nvec) {
+      if constexpr (!EARLY) {
+        gm[i][0] = *reinterpret_cast<const floatx4*>(gamma + v * 8);
+        gm[i][1] = *reinterpret_cast<const floatx4*>(gamma + v * 8 + 4);
+        bt[i][0] = *reinterpret_cast<const floatx4*>(beta + v * 8);
+        bt[i][1] = *reinterpret_cast<const floatx4*>(beta + v * 8 + 4);
+      }
       half8 o;
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = (half_t)(beta[v * 8 + e] + gamma[v * 8 + e] * (t[i][e] - mean) * den);
+      for (int e = 0; e < 8; e++) o[e] = (half_t)(bt[i][e / 4][e % 4] + gm[i][e / 4][e % 4] * (t[i][e] - mean) * den);
       *reinterpret_cast<half8*>(y + (long long)row * C + v * 8) = o;
     }
   }
@@ -1422,8 +1516,13 @@ void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_s
                          int pre_act, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows,
                          int C, float alpha, float eps, hipStream_t stream) {
   if (rows <= 0) return;
-  hipLaunchKernelGGL(layer_norm_rows_kernel, dim3(rows), dim3(256), 0, stream, x_f32, n_partials, partial_stride,
-                     x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps);
+  if (rows <= 64) {
+    hipLaunchKernelGGL(layer_norm_rows_kernel<true>, dim3(rows), dim3(256), 0, stream, x_f32, n_partials,
+                       partial_stride, x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps);
+  } else {
+    hipLaunchKernelGGL(layer_norm_rows_kernel<false>, dim3(rows), dim3(256), 0, stream, x_f32, n_partials,
+                       partial_stride, x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps);
+  }
 }
 
 void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,

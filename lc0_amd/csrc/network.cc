@@ -283,6 +283,7 @@ struct ModelState {
   bool fold_layer_norm_ = false;
   bool fused_smolgen_attention_ = true;
   int fused_smolgen_min_batch_ = 96;
+  int dense1_split_min_batch_ = 64;   // smallest batch whose smolgen dense1 splits K between workgroups
   bool qkv_first_ = true;
   half_t* smolgen_wfrag_ = nullptr;   // smolgen_w in the fragment order of smolgen_attention_kernel (null: not fused)
   bool any_smolgen_ = false;
@@ -874,6 +875,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   // separate GEMM and attention kernels are faster; 15x1024 net: batch 128 +4 %, 256 +1.5 %, 1024 +2 %, 64 -1 %, 16 -6 %).
   fused_smolgen_attention_ = options.GetBool("fused_smolgen_attention", true);
   fused_smolgen_min_batch_ = options.GetInt("fused_smolgen_min_batch", 96);
+  dense1_split_min_batch_ = options.GetInt("dense1_split_min_batch", 64);
   qkv_first_ = options.GetBool("qkv_first", true);
   fp8_fp16_layers_ = options.GetInt("fp8_fp16_layers", 0);
   if (fp8_fp16_layers_ < 0) throw Error("fp8_fp16_layers must not be negative.");
@@ -1660,14 +1662,24 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       const bool chain_first = f8 || B <= 128;
       Gemm("gemm_smolgen_compress", x_, emb_, norm_in ? e.sg_compress_n : e.sg_compress, sg1_, sg_hc_, T, kActNone,
            false, ss, 1, chain_first, norm_in ? &cons_in : nullptr);
-      // dense1 has a long reduction and few outputs: split K, accumulate in float,
-      // and let the layer norm kernel apply the activation.
-      const int split = std::max(1, std::min(16, (64 * sg_hc_) / 256));
-      Gemm("gemm_smolgen_dense1", sg1_, 64 * sg_hc_, e.sg_dense1, sg2f_, sg_hs_, B, kActNone, true, ss, split);
-      Timed("layer_norm_rows", 0.0, (4.0 * split + 2.0) * B * sg_hs_, [&] {
-        LaunchLayerNormRows(sg2f_, split, static_cast<long long>(B) * sg_hs_, nullptr, smolgen_act_, nullptr, sg2_,
-                            e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f, 1e-3f, ss);
-      }, ss);
+      // dense1 has a long reduction and few outputs. With few rows one workgroup per 16x16 outputs splits K over
+      // its waves; from dense1_split_min_batch_ rows on, workgroups split K between them, accumulate in float, and
+      // the layer norm kernel adds the slices and applies the activation.
+      if (B < dense1_split_min_batch_) {
+        Gemm("gemm_smolgen_dense1", sg1_, 64 * sg_hc_, e.sg_dense1, sg2_, sg_hs_, B, smolgen_act_, false, ss, 1,
+             chain_first);
+        Timed("layer_norm_rows", 0.0, 4.0 * B * sg_hs_, [&] {
+          LaunchLayerNormRows(nullptr, 0, 0, sg2_, kActNone, nullptr, sg2_, e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f,
+                              1e-3f, ss);
+        }, ss);
+      } else {
+        const int split = std::max(1, std::min(16, (64 * sg_hc_) / 256));
+        Gemm("gemm_smolgen_dense1", sg1_, 64 * sg_hc_, e.sg_dense1, sg2f_, sg_hs_, B, kActNone, true, ss, split);
+        Timed("layer_norm_rows", 0.0, (4.0 * split + 2.0) * B * sg_hs_, [&] {
+          LaunchLayerNormRows(sg2f_, split, static_cast<long long>(B) * sg_hs_, nullptr, smolgen_act_, nullptr, sg2_,
+                              e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f, 1e-3f, ss);
+        }, ss);
+      }
       Gemm("gemm_smolgen_dense2", sg2_, sg_hs_, e.sg_dense2, sg3_, sg_gen_, B, smolgen_act_, false, ss, 1, chain_first);
       Timed("layer_norm_rows", 0.0, 4.0 * B * sg_gen_, [&] {
         LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f, 1e-3f,

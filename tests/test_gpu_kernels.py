@@ -96,6 +96,50 @@ def test_every_gemm_variant_vs_oracle_fc(variant, m, n, k):
     np.testing.assert_allclose(got, onn.fc(a, w.reshape(-1), b, nr.ACT_MISH), rtol=2e-3, atol=2e-3)
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (1, 256, 2048),      # 16x16 panels, eight steps of 32 per wave in one round
+    (64, 1024, 1536),    # 16x16 panels, six steps
+    (64, 1536, 1024),    # 32x16 panels
+    (7, 8192, 264),      # 16x32 panels, a last step of 8 values
+    (64, 3072, 1024),    # 32x32 panels
+    (512, 1024, 528),    # 64x32 panels, a last step of 16 values
+    (100, 700, 4096),    # sixteen steps per wave: two rounds of eight
+    (130, 600, 3392),    # fourteen steps per wave, a last wave with fewer
+    (33, 50, 40),        # a single full step and a last step of 8 values
+    (16, 16, 8),         # nothing but the last step
+    (20000, 40, 512)])   # more panels than CUs: the largest panel shape
+def test_row_panel_gemm_panel_shapes_and_reduction_tails(m, n, k):
+    """The row-panel kernel (variant 6) picks its panel by problem size and its load depth by K: every panel shape,
+    every depth, reductions that are not multiples of 32, half and float output, with activation and without bias,
+    against FullyConnectedLayer::Forward1D (blas/fully_connected_layer.cc:49-106)."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(m * 5 + n * 3 + k)
+    a = _h(rng.standard_normal((m, k)) * 0.5)
+    w = _h(rng.standard_normal((n, k)) * 0.1)
+    b = rng.standard_normal(n).astype(f32)
+    K.set_gemm_variant(6)
+    try:
+        got32 = K.gemm(a, w, b, act=nr.ACT_MISH, out_f32=True)
+        got16 = K.gemm(a, w, None, act=nr.ACT_NONE).astype(f32)
+    finally:
+        K.set_gemm_variant(-1)
+    np.testing.assert_allclose(got32, onn.fc(a, w.reshape(-1), b, nr.ACT_MISH), rtol=2e-4, atol=2e-4)
+    np.testing.assert_allclose(got16, onn.fc(a, w.reshape(-1), np.zeros(n, f32), nr.ACT_NONE), rtol=2e-3, atol=2e-3)
+
+
+def test_row_panel_gemm_batched_with_scale():
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(11)
+    a = _h(rng.standard_normal((3, 40, 288)))
+    w = _h(rng.standard_normal((3, 70, 288)))
+    K.set_gemm_variant(6)
+    try:
+        got = K.gemm(a, w, None, scale=0.125, out_f32=True)
+    finally:
+        K.set_gemm_variant(-1)
+    np.testing.assert_allclose(got, np.matmul(a, w.transpose(0, 2, 1)) * 0.125, rtol=2e-4, atol=2e-4)
+
+
 @pytest.mark.parametrize("rows,c,f32_in,act", [(256, 256, True, nr.ACT_SWISH), (256, 8192, False, nr.ACT_NONE),
                                                (3, 32, True, nr.ACT_MISH), (17, 1024, False, nr.ACT_RELU)])
 def test_layer_norm_rows_vs_oracle(rows, c, f32_in, act):
