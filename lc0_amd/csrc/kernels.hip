@@ -395,12 +395,16 @@ __device__ __forceinline__ void DmaToLds16(const void* gptr, void* lds_base) {
 // STREAM: the output is written with streaming (non-temporal) stores.
 // EPI (fp16 operands only): 0 the plain epilogue, 1 the consumer and 2 the producer side of a folded layer norm
 // (GemmArgs::row_stats / GemmArgs::skip).
+// NSTAGES k-tiles of LDS: NSTAGES - 1 of them are in flight while one is consumed. Two stages suffice when the
+// operands come from L2; with small tiles and operands that come from memory (a few hundred to a few thousand rows:
+// every workgroup streams weights nobody has touched since the previous pass) a k-tile takes longer to arrive than
+// to consume, and more stages hide that.
 template <int BM, int BN, int BKB, int WAVES_M, int WAVES_N, typename Args, typename OutT, bool STREAM = false,
-          int EPI = 0>
+          int EPI = 0, int NSTAGES = 2>
 // Second launch bound = waves per SIMD: with small wave tiles two workgroups share a CU
 // (4 waves per SIMD, at most 128 VGPRs) and overlap each other's prologue and epilogue.
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
-                             ((BM / WAVES_M / 32) * (BN / WAVES_N / 32) <= 4 && 4 * (BM + BN) * BKB <= 160 * 1024)
+                             ((BM / WAVES_M / 32) * (BN / WAVES_N / 32) <= 4 && 2 * NSTAGES * (BM + BN) * BKB <= 160 * 1024)
                                  ? WAVES_M * WAVES_N / 2
                                  : WAVES_M * WAVES_N / 4)
 void gemm_dma_kernel(Args p) {
@@ -424,7 +428,8 @@ void gemm_dma_kernel(Args p) {
   constexpr int STAT_BYTES = (EPI != 0) ? BM * 8 : 0;
   constexpr int PART_BYTES = (EPI == 2) ? WAVES_N * BM * 8 : 0;
   constexpr int EPI_TOTAL = EPI_BYTES + STAT_BYTES + PART_BYTES;
-  constexpr int SMEM = (2 * STAGE > EPI_TOTAL) ? 2 * STAGE : EPI_TOTAL;
+  constexpr int SMEM = (NSTAGES * STAGE > EPI_TOTAL) ? NSTAGES * STAGE : EPI_TOTAL;
+  static_assert(NSTAGES >= 2 && (NSTAGES - 2) * (A_CPW + W_CPW) <= 63, "transfers in flight must fit the counter");
   static_assert(EPI == 0 || (!F8 && sizeof(OutT) == 2), "folded layer norm: fp16 operands and output");
   // The tile's bias (and per-column scale, fp8 operands) waits in LDS behind the stages: fetched with the first k-tile,
   // so that the epilogue does not start with a round trip to memory.
@@ -485,6 +490,10 @@ void gemm_dma_kernel(Args p) {
 
   const int nk = K * ES / BKB;
   issue(smem, smem + BM * BKB, 0);
+#pragma unroll
+  for (int st = 1; st < NSTAGES - 1; st++) {
+    if (st < nk) issue(smem + st * STAGE, smem + st * STAGE + BM * BKB, st * BKB);
+  }
   if (tid < BN) {
     colv[tid] = my_bias;
     if constexpr (F8) colv[BN + tid] = my_cscale;
@@ -505,12 +514,23 @@ void gemm_dma_kernel(Args p) {
   // epilogue finds it in cache instead of reading memory in the same burst in which every workgroup writes.
   [[maybe_unused]] int touch[(BM * BN * 2 / 128 + NWAVES * 64 - 1) / (NWAVES * 64)] = {};
   for (int kt = 0; kt < nk; kt++) {
-    const char* As = smem + (kt & 1) * STAGE;
+    const char* As = smem + (NSTAGES == 2 ? (kt & 1) : kt % NSTAGES) * STAGE;
     const char* Ws = As + BM * BKB;
-    char* nxt = smem + ((kt + 1) & 1) * STAGE;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of k-tile kt have landed
-    __syncthreads();                     // ... and everybody's; everybody is done reading the other stage
-    if (kt + 1 < nk) issue(nxt, nxt + BM * BKB, (kt + 1) * BKB);
+    char* nxt = smem + (NSTAGES == 2 ? ((kt + 1) & 1) : (kt + NSTAGES - 1) % NSTAGES) * STAGE;
+    // This wave's pieces of k-tile kt have landed: the transfers of the NSTAGES - 2 k-tiles behind it may still be
+    // in flight (near the end of K fewer are, and the wait is for all of them).
+    constexpr int IN_FLIGHT = (NSTAGES - 2) * (A_CPW + W_CPW);
+    if constexpr (NSTAGES > 2) {
+      if (kt + NSTAGES - 2 < nk) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14));
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      }
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    }
+    __syncthreads();                     // ... and everybody's; everybody is done reading the stage filled next
+    if (kt + NSTAGES - 1 < nk) issue(nxt, nxt + BM * BKB, (kt + NSTAGES - 1) * BKB);
     if constexpr (EPI == 2) {
       if (kt == 1) {
         constexpr int LINES_PER_ROW = (BN * 2 + 127) / 128;
@@ -779,7 +799,7 @@ inline bool StreamOutput(long long m, long long n, long long batch, int elem_byt
   return bytes >= (64LL << 20) || (m >= 16384 && bytes >= (32LL << 20));
 }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int NSTAGES = 2>
 void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
   dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch);
   const dim3 block(WAVES_M * WAVES_N * 64);
@@ -787,14 +807,14 @@ void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
     constexpr bool S = decltype(stream_tag)::value;
     if (a.skip != nullptr) {
       if constexpr ((BN / WAVES_N) % 64 == 0 || BN / WAVES_N == 32) {
-        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 2>), grid, block, 0,
+        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 2, NSTAGES>), grid, block, 0,
                            stream, a);
       }
     } else if (a.row_stats != nullptr) {
-      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 1>), grid, block, 0,
+      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 1, NSTAGES>), grid, block, 0,
                          stream, a);
     } else {
-      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 0>), grid, block, 0,
+      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 0, NSTAGES>), grid, block, 0,
                          stream, a);
     }
   };
@@ -805,6 +825,23 @@ void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
     }
   }
   launch(std::false_type{});
+}
+
+// As many LDS stages (2 to 4) as leave room on the CUs for all of the launch's workgroups at once: with one
+// workgroup per CU nothing else hides the time a k-tile takes to arrive from memory, with several per CU they hide it
+// for each other and more stages would only lower their number (15x1024 net, per pass: 16 positions 1.91 -> 1.67 ms
+// with four stages; 64 positions 2.59 -> 2.93 ms if forced there).
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+void LaunchGemmDmaStaged(const GemmArgs& a, hipStream_t stream) {
+  constexpr int kStage = (BM + BN) * BK * 2, kLds = 160 * 1024, kCus = 256;
+  const long long wgs = (long long)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN) * a.batch;
+  if constexpr (4 * kStage + 4096 <= kLds) {
+    if (wgs <= (long long)kCus * (kLds / (4 * kStage + 4096))) return LaunchGemmDma<BM, BN, BK, WAVES_M, WAVES_N, 4>(a, stream);
+  }
+  if constexpr (3 * kStage + 4096 <= kLds) {
+    if (wgs <= (long long)kCus * (kLds / (3 * kStage + 4096))) return LaunchGemmDma<BM, BN, BK, WAVES_M, WAVES_N, 3>(a, stream);
+  }
+  LaunchGemmDma<BM, BN, BK, WAVES_M, WAVES_N, 2>(a, stream);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BKB = 128>
@@ -1037,9 +1074,9 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
     case kPersist256: LaunchGemmPersistent(a, StreamOutput(a.M, a.N, a.batch, 2), stream); break;
     case kDma256x256: LaunchGemmDma<256, 256, 64, 2, 4>(a, stream); break;
     case kDma256x192: LaunchGemmDma<256, 192, 64, 4, 2>(a, stream); break;
-    case kDma256x128: LaunchGemmDma<256, 128, 32, 4, 2>(a, stream); break;
-    case kDma128x128: LaunchGemmDma<128, 128, 64, 2, 2>(a, stream); break;
-    case kDma128x64: LaunchGemmDma<128, 64, 64, 2, 2>(a, stream); break;
+    case kDma256x128: LaunchGemmDmaStaged<256, 128, 32, 4, 2>(a, stream); break;
+    case kDma128x128: LaunchGemmDmaStaged<128, 128, 64, 2, 2>(a, stream); break;
+    case kDma128x64: LaunchGemmDmaStaged<128, 64, 64, 2, 2>(a, stream); break;
     case kDma128x32: LaunchGemmDma<128, 32, 64, 4, 1>(a, stream); break;
     case kRowPanel: LaunchGemmRowPanel(a, stream); break;
     case kTile128: LaunchGemmTile<128, 128, 64, 2, 2>(a, stream); break;
