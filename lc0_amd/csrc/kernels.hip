@@ -942,7 +942,7 @@ inline void LaunchGemmRowPanel(const GemmArgs& a, hipStream_t stream) {
 }
 
 enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDma128x128, kRowPanel, kDma128x64, kPersist256,
-                   kDma128x32 };
+                   kDma128x32, kDma64x64 };
 
 int g_variant_override = -1;
 
@@ -950,7 +950,8 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
   if (g_variant_override >= 0) {
     const bool dma_ok = !a.out_f32 && a.split_k == 1 && a.K % 64 == 0;
     const bool is_dma = g_variant_override <= kDma256x128 || g_variant_override == kDma128x128 ||
-                        g_variant_override == kDma128x64 || g_variant_override == kDma128x32;
+                        g_variant_override == kDma128x64 || g_variant_override == kDma128x32 ||
+                        g_variant_override == kDma64x64;
     bool ok = is_dma ? dma_ok : (g_variant_override != kRowPanel || a.split_k == 1);
     if (g_variant_override == kPersist256) ok = GemmPersistentSupports(a);
     if (ok) return static_cast<GemmVariant>(g_variant_override);
@@ -1008,6 +1009,16 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
   if (a.split_k == 1 && a.K >= 256 && (tiles64 <= 64 || RowPanelWorkgroups(a, kRowPanelShapes[3]) <= kRowPanelWorkgroups)) {
     return kRowPanel;
   }
+  // A few hundred rows (2 to 12 positions), or few columns: too small for the cost model above, too large for row
+  // panels. Small direct-to-LDS tiles with three or four stages in flight stream the weights, which come from
+  // memory, better than the register-staged tiles below (512x1024x1024: 6.8 against 9.9 us; a pass of 8 positions
+  // 1.94 -> 1.46 ms). 128x64 tiles once they fill most CUs (512x3072x1024: 9.6 against 11.1 us), 64x64 before.
+  // (With a short reduction only on request: beside a large GEMM on the other stream the register-staged tiles
+  // disturb it less.)
+  if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= (a.latency_first ? 256 : 512) && a.N >= 64 && a.M >= 256) {
+    const long long wg128 = (long long)((a.M + 127) / 128) * ((a.N + 63) / 64) * a.batch;
+    return wg128 >= 192 ? kDma128x64 : kDma64x64;
+  }
   // A single 32-column panel (the smolgen compression): one workgroup per 64 rows, K split over its waves
   // (16384x32x1024: 9.5 us against 12.3 for the 64x64 tiles, but with twice the threads on every CU).
   if (a.latency_first && a.split_k == 1 && a.N <= 32 && a.K >= 512) return kRowPanel;
@@ -1025,7 +1036,7 @@ int DmaTileN(GemmVariant v) {
     case kDma256x256: return 256;
     case kDma256x192: return 192;
     case kDma256x128: case kDma128x128: return 128;
-    case kDma128x64: return 64;
+    case kDma128x64: case kDma64x64: return 64;
     case kDma128x32: return 32;
     default: return 0;
   }
@@ -1059,6 +1070,7 @@ const char* GemmVariantName(const GemmArgs& a) {
     case kDma128x128: return "gemm_dma_128x128x64";
     case kDma128x64: return "gemm_dma_128x64x64";
     case kDma128x32: return "gemm_dma_128x32x64";
+    case kDma64x64: return "gemm_dma_64x64x64";
     case kRowPanel: return "gemm_rowpanel";
     case kTile128: return "gemm_128x128x64";
     default: return a.split_k > 1 ? "gemm_64x64x64_splitk" : "gemm_64x64x64";
@@ -1078,6 +1090,7 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
     case kDma128x128: LaunchGemmDmaStaged<128, 128, 64, 2, 2>(a, stream); break;
     case kDma128x64: LaunchGemmDmaStaged<128, 64, 64, 2, 2>(a, stream); break;
     case kDma128x32: LaunchGemmDma<128, 32, 64, 4, 1>(a, stream); break;
+    case kDma64x64: LaunchGemmDmaStaged<64, 64, 64, 2, 2>(a, stream); break;
     case kRowPanel: LaunchGemmRowPanel(a, stream); break;
     case kTile128: LaunchGemmTile<128, 128, 64, 2, 2>(a, stream); break;
     default: LaunchGemmTile<64, 64, 64, 2, 2>(a, stream); break;

@@ -1685,7 +1685,9 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
         LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f, 1e-3f,
                             ss);
       }, ss);
-      if (!fused_gen) Gemm("gemm_smolgen_global", sg3_, g, smolgen_w_, sbias_, 4096, B * heads_, kActNone, false, ss);
+      if (!fused_gen) {
+        Gemm("gemm_smolgen_global", sg3_, g, smolgen_w_, sbias_, 4096, B * heads_, kActNone, false, ss, 1, chain_first);
+      }
       if (ss != stream_) HIP_CHECK(hipEventRecord(join_events_[li], ss));
       bias = sbias_;
     }

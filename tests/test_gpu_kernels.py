@@ -78,7 +78,7 @@ def test_persistent_gemm_vs_oracle_fc(m, n, k, act, bias):
     np.testing.assert_allclose(got[rows], want, rtol=2e-3, atol=2e-3)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 9])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 9, 10])
 @pytest.mark.parametrize("m,n,k", [(2048, 1024, 256), (777, 200, 128), (300, 1858, 64), (64, 64, 192), (1000, 32, 256)])
 def test_every_gemm_variant_vs_oracle_fc(variant, m, n, k):
     """Every tile variant (the three direct-to-LDS kernels and the two
