@@ -1009,13 +1009,13 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
   if (a.split_k == 1 && a.K >= 256 && (tiles64 <= 64 || RowPanelWorkgroups(a, kRowPanelShapes[3]) <= kRowPanelWorkgroups)) {
     return kRowPanel;
   }
-  // A few hundred rows (2 to 12 positions), or few columns: too small for the cost model above, too large for row
+  // A few hundred rows (3 to 12 positions), or few columns: too small for the cost model above, too large for row
   // panels. Small direct-to-LDS tiles with three or four stages in flight stream the weights, which come from
   // memory, better than the register-staged tiles below (512x1024x1024: 6.8 against 9.9 us; a pass of 8 positions
   // 1.94 -> 1.46 ms). 128x64 tiles once they fill most CUs (512x3072x1024: 9.6 against 11.1 us), 64x64 before.
   // (With a short reduction only on request: beside a large GEMM on the other stream the register-staged tiles
   // disturb it less.)
-  if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= (a.latency_first ? 256 : 512) && a.N >= 64 && a.M >= 256) {
+  if (!a.out_f32 && a.split_k == 1 && a.K % 64 == 0 && a.K >= (a.latency_first ? 256 : 512) && a.N >= 64 && a.M >= 192) {
     const long long wg128 = (long long)((a.M + 127) / 128) * ((a.N + 63) / 64) * a.batch;
     return wg128 >= 192 ? kDma128x64 : kDma64x64;
   }
