@@ -365,6 +365,86 @@ __global__ __launch_bounds__(512) void gemm_rowpanel_kernel(GemmArgs p) {
   });
 }
 
+// The same panel scheme for e4m3 operands (v_mfma_f32_16x16x128_f8f6f4): a k-step is 128 values, a lane holds 32
+// consecutive bytes of its row, so every fragment load covers sixteen full 128-byte lines.
+template <int RT, int CT, int U, typename OutT>
+__global__ __launch_bounds__(512) void gemm_f8_rowpanel_kernel(GemmF8Args p) {
+  constexpr int NW = 8, ROWS = 16 * RT, COLS = 16 * CT, LD = COLS + 1;
+  __shared__ float part[NW][ROWS * LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int m0 = blockIdx.x * ROWS, n0 = blockIdx.y * COLS;
+  const int M = p.M, N = p.N;
+  const int steps = p.K / 128;
+  const int per_wave = (steps + NW - 1) / NW;
+  const int s_begin = min(steps, wave * per_wave), s_end = min(steps, s_begin + per_wave);
+  const uint8_t* a_row[RT];
+  const uint8_t* w_row[CT];
+#pragma unroll
+  for (int t = 0; t < RT; t++) a_row[t] = p.A + (long long)min(m0 + 16 * t + r, M - 1) * p.lda + 32 * g;
+#pragma unroll
+  for (int c = 0; c < CT; c++) w_row[c] = p.W + (long long)min(n0 + 16 * c + r, N - 1) * p.ldw + 32 * g;
+  floatx4 acc[RT][CT];
+#pragma unroll
+  for (int t = 0; t < RT; t++)
+#pragma unroll
+    for (int c = 0; c < CT; c++) acc[t][c] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+  auto load32 = [](const uint8_t* ptr) {
+    const intx4 lo = *reinterpret_cast<const intx4*>(ptr);
+    const intx4 hi = *reinterpret_cast<const intx4*>(ptr + 16);
+    return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+  for (int st = s_begin; st < s_end; st += U) {
+    intx8 fa[RT][U], fw[CT][U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {   // steps past the end re-read the last one (never used)
+      const int k = min(st + u, s_end - 1) * 128;
+#pragma unroll
+      for (int t = 0; t < RT; t++) fa[t][u] = load32(a_row[t] + k);
+#pragma unroll
+      for (int c = 0; c < CT; c++) fw[c][u] = load32(w_row[c] + k);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      if (st + u < s_end) {
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+          for (int c = 0; c < CT; c++)
+            acc[t][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fw[c][u], fa[t][u], acc[t][c], 0, 0, 0, 0, 0, 0);
+      }
+    }
+  }
+  float* mine = part[wave];
+#pragma unroll
+  for (int t = 0; t < RT; t++)
+#pragma unroll
+    for (int c = 0; c < CT; c++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) mine[(16 * t + r) * LD + 16 * c + 4 * g + e] = acc[t][c][e];
+  __syncthreads();
+  OutT* C = reinterpret_cast<OutT*>(p.C);
+  DispatchAct(p.act, [&](auto act_fn) {
+#pragma unroll
+    for (int i = 0; i < (ROWS * COLS + 511) / 512; i++) {
+      const int idx = tid + 512 * i;        // consecutive threads along n
+      const int row = idx / COLS, col = idx % COLS;
+      const int m = m0 + row, n = n0 + col;
+      if (row < ROWS && m < M && n < N) {
+        float sum = part[0][row * LD + col];
+#pragma unroll
+        for (int w = 1; w < NW; w++) sum += part[w][row * LD + col];
+        const float v = act_fn(sum * p.col_scale[n] + (p.bias ? p.bias[n] : 0.0f));
+        if constexpr (sizeof(OutT) == 1) {
+          C[(long long)m * p.ldc + n] = (uint8_t)(PackFp8x4(v * p.out_mul, 0.0f, 0.0f, 0.0f) & 0xFFu);
+        } else {
+          C[(long long)m * p.ldc + n] = (OutT)v;
+        }
+      }
+    }
+  });
+}
+
 // ---------------------------------------------------------------------------
 // Large-shape GEMM: same contract as gemm_kernel for K % BK == 0 and half output.
 //
@@ -1100,11 +1180,51 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
 namespace {
 // 0: 256x256, 1: 256x192, 2: 256x128, 5: 128x128 and 7: 128x64 with 4 waves (two / three workgroups per CU); chosen by
 // the cost model of the fp16 kernels (the k-tile structure is the same).
+template <int RT, int CT>
+void LaunchGemmF8RowPanelSteps(const GemmF8Args& a, hipStream_t stream) {
+  dim3 grid((a.M + 16 * RT - 1) / (16 * RT), (a.N + 16 * CT - 1) / (16 * CT), 1);
+  const int per_wave = (a.K / 128 + 7) / 8;   // steps of 128 per wave: all of them in flight, up to four
+  auto launch = [&](auto u_tag) {
+    constexpr int U = decltype(u_tag)::value;
+    if (a.out_f8) {
+      hipLaunchKernelGGL((gemm_f8_rowpanel_kernel<RT, CT, U, uint8_t>), grid, dim3(512), 0, stream, a);
+    } else {
+      hipLaunchKernelGGL((gemm_f8_rowpanel_kernel<RT, CT, U, half_t>), grid, dim3(512), 0, stream, a);
+    }
+  };
+  if (per_wave <= 1) launch(std::integral_constant<int, 1>{});
+  else if (per_wave == 2) launch(std::integral_constant<int, 2>{});
+  else launch(std::integral_constant<int, 4>{});
+}
+
+GemmArgs PanelShapeArgs(const GemmF8Args& a) {
+  GemmArgs g;
+  g.M = a.M; g.N = a.N; g.K = a.K; g.batch = 1;
+  return g;
+}
+
+void LaunchGemmF8RowPanel(const GemmF8Args& a, hipStream_t stream) {
+  const RowPanelShape c = PickRowPanelShape(PanelShapeArgs(a));
+  if (c.rt == 1 && c.ct == 1) LaunchGemmF8RowPanelSteps<1, 1>(a, stream);
+  else if (c.rt == 2 && c.ct == 1) LaunchGemmF8RowPanelSteps<2, 1>(a, stream);
+  else if (c.rt == 1 && c.ct == 2) LaunchGemmF8RowPanelSteps<1, 2>(a, stream);
+  else if (c.rt == 2 && c.ct == 2) LaunchGemmF8RowPanelSteps<2, 2>(a, stream);
+  else LaunchGemmF8RowPanelSteps<4, 2>(a, stream);
+}
+
+// Few rows: row panels, as for fp16 operands.
+bool GemmF8TakesRowPanels(const GemmF8Args& a) {
+  const long long tiles64 = (long long)((a.M + 63) / 64) * ((a.N + 63) / 64);
+  return a.K >= 256 &&
+         (tiles64 <= 64 || RowPanelWorkgroups(PanelShapeArgs(a), kRowPanelShapes[3]) <= kRowPanelWorkgroups);
+}
+
 int PickGemmF8Variant(const GemmF8Args& a) {
-  if (g_variant_override >= 0 &&
-      (g_variant_override <= 2 || g_variant_override == kDma128x128 || g_variant_override == kDma128x64)) {
+  if (g_variant_override >= 0 && (g_variant_override <= 2 || g_variant_override == kDma128x128 ||
+                                  g_variant_override == kDma128x64 || g_variant_override == kRowPanel)) {
     return g_variant_override;
   }
+  if (GemmF8TakesRowPanels(a)) return kRowPanel;
   auto rounds = [&](int bm, int bn) {
     const long long tiles = (long long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn);
     return (double)((tiles + 255) / 256);
@@ -1132,6 +1252,7 @@ const char* GemmF8VariantName(const GemmF8Args& a) {
     case 1: return "gemm_f8_256x192x128";
     case 2: return "gemm_f8_256x128x128";
     case kDma128x64: return "gemm_f8_128x64x128";
+    case kRowPanel: return "gemm_f8_rowpanel";
     default: return "gemm_f8_128x128x128";
   }
 }
@@ -1143,6 +1264,7 @@ void LaunchGemmF8(const GemmF8Args& a, hipStream_t stream) {
     case 1: LaunchGemmDmaF8<256, 192, 4, 2>(a, stream); break;
     case 2: LaunchGemmDmaF8<256, 128, 4, 2>(a, stream); break;
     case kDma128x64: LaunchGemmDmaF8<128, 64, 2, 2>(a, stream); break;
+    case kRowPanel: LaunchGemmF8RowPanel(a, stream); break;
     default: LaunchGemmDmaF8<128, 128, 2, 2>(a, stream); break;
   }
 }

@@ -316,11 +316,14 @@ def test_quantize_f8_bit_exact():
         np.testing.assert_array_equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 5, 7])
-@pytest.mark.parametrize("m,n,k", [(512, 512, 128), (300, 200, 256), (2048, 1536, 1024), (64, 3072, 1024), (1, 17, 128)])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 5, 6, 7])
+@pytest.mark.parametrize("m,n,k", [(512, 512, 128), (300, 200, 256), (2048, 1536, 1024), (64, 3072, 1024), (1, 17, 128),
+                                   (64, 1024, 1536), (64, 1536, 1024), (5, 8192, 256), (700, 40, 4096)])
 def test_gemm_f8_vs_exact_product(variant, m, n, k):
     """e4m3 operands are exact inputs, so the product is pinned by float64 arithmetic on the decoded
-    values; tolerance covers fp32 accumulation and the fp16 output rounding."""
+    values; tolerance covers fp32 accumulation and the fp16 output rounding. Variant 6 is the row-panel kernel
+    (the last four shapes and (64, 3072, 1024) take one panel shape each; one, two and four 128-wide k-steps per
+    wave)."""
     from lc0_amd import kernels as K
     from oracle import fp8
     rng = np.random.default_rng(m + n + k)
