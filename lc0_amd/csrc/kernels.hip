@@ -924,7 +924,7 @@ void LaunchGemmDmaStaged(const GemmArgs& a, hipStream_t stream) {
   LaunchGemmDma<BM, BN, BK, WAVES_M, WAVES_N, 2>(a, stream);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BKB = 128>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKB = 128, int NSTAGES = 2>
 void LaunchGemmDmaF8(const GemmF8Args& a, hipStream_t stream) {
   dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, 1);
   const dim3 block(WAVES_M * WAVES_N * 64);
@@ -941,10 +941,26 @@ void LaunchGemmDmaF8(const GemmF8Args& a, hipStream_t stream) {
     }
   }
   if (a.out_f8) {
-    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, uint8_t>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, uint8_t, false, 0, NSTAGES>), grid,
+                       block, 0, stream, a);
   } else {
-    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, half_t>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, half_t, false, 0, NSTAGES>), grid,
+                       block, 0, stream, a);
   }
+}
+
+// Stage count by the launch's workgroup count, as LaunchGemmDmaStaged does for fp16 operands.
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+void LaunchGemmDmaF8Staged(const GemmF8Args& a, hipStream_t stream) {
+  constexpr int kStage = (BM + BN) * 128, kLds = 160 * 1024, kCus = 256;
+  const long long wgs = (long long)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  if constexpr (4 * kStage + 4096 <= kLds) {
+    if (wgs <= (long long)kCus * (kLds / (4 * kStage + 4096))) return LaunchGemmDmaF8<BM, BN, WAVES_M, WAVES_N, 128, 4>(a, stream);
+  }
+  if constexpr (3 * kStage + 4096 <= kLds) {
+    if (wgs <= (long long)kCus * (kLds / (3 * kStage + 4096))) return LaunchGemmDmaF8<BM, BN, WAVES_M, WAVES_N, 128, 3>(a, stream);
+  }
+  LaunchGemmDmaF8<BM, BN, WAVES_M, WAVES_N, 128, 2>(a, stream);
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
@@ -1221,10 +1237,16 @@ bool GemmF8TakesRowPanels(const GemmF8Args& a) {
 
 int PickGemmF8Variant(const GemmF8Args& a) {
   if (g_variant_override >= 0 && (g_variant_override <= 2 || g_variant_override == kDma128x128 ||
-                                  g_variant_override == kDma128x64 || g_variant_override == kRowPanel)) {
+                                  g_variant_override == kDma128x64 || g_variant_override == kRowPanel ||
+                                  g_variant_override == kDma64x64)) {
     return g_variant_override;
   }
   if (GemmF8TakesRowPanels(a)) return kRowPanel;
+  // A few hundred rows: small tiles with three or four stages in flight, as for fp16 operands.
+  if (a.M < 1024 && a.N >= 64) {
+    const long long wg128 = (long long)((a.M + 127) / 128) * ((a.N + 63) / 64);
+    return wg128 >= 192 ? kDma128x64 : kDma64x64;
+  }
   auto rounds = [&](int bm, int bn) {
     const long long tiles = (long long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn);
     return (double)((tiles + 255) / 256);
@@ -1253,6 +1275,7 @@ const char* GemmF8VariantName(const GemmF8Args& a) {
     case 2: return "gemm_f8_256x128x128";
     case kDma128x64: return "gemm_f8_128x64x128";
     case kRowPanel: return "gemm_f8_rowpanel";
+    case kDma64x64: return "gemm_f8_64x64x128";
     default: return "gemm_f8_128x128x128";
   }
 }
@@ -1263,9 +1286,10 @@ void LaunchGemmF8(const GemmF8Args& a, hipStream_t stream) {
     case 0: LaunchGemmDmaF8<256, 256, 2, 4>(a, stream); break;
     case 1: LaunchGemmDmaF8<256, 192, 4, 2>(a, stream); break;
     case 2: LaunchGemmDmaF8<256, 128, 4, 2>(a, stream); break;
-    case kDma128x64: LaunchGemmDmaF8<128, 64, 2, 2>(a, stream); break;
+    case kDma128x64: LaunchGemmDmaF8Staged<128, 64, 2, 2>(a, stream); break;
+    case kDma64x64: LaunchGemmDmaF8Staged<64, 64, 2, 2>(a, stream); break;
     case kRowPanel: LaunchGemmF8RowPanel(a, stream); break;
-    default: LaunchGemmDmaF8<128, 128, 2, 2>(a, stream); break;
+    default: LaunchGemmDmaF8Staged<128, 128, 2, 2>(a, stream); break;
   }
 }
 

@@ -316,7 +316,7 @@ def test_quantize_f8_bit_exact():
         np.testing.assert_array_equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 5, 6, 7])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 5, 6, 7, 10])
 @pytest.mark.parametrize("m,n,k", [(512, 512, 128), (300, 200, 256), (2048, 1536, 1024), (64, 3072, 1024), (1, 17, 128),
                                    (64, 1024, 1536), (64, 1536, 1024), (5, 8192, 256), (700, 40, 4096)])
 def test_gemm_f8_vs_exact_product(variant, m, n, k):
