@@ -282,8 +282,8 @@ struct ModelState {
   float alpha_ = 1.0f, eps_ = 1e-6f;
   bool fold_layer_norm_ = false;
   bool fused_smolgen_attention_ = true;
-  int fused_smolgen_min_batch_ = 96;
-  int dense1_split_min_batch_ = 64;   // smallest batch whose smolgen dense1 splits K between workgroups
+  int fused_smolgen_min_batch_ = 72;
+  int dense1_split_min_batch_ = 112;   // smallest batch whose smolgen dense1 splits K between workgroups
   bool qkv_first_ = true;
   half_t* smolgen_wfrag_ = nullptr;   // smolgen_w in the fragment order of smolgen_attention_kernel (null: not fused)
   bool any_smolgen_ = false;
@@ -874,17 +874,18 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   // samples and a quarter of the queries, and its two phases do not overlap: at fewer positions than fill the CUs the
   // separate GEMM and attention kernels are faster; 15x1024 net: batch 128 +4 %, 256 +1.5 %, 1024 +2 %, 64 -1 %, 16 -6 %).
   fused_smolgen_attention_ = options.GetBool("fused_smolgen_attention", true);
-  fused_smolgen_min_batch_ = options.GetInt("fused_smolgen_min_batch", 96);
-  dense1_split_min_batch_ = options.GetInt("dense1_split_min_batch", 64);
+  fused_smolgen_min_batch_ = options.GetInt("fused_smolgen_min_batch", 72);
+  dense1_split_min_batch_ = options.GetInt("dense1_split_min_batch", 112);
   qkv_first_ = options.GetBool("qkv_first", true);
   fp8_fp16_layers_ = options.GetInt("fp8_fp16_layers", 0);
   if (fp8_fp16_layers_ < 0) throw Error("fp8_fp16_layers must not be negative.");
   use_graphs_ = options.GetBool("graphs", true);
   // Running the smolgen chain beside the QKV projection costs two cross-queue dependencies per layer; below
-  // these batch sizes the chain on the main stream is faster (measured on the 15x1024 net: fp16 batch 1
-  // 1.81 -> 1.73 ms, fp8 batch 16 1.69 -> 1.57 ms; from batch 4 / 64 up the overlap wins).
+  // this batch size the chain on the main stream is faster (measured on the 15x1024 net, chain on the main stream
+  // against beside the projection: fp16 batch 8 1.26 against 1.45 ms, batch 64 2.50 against 2.53, batch 96 3.43
+  // against 3.24; fp8 batch 64 2.00 against 2.25, batch 96 2.60 against 2.54).
   overlap_min_batch_ = options.GetInt("overlap_min_batch", -1);
-  if (overlap_min_batch_ < 0) overlap_min_batch_ = fp8_ ? 48 : 2;
+  if (overlap_min_batch_ < 0) overlap_min_batch_ = 80;
   heads_overlap_min_batch_ = options.GetInt("heads_overlap_min_batch", -1);
   lane_count_ = options.GetInt("lanes", 4);
   if (lane_count_ < 1 || lane_count_ > 8) throw Error("lanes must be in 1..8.");

@@ -85,8 +85,8 @@ class Mi355xNetwork : public Network {
     add("overlap_min_batch", std::to_string(options.GetOrDefault<int>("overlap_min_batch", -1)));
     add("heads_overlap_min_batch", std::to_string(options.GetOrDefault<int>("heads_overlap_min_batch", -1)));
     add("fused_smolgen_attention", options.GetOrDefault<bool>("fused_smolgen_attention", true) ? "true" : "false");
-    add("fused_smolgen_min_batch", std::to_string(options.GetOrDefault<int>("fused_smolgen_min_batch", 96)));
-    add("dense1_split_min_batch", std::to_string(options.GetOrDefault<int>("dense1_split_min_batch", 64)));
+    add("fused_smolgen_min_batch", std::to_string(options.GetOrDefault<int>("fused_smolgen_min_batch", 72)));
+    add("dense1_split_min_batch", std::to_string(options.GetOrDefault<int>("dense1_split_min_batch", 112)));
     add("fold_layer_norm", options.GetOrDefault<bool>("fold_layer_norm", false) ? "true" : "false");
     const std::string precision = options.GetOrDefault<std::string>("precision", "fp16");
     add("precision", precision);

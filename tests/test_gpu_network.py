@@ -85,7 +85,7 @@ def test_attention_nets_match_oracle(name, batch, positions):
 @pytest.mark.parametrize("name,batch,options", [("tiny_attn", 37, ""), ("c2_bt4_15x1024", 33, ""),
                                                 ("tiny_attn_f8", 21, "precision=fp8,")])
 def test_smolgen_generator_inside_attention_and_as_a_gemm_of_its_own(name, batch, options, positions):
-    """The shared smolgen_w layer (network_blas.cc:332-347) runs inside the attention kernel (by default from 96
+    """The shared smolgen_w layer (network_blas.cc:332-347) runs inside the attention kernel (by default from 72
     positions up, here forced) and as a separate GEMM with fused_smolgen_attention=false: both against the oracle,
     and the profile names which ran."""
     path = netgen.cached_config(name)
