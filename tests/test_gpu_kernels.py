@@ -127,6 +127,27 @@ def test_row_panel_gemm_panel_shapes_and_reduction_tails(m, n, k):
     np.testing.assert_allclose(got16, onn.fc(a, w.reshape(-1), np.zeros(n, f32), nr.ACT_NONE), rtol=2e-3, atol=2e-3)
 
 
+def test_gemm_automatic_choice_over_random_shapes():
+    """The launcher picks the kernel by shape (row panels of five sizes, direct-to-LDS tiles of seven with two to four
+    stages, register-staged tiles): sixty seeded shapes between 1x1x8 and 6000x4000x4096, ragged in every dimension,
+    against FullyConnectedLayer::Forward1D (blas/fully_connected_layer.cc:49-106)."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(2718)
+    for case in range(60):
+        m = int(rng.choice([1, 3, 16, 17, 64, 100, 192, 256, 500, 1024, 3000, 6000]))
+        n = int(rng.choice([1, 8, 31, 32, 64, 130, 256, 1000, 1024, 1858, 3072, 4000]))
+        k = int(rng.choice([8, 24, 64, 128, 200, 256, 512, 1000, 1024, 1536, 4096]))
+        if m * n * k > 6000 * 1024 * 1536:
+            continue
+        a = _h(rng.standard_normal((m, k)) * 0.5)
+        w = _h(rng.standard_normal((n, k)) * (2.0 / np.sqrt(k)))
+        b = rng.standard_normal(n).astype(f32)
+        act = [nr.ACT_NONE, nr.ACT_MISH, nr.ACT_RELU][case % 3]
+        want = onn.fc(a, w.reshape(-1), b, act)
+        got = K.gemm(a, w, b, act=act).astype(f32)
+        np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3, err_msg="shape %dx%dx%d" % (m, n, k))
+
+
 def test_row_panel_gemm_batched_with_scale():
     from lc0_amd import kernels as K
     rng = np.random.default_rng(11)
