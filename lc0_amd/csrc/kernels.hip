@@ -1102,7 +1102,9 @@ GemmVariant PickGemmVariant(const GemmArgs& a) {
   // The same holds for a handful of rows with thousands of columns, as long as panels of at most 32x32 cover them
   // with one workgroup per CU (1x8192x256: 2.9 vs 5.0 us).
   const long long tiles64 = (long long)((a.M + 63) / 64) * ((a.N + 63) / 64) * a.batch;
-  if (a.split_k == 1 && a.K >= 256 && (tiles64 <= 64 || RowPanelWorkgroups(a, kRowPanelShapes[3]) <= kRowPanelWorkgroups)) {
+  if (a.split_k == 1 && a.K >= 256 &&
+      (tiles64 <= 64 || (a.M <= 128 && tiles64 <= 128) ||
+       RowPanelWorkgroups(a, kRowPanelShapes[3]) <= kRowPanelWorkgroups)) {
     return kRowPanel;
   }
   // A few hundred rows (3 to 12 positions), or few columns: too small for the cost model above, too large for row
