@@ -285,6 +285,7 @@ struct ModelState {
   int fused_smolgen_min_batch_ = 72;
   int dense1_split_min_batch_ = 112;   // smallest batch whose smolgen dense1 splits K between workgroups
   bool qkv_first_ = true;
+  int chain_latency_max_batch_ = 128;   // largest fp16 batch whose smolgen chain takes the shortest-latency GEMM variants
   half_t* smolgen_wfrag_ = nullptr;   // smolgen_w in the fragment order of smolgen_attention_kernel (null: not fused)
   bool any_smolgen_ = false;
   // Dense position encoding (PE_DENSE nets): preprocessing layer, embedding layer norm and
@@ -624,7 +625,7 @@ bool Mi355xNetwork::CanFoldLayerNorms(int B) const {
   cons.row_stats = any_f; cons.row_parts = 1; cons.norm_n = emb_;
   NormFold prod;
   prod.skip = any_h; prod.ldskip = emb_; prod.stats_out = ln_stats_a_; prod.norm_n = emb_;
-  const bool chain_first = B <= 128;
+  const bool chain_first = B <= chain_latency_max_batch_;
   if (!GemmSupportsNormFolding(MakeGemmArgs(x_, emb_, e.qkv_n, qkv_, 3 * d_model_, T, kActNone, false, 1, false, &cons)) ||
       !GemmSupportsNormFolding(MakeGemmArgs(x_, emb_, e.ffn1_n, ffn_, dff_, T, ffn_act_, false, 1, false, &cons)) ||
       !GemmSupportsNormFolding(MakeGemmArgs(att_, d_model_, e.dense, x_, emb_, T, kActNone, false, 1, false, &prod)) ||
@@ -877,6 +878,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   fused_smolgen_min_batch_ = options.GetInt("fused_smolgen_min_batch", 72);
   dense1_split_min_batch_ = options.GetInt("dense1_split_min_batch", 112);
   qkv_first_ = options.GetBool("qkv_first", true);
+  chain_latency_max_batch_ = options.GetInt("chain_latency_max_batch", 128);
   fp8_fp16_layers_ = options.GetInt("fp8_fp16_layers", 0);
   if (fp8_fp16_layers_ < 0) throw Error("fp8_fp16_layers must not be negative.");
   use_graphs_ = options.GetBool("graphs", true);
@@ -1660,7 +1662,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       // The chain is the critical path of this phase when the QKV projection beside it is short (e4m3 operands,
       // or at most 128 positions): its kernels then take the variants with the shortest latency. At larger fp16
       // batches the two are balanced and the leaner variants disturb the projection less (batch 256: 1.5 %).
-      const bool chain_first = f8 || B <= 128;
+      const bool chain_first = f8 || B <= chain_latency_max_batch_;
       Gemm("gemm_smolgen_compress", x_, emb_, norm_in ? e.sg_compress_n : e.sg_compress, sg1_, sg_hc_, T, kActNone,
            false, ss, 1, chain_first, norm_in ? &cons_in : nullptr);
       // dense1 has a long reduction and few outputs. With few rows one workgroup per 16x16 outputs splits K over

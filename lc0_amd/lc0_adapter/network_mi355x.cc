@@ -87,6 +87,7 @@ class Mi355xNetwork : public Network {
     add("fused_smolgen_attention", options.GetOrDefault<bool>("fused_smolgen_attention", true) ? "true" : "false");
     add("fused_smolgen_min_batch", std::to_string(options.GetOrDefault<int>("fused_smolgen_min_batch", 72)));
     add("dense1_split_min_batch", std::to_string(options.GetOrDefault<int>("dense1_split_min_batch", 112)));
+    add("chain_latency_max_batch", std::to_string(options.GetOrDefault<int>("chain_latency_max_batch", 128)));
     add("fold_layer_norm", options.GetOrDefault<bool>("fold_layer_norm", false) ? "true" : "false");
     const std::string precision = options.GetOrDefault<std::string>("precision", "fp16");
     add("precision", precision);
