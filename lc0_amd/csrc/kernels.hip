@@ -885,14 +885,17 @@ void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
   const dim3 block(WAVES_M * WAVES_N * 64);
   auto launch = [&](auto stream_tag) {
     constexpr bool S = decltype(stream_tag)::value;
+    // The folded-layer-norm epilogues exist with two stages only (LaunchGemmDmaStaged sends them there).
     if (a.skip != nullptr) {
-      if constexpr ((BN / WAVES_N) % 64 == 0 || BN / WAVES_N == 32) {
-        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 2, NSTAGES>), grid, block, 0,
+      if constexpr (((BN / WAVES_N) % 64 == 0 || BN / WAVES_N == 32) && NSTAGES == 2) {
+        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 2, 2>), grid, block, 0,
                            stream, a);
       }
     } else if (a.row_stats != nullptr) {
-      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 1, NSTAGES>), grid, block, 0,
-                         stream, a);
+      if constexpr (NSTAGES == 2) {
+        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 1, 2>), grid, block, 0,
+                           stream, a);
+      }
     } else {
       hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 0, NSTAGES>), grid, block, 0,
                          stream, a);
@@ -915,6 +918,7 @@ template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 void LaunchGemmDmaStaged(const GemmArgs& a, hipStream_t stream) {
   constexpr int kStage = (BM + BN) * BK * 2, kLds = 160 * 1024, kCus = 256;
   const long long wgs = (long long)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN) * a.batch;
+  if (a.skip != nullptr || a.row_stats != nullptr) return LaunchGemmDma<BM, BN, BK, WAVES_M, WAVES_N, 2>(a, stream);
   if constexpr (4 * kStage + 4096 <= kLds) {
     if (wgs <= (long long)kCus * (kLds / (4 * kStage + 4096))) return LaunchGemmDma<BM, BN, BK, WAVES_M, WAVES_N, 4>(a, stream);
   }
