@@ -182,17 +182,22 @@ __global__ void winograd_output_transform_kernel(const MT* __restrict__ m, const
 }
 
 // Same for C <= 256 with four times the parallelism: one thread per (tile, channel),
-// blockDim.x == 4 * C. Shared memory: part[4][C] | hidden[K] | gate[2][C] floats.
+// blockDim.x == 4 * C. Shared memory: part[4][C] | hidden[K] | fc2[4][2][C] floats.
+// The squeeze-and-excitation layers sit on the critical path of every workgroup (nothing moves through memory while
+// they run), so they are spread over all threads: every wave pools the channels it needs itself, the second layer is
+// split four ways over k with the weights of a thread's share asked for at once, and every thread adds the four
+// partial sums of its own channel.
 template <typename T, typename MT>
-__global__ __launch_bounds__(1024) void winograd_output_transform_tiles_kernel(
+// (eight waves per SIMD, i.e. two workgroups of 1024 threads per CU: at most 64 registers)
+__global__ __launch_bounds__(1024, 8) void winograd_output_transform_tiles_kernel(
     const MT* __restrict__ m, const float* __restrict__ bias, const T* skip, const float* __restrict__ se_w1,
     const float* __restrict__ se_b1, const float* __restrict__ se_w2, const float* __restrict__ se_b2, int se_k,
     T* out, T* __restrict__ v_next, int ldv, int batch, int C, int act) {
   extern __shared__ float shm[];
   float* part = shm;               // [4][C], then pool[C] in its first row
   float* hidden = shm + 4 * C;     // [K]
-  float* gate = hidden + se_k;     // gamma[C] | beta[C]
-  T* xs = reinterpret_cast<T*>(gate + 2 * C + ((se_k & 1) ? 1 : 0));   // [64][C] activations for the fused input transform
+  float* fc2 = hidden + se_k;      // [4][gamma | beta][C] partial sums of the second layer
+  T* xs = reinterpret_cast<T*>(fc2 + 8 * C + ((se_k & 1) ? 1 : 0));   // [64][C] activations for the fused input transform
   const int b = blockIdx.x;
   const int tile = threadIdx.x / C, c = threadIdx.x - tile * C;
   const long long kstride = (long long)batch * 4 * C;
@@ -225,32 +230,60 @@ __global__ __launch_bounds__(1024) void winograd_output_transform_tiles_kernel(
   if (se_k > 0) {
     part[tile * C + c] = sum;
     __syncthreads();
-    if (tile == 0) part[c] = (part[c] + part[C + c] + part[2 * C + c] + part[3 * C + c]) * (1.0f / 64.0f) + bc;
-    __syncthreads();
-    // hidden[k] = act(w1[k] . pool + b1[k]): one wave per k, lanes stride over the channels.
+    // hidden[k] = act(w1[k] . pool + b1[k]): one wave per k, lanes stride over the channels (pooled on the way).
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-    for (int k = wave; k < se_k; k += nwaves) {
-      const float* w = se_w1 + (long long)k * C;
-      float h = 0.0f;
-      for (int i = lane; i < C; i += 64) h += w[i] * part[i];
+    constexpr int kMaxPerLane = 4;   // C <= 256
+    float pool[kMaxPerLane];
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) h += __shfl_xor(h, off, 64);
-      if (lane == 0) hidden[k] = RActivate(h + se_b1[k], act);
+    for (int q = 0; q < kMaxPerLane; q++) {
+      const int i = lane + 64 * q;
+      pool[q] = i < C ? (part[i] + part[C + i] + part[2 * C + i] + part[3 * C + i]) * (1.0f / 64.0f) + bias[i] : 0.0f;
     }
-    __syncthreads();
-    if (tile == 0) {
-      float sg = se_b2[c], sb = se_b2[C + c];
-      for (int k = 0; k < se_k; k++) {
-        sg += se_w2[(long long)k * 2 * C + c] * hidden[k];
-        sb += se_w2[(long long)k * 2 * C + C + c] * hidden[k];
+    for (int k0 = wave; k0 < se_k; k0 += 2 * nwaves) {   // two k per round: their weights are asked for together
+      float w[2][kMaxPerLane];
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        const int k = min(k0 + u * nwaves, se_k - 1);
+#pragma unroll
+        for (int q = 0; q < kMaxPerLane; q++) w[u][q] = se_w1[(long long)k * C + min(lane + 64 * q, C - 1)];
       }
-      const float gm = 1.0f / (1.0f + __expf(-sg));
-      gate[c] = gm;
-      gate[C + c] = sb + gm * bc;
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        const int k = k0 + u * nwaves;
+        float h = 0.0f;
+#pragma unroll
+        for (int q = 0; q < kMaxPerLane; q++) h += w[u][q] * pool[q];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) h += __shfl_xor(h, off, 64);
+        if (lane == 0 && k < se_k) hidden[k] = RActivate(h + se_b1[k], act);
+      }
     }
     __syncthreads();
-    gamma = gate[c];
-    beta = gate[C + c];
+    // Second layer: this thread's share is k = tile, tile + 4, ...
+    float sg = 0.0f, sb = 0.0f;
+    for (int k0 = tile; k0 < se_k; k0 += 16) {
+      float wg[4], wb[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int k = min(k0 + 4 * u, se_k - 1);
+        wg[u] = se_w2[(long long)k * 2 * C + c];
+        wb[u] = se_w2[(long long)k * 2 * C + C + c];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int k = k0 + 4 * u;
+        const float h = k < se_k ? hidden[k] : 0.0f;
+        sg += wg[u] * h;
+        sb += wb[u] * h;
+      }
+    }
+    fc2[(tile * 2) * C + c] = sg;
+    fc2[(tile * 2 + 1) * C + c] = sb;
+    __syncthreads();
+    sg = se_b2[c] + ((fc2[c] + fc2[2 * C + c]) + (fc2[4 * C + c] + fc2[6 * C + c]));
+    sb = se_b2[C + c] + ((fc2[C + c] + fc2[3 * C + c]) + (fc2[5 * C + c] + fc2[7 * C + c]));
+    gamma = 1.0f / (1.0f + __expf(-sg));
+    beta = sb + gamma * bc;
   }
   const int ty = (tile >> 1) * 4, tx = (tile & 1) * 4;
   const T* sk = skip ? skip + (long long)b * 64 * C + c : nullptr;
@@ -362,7 +395,7 @@ void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip
   if (batch <= 0) return;
   const int k = se_k > 0 ? se_k : 0;
   if (C <= 256 && C % 16 == 0) {   // 4 * C threads in whole waves (the SE reduction shuffles across a wave)
-    size_t shm = sizeof(float) * (size_t)(6 * C + k + (k & 1));
+    size_t shm = sizeof(float) * (size_t)(12 * C + k + (k & 1));
     if (v_next) shm += sizeof(T) * 64 * (size_t)C;
     hipLaunchKernelGGL((winograd_output_transform_tiles_kernel<T, MT>), dim3(batch), dim3(4 * C), shm, stream, m, bias,
                        skip, se_w1, se_b1, se_w2, se_b2, se_k, out, v_next, ldv_next, batch, C, act);
@@ -375,7 +408,7 @@ void LaunchWinogradOutputTransform(const MT* m, const float* bias, const T* skip
 }
 // The fused kernel needs 4 * C threads and its staging area in the 64 KiB of dynamic LDS.
 bool WinogradFusedInputTransform(int C, int elem_size, int se_k) {
-  return C <= 256 && C % 16 == 0 && sizeof(float) * (6 * C + se_k + 1) + (size_t)elem_size * 64 * C <= 64 * 1024;
+  return C <= 256 && C % 16 == 0 && sizeof(float) * (12 * C + se_k + 1) + (size_t)elem_size * 64 * C <= 64 * 1024;
 }
 
 template void LaunchWinogradOutputTransform<half_t, half_t>(const half_t*, const float*, const half_t*, const float*,
