@@ -243,10 +243,14 @@ def main():
         g = groups.get(variant, Agg(variant, 0.0, 0, 0.0, 0.0))
         groups[variant] = Agg(variant, g.ms + k.ms, g.launches + k.launches, g.flops + k.flops, g.bytes + k.bytes)
     dom = max(groups.values(), key=lambda g: g.ms)
-    if dom.flops > 0:
+    peak = (PEAK_FP8_TFLOPS if dom.name.startswith("gemm_f8") else
+            PEAK_FP32_TFLOPS if dom.name.startswith("gemm_f32") else PEAK_FP16_TFLOPS)
+    # A matrix kernel is priced against the MFMA peak only when its flops per algorithmic byte lie above the ridge
+    # point peak flops / peak bandwidth (fp16: 312 flop/B); below it the memory roofline is the one that bounds it
+    # (the 36 batched winograd-domain GEMMs of a 256-filter convolution: 121 flop/B).
+    mfma_bound = dom.flops > 0 and (dom.bytes <= 0 or dom.flops / dom.bytes >= peak * 1e12 / (PEAK_HBM_GBS * 1e9))
+    if mfma_bound:
         achieved = dom.flops / dom.launches / (dom.ms / dom.launches * 1e-3) / 1e12
-        peak = (PEAK_FP8_TFLOPS if dom.name.startswith("gemm_f8") else
-                PEAK_FP32_TFLOPS if dom.name.startswith("gemm_f32") else PEAK_FP16_TFLOPS)
         roofline = {"bound": "mfma", "kernel": dom.name, "achieved": achieved, "peak": peak,
                     "unit": "TFLOP/s", "frac": achieved / peak, "traffic": None,
                     "avg_launch_ms": dom.ms / dom.launches, "launches_per_step": dom.launches // prof_iters}
