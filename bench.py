@@ -186,32 +186,43 @@ def main():
     io_legal_ms = timed_blocking(comp_legal)
     comp_legal.close()
 
-    # Two search threads, each with its own computation in flight on the shared network (host I/O included):
-    # how lc0 drives a backend (backendbench.cc:177-184 does the same with --threads).
+    # Two and four search threads, each with its own computation in flight on the shared network (host I/O
+    # included): how lc0 drives a backend (backendbench.cc:177-184 does the same with --threads). Passes of
+    # different lanes overlap on the GPU, so the aggregate rate is above that of one computation at a time.
     import threading
-    comp2 = net.NewComputation()
-    comp2.AddInputs(masks[:batch], values[:batch])
-    comp2.ComputeBlocking()
-    gate = threading.Barrier(3)
 
-    def search_thread(c):
-        for _ in range(2):
+    def threads_ms(n_threads):
+        comps = [comp]
+        for _ in range(n_threads - 1):
+            c = net.NewComputation()
+            c.AddInputs(masks[:batch], values[:batch])
             c.ComputeBlocking()
-        gate.wait()
-        for _ in range(io_iters):
-            c.ComputeBlocking()
-        gate.wait()
+            comps.append(c)
+        gate = threading.Barrier(n_threads + 1)
 
-    workers = [threading.Thread(target=search_thread, args=(c,)) for c in (comp, comp2)]
-    for w in workers:
-        w.start()
-    gate.wait()
-    t0 = time.perf_counter()
-    gate.wait()
-    two_threads_ms = (time.perf_counter() - t0) * 1e3 / io_iters
-    for w in workers:
-        w.join()
-    comp2.close()
+        def search_thread(c):
+            for _ in range(2):
+                c.ComputeBlocking()
+            gate.wait()
+            for _ in range(io_iters):
+                c.ComputeBlocking()
+            gate.wait()
+
+        workers = [threading.Thread(target=search_thread, args=(c,)) for c in comps]
+        for w in workers:
+            w.start()
+        gate.wait()
+        t0 = time.perf_counter()
+        gate.wait()
+        ms = (time.perf_counter() - t0) * 1e3 / io_iters
+        for w in workers:
+            w.join()
+        for c in comps[1:]:
+            c.close()
+        return ms
+
+    two_threads_ms = threads_ms(2)
+    four_threads_ms = threads_ms(4)
 
     # Timed region: K device passes over the resident batch, bracketed by stream
     # synchronisation on both sides (inside TimeResidentForward) and by the host clock.
@@ -278,6 +289,7 @@ def main():
         "with_host_io_evals_per_s": batch / (io_ms * 1e-3),
         "with_host_io_legal_policy_evals_per_s": batch / (io_legal_ms * 1e-3),
         "with_host_io_two_threads_evals_per_s": 2 * batch / (two_threads_ms * 1e-3),
+        "with_host_io_four_threads_evals_per_s": 4 * batch / (four_threads_ms * 1e-3),
         "all_gemm_attention": {"ms_per_step": gemm_ms, "tflops": gemm_flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None,
                                "frac_of_mfma_peak": gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS if gemm_ms else None},
         "kernel_ms_per_step": {k.name: round(k.ms / prof_iters, 4) for k in kernels},
