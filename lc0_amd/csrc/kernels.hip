@@ -663,6 +663,22 @@ void gemm_dma_kernel(Args p) {
           for (int j = 0; j < TN; j++)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[i][j], 0, 0, 0);
       }
+      if constexpr ((BM / WAVES_M / 32) * (BN / WAVES_N / 32) >= (BM / WAVES_M / 32) + (BN / WAVES_N / 32) && EPI == 0) {
+        // Order of the k-tile's 32 MFMAs and 24 fragment reads: the reads of a k-step one by one between the MFMAs
+        // of the step before it.
+        constexpr int KS = BKB / 32, RD = TM + TN, MF = TM * TN;
+        __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);
+#pragma unroll
+        for (int ks = 0; ks + 1 < KS; ks++) {
+#pragma unroll
+          for (int q = 0; q < RD; q++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, MF - RD, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, MF, 0);
+      }
     }
   }
 
