@@ -110,6 +110,12 @@ int lc0mi_net_time_resident_forward(lc0mi_net* net, int batch, int iters, double
  * itself on built-in pseudo-positions; this call replaces those scales with ones derived from n
  * caller-supplied positions (same packed planes as lc0mi_comp_add_inputs). */
 int lc0mi_net_calibrate_fp8(lc0mi_net* net, int n, const uint64_t* masks, const float* values);
+/* The activation scales in use (value = code x scale), seven floats per encoder layer: the operands of the Q/K/V,
+ * attention-output, FFN1 and FFN2 layers, then of smolgen's first dense layer, second dense layer and generator
+ * (1 where an operand stays in fp16). Writes at most cap floats and returns the number there are, -1 on error.
+ * No counterpart in the reference (it has no fp8 arithmetic of its own); used to check the fp8 pass against an
+ * emulation of the same arithmetic. */
+int lc0mi_net_fp8_scales(const lc0mi_net* net, float* out, int cap);
 
 /* ---- decoded weights (host only, needs no GPU) ----
  * What the library reads from a weights file, for checking the loader: LayerAdapter decoding of the four

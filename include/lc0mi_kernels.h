@@ -44,7 +44,7 @@ int lc0mi_k_gemm_norm_consumer(const uint16_t* U, int ldu, const uint16_t* W, in
                                int act, int latency_first, uint16_t* C, int ldc, int time_iters, double* ms);
 /* Forces the GEMM tile variant of subsequent calls (-1 automatic; 0 256x256x64,
  * 1 256x192x64, 2 256x128x32 direct-to-LDS kernels, 3 128x128x64, 4 64x64x64, 5 direct-to-LDS 128x128x64,
- * 6 row panels of 16x16 to 64x32 outputs, 7 direct-to-LDS 128x64x64, 8 persistent 256x256x64, 9 direct-to-LDS
+ * 6 row panels of 16x16 to 64x32 outputs, 7 direct-to-LDS 128x64x64, 8 unused (automatic choice), 9 direct-to-LDS
  * 128x32x64, 10 direct-to-LDS 64x64x64). */
 int lc0mi_k_set_gemm_variant(int variant);
 /* float variant (fp32 configuration). */

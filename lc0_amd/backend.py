@@ -68,6 +68,7 @@ def load_library():
     lib.lc0mi_net_take_profile.argtypes = [vp, C.c_char_p, ci]
     lib.lc0mi_net_time_resident_forward.argtypes = [vp, ci, ci, C.POINTER(C.c_double)]
     lib.lc0mi_net_calibrate_fp8.argtypes = [vp, ci, vp, vp]
+    lib.lc0mi_net_fp8_scales.argtypes = [vp, vp, ci]
     lib.lc0mi_weights_list.argtypes = [vp, C.c_size_t, C.c_char_p, ci]
     lib.lc0mi_weights_tensor.argtypes = [vp, C.c_size_t, C.c_char_p, vp, C.c_longlong]
     lib.lc0mi_weights_tensor.restype = C.c_longlong
@@ -197,6 +198,18 @@ class Network:
         if masks.shape != values.shape or masks.ndim != 2 or masks.shape[1] != 112:
             raise BackendError("masks and values must both be [n, 112]")
         _check(load_library().lc0mi_net_calibrate_fp8(self._h, masks.shape[0], masks.ctypes.data, values.ctypes.data))
+
+    def Fp8Scales(self):
+        """precision=fp8: float32 [layers, 7], the activation scales of the operands of Q/K/V, attention output,
+        FFN1, FFN2 and of smolgen's first dense, second dense and generator layers (1 where unused)."""
+        import numpy as np
+        lib = load_library()
+        n = lib.lc0mi_net_fp8_scales(self._h, None, 0)
+        if n < 0:
+            raise BackendError(lib.lc0mi_last_error().decode())
+        out = np.zeros(n, np.float32)
+        lib.lc0mi_net_fp8_scales(self._h, out.ctypes.data, n)
+        return out.reshape(-1, 7)
 
     def TimeResidentForward(self, batch, iters):
         ms = C.c_double()

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "liblc0mi.so")
-SOURCES = ["weights.cc", "tables.cc", "network.cc", "capi.cc", "kernel_api.cc", "kernels.hip", "gemm_persistent.hip", "smolgen_attention.hip", "resnet_kernels.hip"]
+SOURCES = ["weights.cc", "tables.cc", "network.cc", "capi.cc", "kernel_api.cc", "kernels.hip", "gemm_kernels.hip", "smolgen_attention.hip", "resnet_kernels.hip"]
 # -packed-fp32-ops off: packed fp32 forms are not trusted on this hardware pool.
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result", "-Wno-unknown-warning-option"]

@@ -226,6 +226,17 @@ int lc0mi_net_calibrate_fp8(lc0mi_net* net, int n, const uint64_t* masks, const 
   });
 }
 
+int lc0mi_net_fp8_scales(const lc0mi_net* net, float* out, int cap) {
+  int needed = -1;
+  Guard([&] {
+    if (!net) throw lc0mi::Error("null network");
+    const std::vector<float> v = net->impl->Fp8Scales();
+    if (out != nullptr && cap > 0) std::memcpy(out, v.data(), sizeof(float) * std::min<size_t>(v.size(), static_cast<size_t>(cap)));
+    needed = static_cast<int>(v.size());
+  });
+  return needed;
+}
+
 }  // extern "C"
 
 // ---- decoded weights, for checking the loader without a GPU ----

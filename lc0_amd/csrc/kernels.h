@@ -68,10 +68,6 @@ void LaunchGemm(const GemmArgs& args, hipStream_t stream);
 // epilogue), and the number of partial sums per row a producer launch writes to stats_out.
 bool GemmSupportsNormFolding(const GemmArgs& args);
 int GemmStatsParts(const GemmArgs& args);
-// The persistent 256x256 kernel (gemm_persistent.hip) behind LaunchGemm: whether it takes these arguments, and
-// its launch (stream_stores: write the output with streaming stores).
-bool GemmPersistentSupports(const GemmArgs& args);
-void LaunchGemmPersistent(const GemmArgs& args, bool stream_stores, hipStream_t stream);
 // Name of the kernel variant LaunchGemm picks for these arguments (tile shape).
 const char* GemmVariantName(const GemmArgs& args);
 

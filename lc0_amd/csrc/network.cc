@@ -178,6 +178,10 @@ struct EncoderDev {
   float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
   bool has_smolgen = false;
   Linear sg_compress, sg_dense1, sg_dense2;
+  // Option fp8_gemms=...+smolgen: e4m3 copies of the chain's layers (sg_global8: the shared generator weights with
+  // this layer's activation scale) and the scales of their three operands besides x.
+  LinearF8 sg_compress8, sg_dense18, sg_dense28, sg_global8;
+  float s_sg1 = 1.0f, s_sg2 = 1.0f, s_sg3 = 1.0f;
   float *sg_ln1_g = nullptr, *sg_ln1_b = nullptr, *sg_ln2_g = nullptr, *sg_ln2_b = nullptr;
   // Folded layer norms: the three layers that read normalised rows, with the gamma / beta of the norm before them
   // multiplied in (qkv and sg_compress: the second norm of the previous encoder layer, absent in the first layer;
@@ -311,6 +315,9 @@ struct ModelState {
   // fp8 configuration: the four large GEMMs of every encoder layer run on e4m3 operands.
   bool fp8_ = false;
   bool q_qkv_ = true, q_dense_ = true, q_ffn1_ = true, q_ffn2_ = true;   // option fp8_gemms
+  bool q_smolgen_ = false;   // ... +smolgen: the four layers of the smolgen chain as well
+  uint8_t* smolgen_w8_ = nullptr;        // e4m3 codes of the shared generator layer (rows in SmolgenBiasIndex order)
+  std::vector<float> smolgen_w8_scale_;  // their per-row scales
   int fp8_fp16_layers_ = 0;   // option fp8_fp16_layers: the last that many encoder layers keep fp16 operands
 
   // Residual tower.
@@ -345,6 +352,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   std::vector<KernelTime> TakeProfile() override;
   double TimeResidentForward(int batch, int iters) override;
   void CalibrateFp8(int n, const uint64_t* masks, const float* values) override;
+  std::vector<float> Fp8Scales() const override;
 
   // Used by the computation.
   std::unique_ptr<HostSlot> GetSlot();
@@ -377,8 +385,11 @@ class Mi355xNetwork : public Network, protected ModelState {
   Linear MakeLinearNormFolded(const Vec& w, const Vec& b, const Vec& gamma, const Vec& beta, int out, int in);
   LinearF8 MakeLinearF8(const Vec& w, int out, int in);
   void GemmF8(const char* name, const uint8_t* A, const Linear& lin, const LinearF8& q, void* C, int M, int act,
-              bool out_f8, float out_mul);
-  void RecordAbsMax(const half_t* x, size_t n, int slot);
+              bool out_f8, float out_mul, hipStream_t st = nullptr);
+  void RecordAbsMax(const half_t* x, size_t n, int slot, hipStream_t st = nullptr);
+  // Slot of the calibration maxima: 4 per layer plus the last layer's output, then 3 per layer for the smolgen chain.
+  int SmolgenSlot(size_t li, int which) const { return static_cast<int>(4 * encoders_.size() + 1 + 3 * li + which); }
+  size_t CalibrationSlots() const { return 7 * encoders_.size() + 1; }
   void ApplyCalibration(const std::vector<float>& absmax);
   void CalibrateExclusive(int n, const uint64_t* masks, const float* values);
   void DefaultCalibration();
@@ -431,6 +442,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   bool calibrating_ = false;
   float* d_absmax_ = nullptr;   // [4 * layers + 1] calibration maxima (float bits, non-negative)
   uint8_t *xq_ = nullptr, *attq_ = nullptr, *ffnq_ = nullptr;
+  uint8_t *sg1q_ = nullptr, *sg2q_ = nullptr, *sg3q_ = nullptr;   // e4m3 operands of the smolgen chain
   void *r_in_ = nullptr, *r_x_ = nullptr, *r_y_ = nullptr, *r_v_ = nullptr, *r_m_ = nullptr, *r_h1_ = nullptr,
        *r_h2_ = nullptr;
 
@@ -682,7 +694,8 @@ LinearF8 Mi355xNetwork::MakeLinearF8(const Vec& w, int out, int in) {
 }
 
 void Mi355xNetwork::GemmF8(const char* name, const uint8_t* A, const Linear& lin, const LinearF8& q, void* C, int M,
-                           int act, bool out_f8, float out_mul) {
+                           int act, bool out_f8, float out_mul, hipStream_t st) {
+  if (st == nullptr) st = stream_;
   GemmF8Args g;
   g.A = A; g.lda = lin.in;
   g.W = q.w; g.ldw = lin.in;
@@ -697,11 +710,11 @@ void Mi355xNetwork::GemmF8(const char* name, const uint8_t* A, const Linear& lin
   const double bytes = static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in +
                        static_cast<double>(M) * lin.out * (out_f8 ? 1 : 2);
   const std::string label = std::string(name) + "|" + GemmF8VariantName(g);
-  Timed(label.c_str(), flops, bytes, [&] { LaunchGemmF8(g, stream_); });
+  Timed(label.c_str(), flops, bytes, [&] { LaunchGemmF8(g, st); }, st);
 }
 
-void Mi355xNetwork::RecordAbsMax(const half_t* x, size_t n, int slot) {
-  LaunchAbsMax(x, static_cast<long long>(n), d_absmax_ + slot, stream_);
+void Mi355xNetwork::RecordAbsMax(const half_t* x, size_t n, int slot, hipStream_t st) {
+  LaunchAbsMax(x, static_cast<long long>(n), d_absmax_ + slot, st == nullptr ? stream_ : st);
 }
 
 // Activation scales from the maxima seen during calibration: the largest value maps to
@@ -724,7 +737,26 @@ void Mi355xNetwork::ApplyCalibration(const std::vector<float>& absmax) {
     upload(e.dense8, e.s_att);
     upload(e.ffn18, e.s_x1);
     upload(e.ffn28, e.s_ffn);
+    if (q_smolgen_ && e.has_smolgen) {
+      e.s_sg1 = scale_of(absmax[SmolgenSlot(li, 0)]);
+      e.s_sg2 = scale_of(absmax[SmolgenSlot(li, 1)]);
+      e.s_sg3 = scale_of(absmax[SmolgenSlot(li, 2)]);
+      upload(e.sg_compress8, e.s_x);
+      upload(e.sg_dense18, e.s_sg1);
+      upload(e.sg_dense28, e.s_sg2);
+      upload(e.sg_global8, e.s_sg3);
+    }
   }
+}
+
+// Per layer: the scales of x, attention output, x1, FFN hidden, and of the three smolgen operands (1 when unused).
+std::vector<float> Mi355xNetwork::Fp8Scales() const {
+  if (!fp8_) throw Error("Fp8Scales needs a network created with precision=fp8.");
+  std::vector<float> out;
+  for (const EncoderDev& e : encoders_) {
+    for (float v : {e.s_x, e.s_att, e.s_x1, e.s_ffn, e.s_sg1, e.s_sg2, e.s_sg3}) out.push_back(v);
+  }
+  return out;
 }
 
 void Mi355xNetwork::CalibrateFp8(int n, const uint64_t* masks, const float* values) {
@@ -744,7 +776,7 @@ void Mi355xNetwork::CalibrateFp8(int n, const uint64_t* masks, const float* valu
 void Mi355xNetwork::CalibrateExclusive(int n, const uint64_t* masks, const float* values) {
   std::lock_guard<std::mutex> lock(eval_mutex_);
   HIP_CHECK(hipSetDevice(device_));
-  const size_t slots = 4 * encoders_.size() + 1;
+  const size_t slots = CalibrationSlots();
   std::vector<float> absmax(slots, 0.0f), part(slots);
   for (int done = 0; done < n; done += max_batch_) {
     const int b = std::min(max_batch_, n - done);
@@ -766,6 +798,7 @@ void Mi355xNetwork::CalibrateExclusive(int n, const uint64_t* masks, const float
     calibrating_ = false;
     profiling_ = was_profiling;
     HIP_CHECK(hipStreamSynchronize(stream_));
+    HIP_CHECK(hipStreamSynchronize(side_stream_));
     HIP_CHECK(hipMemcpy(part.data(), d_absmax_, slots * sizeof(float), hipMemcpyDeviceToHost));
     for (size_t i = 0; i < slots; i++) absmax[i] = std::max(absmax[i], part[i]);
   }
@@ -857,7 +890,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   {
     // Which of the four encoder GEMMs use e4m3 operands: names joined by '+'.
     const std::string which = options.GetString("fp8_gemms", "qkv+dense+ffn1+ffn2");
-    q_qkv_ = q_dense_ = q_ffn1_ = q_ffn2_ = false;
+    q_qkv_ = q_dense_ = q_ffn1_ = q_ffn2_ = q_smolgen_ = false;
     size_t pos = 0;
     while (pos <= which.size()) {
       const size_t end = std::min(which.find('+', pos), which.size());
@@ -866,7 +899,8 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
       else if (name == "dense") q_dense_ = true;
       else if (name == "ffn1") q_ffn1_ = true;
       else if (name == "ffn2") q_ffn2_ = true;
-      else if (!name.empty()) throw Error("Unknown name '" + name + "' in fp8_gemms (qkv, dense, ffn1, ffn2).");
+      else if (name == "smolgen") q_smolgen_ = true;
+      else if (!name.empty()) throw Error("Unknown name '" + name + "' in fp8_gemms (qkv, dense, ffn1, ffn2, smolgen).");
       pos = end + 1;
     }
   }
@@ -1044,7 +1078,12 @@ void Mi355xNetwork::AllocActivations() {
     xq_ = static_cast<uint8_t*>(arena_.Alloc(T * emb_));
     attq_ = static_cast<uint8_t*>(arena_.Alloc(T * d_model_));
     ffnq_ = static_cast<uint8_t*>(arena_.Alloc(T * dff_));
-    d_absmax_ = AllocF(4 * encoders_.size() + 1);
+    d_absmax_ = AllocF(CalibrationSlots());
+    if (q_smolgen_ && any_smolgen_) {
+      sg1q_ = static_cast<uint8_t*>(arena_.Alloc(T * sg_hc_));
+      sg2q_ = static_cast<uint8_t*>(arena_.Alloc(static_cast<size_t>(max_batch_) * sg_hs_));
+      sg3q_ = static_cast<uint8_t*>(arena_.Alloc(static_cast<size_t>(max_batch_) * sg_gen_));
+    }
   }
   head1_ = AllocH(T * std::max(val_ch_, mov_ch_));
   head2_ = AllocH(static_cast<size_t>(max_batch_) * std::max(val_fc_, mov_fc_));
@@ -1258,6 +1297,15 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
       e.sg_dense2 = MakeLinear(s.dense2_w, s.dense2_b, gen, hs);
       e.sg_ln1_g = UploadN(s.ln1_gammas, hs, "Smolgen layer norm gamma"); e.sg_ln1_b = UploadN(s.ln1_betas, hs, "Smolgen layer norm beta");
       e.sg_ln2_g = UploadN(s.ln2_gammas, gen, "Smolgen layer norm gamma"); e.sg_ln2_b = UploadN(s.ln2_betas, gen, "Smolgen layer norm beta");
+      if (fp8_ && q_smolgen_) {
+        if ((64 * hc) % 128 || hs % 128 || (gen / heads_) % 128) {
+          throw Error("fp8_gemms=smolgen needs smolgen widths (64 x compression, hidden, generator per head) that are "
+                      "multiples of 128.");
+        }
+        e.sg_compress8 = MakeLinearF8(s.compress, hc, emb_);
+        e.sg_dense18 = MakeLinearF8(s.dense1_w, hs, 64 * hc);
+        e.sg_dense28 = MakeLinearF8(s.dense2_w, gen, hs);
+      }
     }
     if (fold_layer_norm_ && !fp8_ && emb_ % 8 == 0) {
       // Folded layer norms (fp16 path): the layers after a norm get its gamma and beta multiplied in, the layers
@@ -1292,6 +1340,18 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
         std::memcpy(&perm[static_cast<size_t>(SmolgenBiasIndex(q, k)) * g], &w.smolgen_w[static_cast<size_t>(q * 64 + k) * g],
                     sizeof(float) * g);
     smolgen_w_ = MakeLinear(perm, Vec(), 4096, g);
+    if (fp8_ && q_smolgen_) {
+      // One set of codes for all layers; every layer brings the scale of its own operand.
+      LinearF8 shared = MakeLinearF8(perm, 4096, g);
+      smolgen_w8_ = shared.w;
+      smolgen_w8_scale_ = shared.wscale;
+      for (EncoderDev& e : encoders_) {
+        if (!e.has_smolgen) continue;
+        e.sg_global8.w = smolgen_w8_;
+        e.sg_global8.wscale = smolgen_w8_scale_;
+        e.sg_global8.col_scale = AllocF(4096);
+      }
+    }
     if (fused_smolgen_attention_ && SmolgenAttentionSupported(heads_, depth_, g)) {
       // The same weights in the fragment order of the kernel that generates the logits inside the attention.
       std::vector<half_t> frag(w.smolgen_w.size());
@@ -1607,7 +1667,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
   const size_t n_f8_layers = encoders_.size() - std::min<size_t>(encoders_.size(), static_cast<size_t>(fp8_fp16_layers_));
   const size_t nx = static_cast<size_t>(T) * emb_;
   if (calibrating_) RecordAbsMax(x_, nx, 0);
-  if (f8_any && n_f8_layers > 0 && q_qkv_) {
+  if (f8_any && n_f8_layers > 0 && (q_qkv_ || q_smolgen_)) {
     Timed("quantize_f8", 0.0, 3.0 * nx,
           [&] { LaunchQuantizeF8(x_, xq_, static_cast<long long>(nx), 1.0f / encoders_[0].s_x, stream_); });
   }
@@ -1639,7 +1699,9 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     // QKV projection (on the main stream when profiling, for clean per-kernel times).
     hipStream_t ss = (profiling_ || single_stream_ || B < overlap_min_batch_) ? stream_ : side_stream_;
     // The generator layer (smolgen_w) runs inside the attention kernel where that kernel serves the shape.
-    const bool fused_gen = e.has_smolgen && smolgen_wfrag_ != nullptr && B >= fused_smolgen_min_batch_;
+    // (not with e4m3 operands in the chain: the generator is then an fp8 GEMM of its own)
+    const bool chain_f8 = f8 && q_smolgen_ && e.has_smolgen;
+    const bool fused_gen = e.has_smolgen && smolgen_wfrag_ != nullptr && B >= fused_smolgen_min_batch_ && !chain_f8;
     auto launch_qkv = [&] {
       if (f8 && q_qkv_) {
         GemmF8("gemm_qkv", xq_, e.qkv, e.qkv8, qkv_, T, kActNone, false, 1.0f);
@@ -1663,6 +1725,28 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       // or at most 128 positions): its kernels then take the variants with the shortest latency. At larger fp16
       // batches the two are balanced and the leaner variants disturb the projection less (batch 256: 1.5 %).
       const bool chain_first = f8 || B <= chain_latency_max_batch_;
+      if (chain_f8) {
+        // The whole chain on e4m3 operands: the compression reads the e4m3 copy of x that the QKV projection reads
+        // and writes e4m3 itself; the two row norms write halves, which a small kernel quantises.
+        GemmF8("gemm_smolgen_compress", xq_, e.sg_compress, e.sg_compress8, sg1q_, T, kActNone, true, 1.0f / e.s_sg1, ss);
+        GemmF8("gemm_smolgen_dense1", sg1q_, e.sg_dense1, e.sg_dense18, sg2_, B, smolgen_act_, false, 1.0f, ss);
+        Timed("layer_norm_rows", 0.0, 4.0 * B * sg_hs_, [&] {
+          LaunchLayerNormRows(nullptr, 0, 0, sg2_, kActNone, nullptr, sg2_, e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f,
+                              1e-3f, ss);
+        }, ss);
+        Timed("quantize_f8", 0.0, 3.0 * B * sg_hs_, [&] {
+          LaunchQuantizeF8(sg2_, sg2q_, static_cast<long long>(B) * sg_hs_, 1.0f / e.s_sg2, ss);
+        }, ss);
+        GemmF8("gemm_smolgen_dense2", sg2q_, e.sg_dense2, e.sg_dense28, sg3_, B, smolgen_act_, false, 1.0f, ss);
+        Timed("layer_norm_rows", 0.0, 4.0 * B * sg_gen_, [&] {
+          LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f,
+                              1e-3f, ss);
+        }, ss);
+        Timed("quantize_f8", 0.0, 3.0 * B * sg_gen_, [&] {
+          LaunchQuantizeF8(sg3_, sg3q_, static_cast<long long>(B) * sg_gen_, 1.0f / e.s_sg3, ss);
+        }, ss);
+        GemmF8("gemm_smolgen_global", sg3q_, smolgen_w_, e.sg_global8, sbias_, B * heads_, kActNone, false, 1.0f, ss);
+      } else {
       Gemm("gemm_smolgen_compress", x_, emb_, norm_in ? e.sg_compress_n : e.sg_compress, sg1_, sg_hc_, T, kActNone,
            false, ss, 1, chain_first, norm_in ? &cons_in : nullptr);
       // dense1 has a long reduction and few outputs. With few rows one workgroup per 16x16 outputs splits K over
@@ -1683,13 +1767,19 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
                               e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f, 1e-3f, ss);
         }, ss);
       }
+      if (calibrating_ && q_smolgen_) {
+        RecordAbsMax(sg1_, static_cast<size_t>(T) * sg_hc_, SmolgenSlot(li, 0), ss);
+        RecordAbsMax(sg2_, static_cast<size_t>(B) * sg_hs_, SmolgenSlot(li, 1), ss);
+      }
       Gemm("gemm_smolgen_dense2", sg2_, sg_hs_, e.sg_dense2, sg3_, sg_gen_, B, smolgen_act_, false, ss, 1, chain_first);
       Timed("layer_norm_rows", 0.0, 4.0 * B * sg_gen_, [&] {
         LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f, 1e-3f,
                             ss);
       }, ss);
+      if (calibrating_ && q_smolgen_) RecordAbsMax(sg3_, static_cast<size_t>(B) * sg_gen_, SmolgenSlot(li, 2), ss);
       if (!fused_gen) {
         Gemm("gemm_smolgen_global", sg3_, g, smolgen_w_, sbias_, 4096, B * heads_, kActNone, false, ss, 1, chain_first);
+      }
       }
       if (ss != stream_) HIP_CHECK(hipEventRecord(join_events_[li], ss));
       bias = sbias_;
@@ -1767,7 +1857,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     } else {
       Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, t_, emb_, T, kActNone);
     }
-    const bool ln2_f8 = f8_any && li + 1 < n_f8_layers && q_qkv_;   // the next layer reads an e4m3 copy
+    const bool ln2_f8 = f8_any && li + 1 < n_f8_layers && (q_qkv_ || q_smolgen_);   // the next layer reads an e4m3 copy
     Timed("layer_norm_skip", 0.0, (ln2_f8 ? 7.0 : 6.0) * T * emb_, [&] {
       LaunchLayerNorm(t_, x_, x_, e.ln2_g, e.ln2_b, T, emb_, alpha_, eps_, stream_, ln2_f8 ? xq_ : nullptr,
                       last ? 1.0f : 1.0f / encoders_[li + 1].s_x);

@@ -107,6 +107,10 @@ class Network {
   // precision=fp8 only: re-derives the per-tensor activation scales from the maxima
   // that these n positions (packed planes as for AddInputs) produce in an fp16 pass.
   virtual void CalibrateFp8(int n, const uint64_t* masks, const float* values) = 0;
+  // precision=fp8 only: the activation scales in use (value = code x scale), seven per encoder layer: the operands of
+  // Q/K/V, attention output, FFN1 and FFN2, then of smolgen's first dense layer, second dense layer and generator
+  // (1 where that operand stays in fp16).
+  virtual std::vector<float> Fp8Scales() const = 0;
 };
 
 // Factory: the counterpart of MakeBlasNetwork (src/neural/backends/blas/network_blas.cc:1115-1182).

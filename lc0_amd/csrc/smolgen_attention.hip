@@ -21,6 +21,7 @@
 #include <hip/hip_runtime.h>
 
 #include <stdexcept>
+#include <type_traits>
 
 #include "device_math.h"
 #include "kernels.h"
@@ -46,7 +47,26 @@ __device__ __forceinline__ int LogitSlot(int c, int qq, int g4, int t) {
   return (((c * 16 + (qq ^ ((c >> 2) & 1))) * 4 + (g4 ^ (c & 3))) * 32) + t * 8;
 }
 
-template <int NKS, typename OutT>
+// x combined with the values of the lanes 16, 32 and 48 away, with the lane-swap instructions of gfx950 (two vector
+// ALU operations per step instead of a round trip through the LDS crossbar). v_permlane16_swap exchanges the odd
+// 16-lane rows of its first register with the even rows of its second, v_permlane32_swap the upper half of the
+// first with the lower half of the second: fed the same value twice, the two registers afterwards hold the value
+// of this lane's row (half) and of its neighbour's. Written as assembly: the compiler's builtin for these
+// instructions loses track of the second result register. The no-ops cover the wait states between a vector ALU
+// write and a lane swap that reads it, and between the swap and its readers.
+template <typename F>
+__device__ __forceinline__ float Reduce4Rows(float x, F&& op) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  float y = op(a, b);
+  float c = y;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(y), "+v"(c));
+  return op(y, c);
+}
+
+// FULL: 32 heads and an even number of samples, so that every (sample, head) column of every workgroup exists and
+// the loop over head pairs carries no branches (the compiler then overlaps neighbouring pairs).
+template <int NKS, typename OutT, bool FULL>
 __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t* __restrict__ qkv,
                                                                     const half_t* __restrict__ gen,
                                                                     const half_t* __restrict__ wfrag,
@@ -155,8 +175,8 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
     const int ca = wave * 8 + 2 * pi;
     const int b = ca >= 32 ? b1 : b0;
     const int ha = ca & 31;
-    const int ha_c = ha < heads ? ha : 0;
-    const bool has_b = ha_c + 1 < heads;
+    const int ha_c = (FULL || ha < heads) ? ha : 0;
+    const bool has_b = FULL || ha_c + 1 < heads;
     const half_t* base = qkv + (long long)b * 64 * ld;
     // (without a head B the upper half of the row repeats head A instead of running past the row)
     const half_t* Kp = base + d_model + ha_c * DEPTH + (has_b ? ch : (ch & 3)) * 8 + (unsigned)lr * (unsigned)ld;
@@ -202,8 +222,8 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
   for (int pi = 0; pi < 4; pi++) {
     const int ca = wave * 8 + 2 * pi;
     const int ha = ca & 31;
-    const bool live_a = ha < heads && (ca < 32 || valid1);   // uniform over the wave
-    const bool live_b = live_a && ha + 1 < heads;
+    const bool live_a = FULL || (ha < heads && (ca < 32 || valid1));   // uniform over the wave
+    const bool live_b = FULL || (live_a && ha + 1 < heads);
     if (pi + 1 < 4) load_pair(pi + 1, nxt);
     if (live_a) {
       const int b = ca >= 32 ? b1 : b0;
@@ -254,8 +274,7 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
             sv[4 * t + e] = st[hb][t][e] * scale + lgv;
             mx = fmaxf(mx, sv[4 * t + e]);
           }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = Reduce4Rows(mx, [](float a, float b) { return fmaxf(a, b); });
         float sum = 0.0f;
         const float kLog2e = 1.44269504f, neg_mx = -mx * kLog2e;
 #pragma unroll
@@ -263,8 +282,7 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
           sv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[e], kLog2e, neg_mx));   // e^(s - mx) <= 1
           sum += sv[e];
         }
-        sum += __shfl_xor(sum, 16, 64);
-        sum += __shfl_xor(sum, 32, 64);
+        sum = Reduce4Rows(sum, [](float a, float b) { return a + b; });
         const float inv = __builtin_amdgcn_rcpf(sum);   // 1 ulp
         half8 pf[2];
 #pragma unroll
@@ -303,20 +321,20 @@ void LaunchT(const half_t* qkv, const half_t* gen, const half_t* wfrag, OutT* ou
   if (batch <= 0) return;
   const int pairs = (batch + 1) / 2;
   const dim3 grid(((pairs + 7) / 8) * 32), block(512);
-  switch (gen_sz) {
-    case 256:
-      hipLaunchKernelGGL((smolgen_attention_kernel<16, OutT>), grid, block, 0, stream, qkv, gen, wfrag, out, batch,
-                         heads, scale, out_mul);
-      break;
-    case 128:
-      hipLaunchKernelGGL((smolgen_attention_kernel<8, OutT>), grid, block, 0, stream, qkv, gen, wfrag, out, batch,
-                         heads, scale, out_mul);
-      break;
-    default:
-      hipLaunchKernelGGL((smolgen_attention_kernel<2, OutT>), grid, block, 0, stream, qkv, gen, wfrag, out, batch,
-                         heads, scale, out_mul);
-      break;
-  }
+  const bool full = heads == 32 && batch % 2 == 0;
+  auto launch = [&](auto nks_tag, auto full_tag) {
+    hipLaunchKernelGGL((smolgen_attention_kernel<decltype(nks_tag)::value, OutT, decltype(full_tag)::value>), grid, block, 0,
+                       stream, qkv, gen, wfrag, out, batch, heads, scale, out_mul);
+  };
+  auto by_width = [&](auto full_tag) {
+    switch (gen_sz) {
+      case 256: launch(std::integral_constant<int, 16>{}, full_tag); break;
+      case 128: launch(std::integral_constant<int, 8>{}, full_tag); break;
+      default: launch(std::integral_constant<int, 2>{}, full_tag); break;
+    }
+  };
+  if (full) by_width(std::true_type{});
+  else by_width(std::false_type{});
 }
 
 }  // namespace

@@ -74,8 +74,7 @@ def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
 def set_gemm_variant(variant):
     """-1 automatic, 0..2 direct-to-LDS 256x{256,192,128} tiles, 3 128x128, 4 64x64, 5 direct-to-LDS 128x128,
     6 row panels (16x16 to 64x32 outputs per workgroup, K split over its waves), 7 direct-to-LDS 128x64,
-    8 persistent 256x256 (one workgroup per CU walks over the tiles; M, N multiples of 256, K of 128; other shapes
-    fall back to the automatic choice), 9 direct-to-LDS 128x32 (very many rows, at most 32 columns), 10 direct-to-LDS
+    8 unused (automatic choice), 9 direct-to-LDS 128x32 (very many rows, at most 32 columns), 10 direct-to-LDS
     64x64 (a few hundred rows)."""
     _lib().lc0mi_k_set_gemm_variant(int(variant))
 

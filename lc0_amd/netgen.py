@@ -295,6 +295,8 @@ CONFIGS = {
     "tiny_attn": lambda: attention_body(64, 2, 2, 96, seed=2001, smolgen=(8, 32, 32), perturb_ln=True, std=0.1),
     # smallest shape the fp8 configuration accepts (all widths multiples of 128)
     "tiny_attn_f8": lambda: attention_body(128, 3, 4, 256, seed=2005, smolgen=(8, 32, 32), perturb_ln=True, std=0.07),
+    # the same with smolgen widths the fp8 form of the smolgen chain accepts (multiples of 128)
+    "tiny_attn_f8_sg": lambda: attention_body(128, 2, 4, 256, seed=2021, smolgen=(8, 128, 128), perturb_ln=True, std=0.07),
     # modern format: dense position encoding + embedding FFN, input gating, multi-head format
     "tiny_attn_dense": lambda: attention_body(64, 2, 2, 96, seed=2006, smolgen=(8, 32, 32), perturb_ln=True,
                                               pe_dense=(16, 128), gating=True, multihead=True, std=0.1),

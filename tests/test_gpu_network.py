@@ -35,7 +35,7 @@ def _run_gpu(path, masks, values, options=""):
     return net, res
 
 
-def _compare(res, want, legal, tol=TOL):
+def _compare(res, want, legal, tol=TOL, logit_frac=None):
     pol_g, pol_o = res["policy"], want["policy"]
     sm_g, sm_o = onn.softmax_rows(pol_g), onn.softmax_rows(pol_o)
     stats = dict(policy_softmax=np.abs(sm_g - sm_o).max(),
@@ -45,20 +45,31 @@ def _compare(res, want, legal, tol=TOL):
                  mlh_rel=(np.abs(res["m"] - want["m"]) / np.maximum(np.abs(want["m"]), 1.0)).max())
     stats["m_max"] = float(np.abs(want["m"]).max())
     legal_err = 0.0
-    top1 = 0
+    # Raw logits: the softmax of a near-uniform policy hides errors, so the logits are bounded on their own, by the
+    # tolerance plus a fraction of their spread over the legal moves (fp16: 5e-3 + 5 %; fp32: 1e-3 + 1 %).
+    spread = float(np.concatenate([pol_o[i, lg] for i, lg in enumerate(legal)]).std())
+    logit_tol = tol + (logit_frac if logit_frac is not None else 0.05 if tol >= 5e-3 else 0.01) * spread
+    top1, flips = 0, []
     for i, lg in enumerate(legal):
         a, b = onn.check_softmax_legal(pol_g[i], lg), onn.check_softmax_legal(pol_o[i], lg)
         legal_err = max(legal_err, float(np.abs(a - b).max()))
-        top1 += int(a.argmax() == b.argmax())
+        if a.argmax() == b.argmax():
+            top1 += 1
+        else:   # how far the oracle itself rates the GPU's choice below its own
+            flips.append(float(pol_o[i, lg[b.argmax()]] - pol_o[i, lg[a.argmax()]]))
     stats["policy_legal_softmax"] = legal_err
     stats["top1_agreement"] = top1 / len(legal)
+    stats["logit_spread"] = spread
     print("parity:", {k: float(v) for k, v in stats.items()})
     assert stats["policy_softmax"] <= tol
     assert stats["policy_legal_softmax"] <= tol
     assert stats["wdl_q"] <= tol and stats["wdl_d"] <= tol
     assert stats["mlh_rel"] <= 2e-2
-    # logits of a random-init net are O(1): 3e-2 absolute is ~1e-2 relative
-    assert stats["logits"] <= 3e-2 * max(1.0, float(np.abs(pol_o).max()))
+    assert stats["logits"] <= logit_tol, (stats["logits"], logit_tol)
+    # Best legal move: the same as the oracle's on at least 99 % of the positions, and where it differs the two
+    # moves are a tie within the logit bound (the only flip that arithmetic within that bound can cause).
+    assert all(gap <= 2 * logit_tol for gap in flips), flips
+    assert stats["top1_agreement"] >= 0.99 or len(flips) <= 1, stats["top1_agreement"]
     return stats
 
 
@@ -202,22 +213,22 @@ def test_file_forms_of_real_nets_match_oracle(name, encoding, options, tol, posi
 
 @pytest.mark.timeout(900)
 def test_bt4_shape_batch_256(positions):
-    """configs[2]: oracle comparison on the first 48 positions (seconds of CPU
-    time), then size-independent properties at the full batch of 256: rows are
-    independent, so the full-batch rows equal the small-batch rows, and a
-    permuted batch gives permuted outputs."""
+    """configs[2] at its full batch: all 256 positions through the default path (256-row streaming tiles, smolgen
+    generator inside the attention kernel, second stream) against the oracle, then the same rows in a small batch
+    (other kernels: unfused attention, main stream only) and a permuted batch."""
     path = netgen.cached_config("c2_bt4_15x1024")
     masks, values = positions["masks"][:256], positions["values"][:256]
-    want = onn.BlasNetwork(nr.load(path)).forward(masks[:48], values[:48])
-    net, res48 = _run_gpu(path, masks[:48], values[:48])
-    _compare(res48, want, positions["legal"][:48])
-    comp = net.NewComputation()
-    comp.AddInputs(masks, values)
-    comp.ComputeBlocking()
-    full = comp.results()
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    net, full = _run_gpu(path, masks, values)
     assert np.isfinite(full["policy"]).all()
-    # Different batch sizes may run different GEMM tile shapes (another summation
-    # order, then fp16 rounding of activations): equal to fp16 accuracy, not bitwise.
+    _compare(full, want, positions["legal"][:256])
+    comp = net.NewComputation()
+    comp.AddInputs(masks[:48], values[:48])
+    comp.ComputeBlocking()
+    res48 = comp.results()
+    _compare(res48, {k: v[:48] for k, v in want.items()}, positions["legal"][:48])
+    # Different batch sizes run different GEMM tile shapes (another summation order, then fp16 rounding of
+    # activations): equal to fp16 accuracy, not bitwise.
     np.testing.assert_allclose(full["policy"][:48], res48["policy"], rtol=0, atol=5e-3)
     np.testing.assert_allclose(full["q"][:48], res48["q"], rtol=0, atol=5e-3)
     perm = np.random.default_rng(0).permutation(256)
@@ -374,11 +385,43 @@ def test_fp8_with_dense_embedding_and_named_heads(positions):
     assert s["q"] <= 0.08 and s["d"] <= 0.04
 
 
+ALL_FP8_GEMMS = ("qkv", "dense", "ffn1", "ffn2")
+
+
+def _legal_logit_rms(a, b, legal):
+    err = np.concatenate([(a[i, lg] - b[i, lg]) for i, lg in enumerate(legal)])
+    return float(np.sqrt((err * err).mean()))
+
+
+def _emulation_of(path, net, gemms=ALL_FP8_GEMMS, **kw):
+    """oracle/fp8_net.py with the activation scales the backend is using."""
+    from oracle import fp8_net
+    sc = net.Fp8Scales()
+    return fp8_net.Fp8BlasNetwork(nr.load(path), scales=sc[:, :4], smolgen_scales=sc[:, 4:], gemms=gemms, **kw)
+
+
+def _check_fp8_against_emulation(res, emu_out, oracle_out, legal, what):
+    """The GPU's e4m3 pass against the numpy emulation of the same arithmetic. Two faithful evaluations of an fp8
+    net differ by a fixed fraction of the format's own noise (a perturbation of half-precision size flips e4m3 codes,
+    each flip moves a value by a whole step), so the bar is relative to that noise, measured against the fp32
+    oracle on the same rows: logit rms difference at most 0.8 of it, and the emulation must be the closer of the two."""
+    noise = _legal_logit_rms(res["policy"], oracle_out["policy"], legal)
+    diff = _legal_logit_rms(res["policy"], emu_out["policy"], legal)
+    top_e = np.mean([lg[res["policy"][i, lg].argmax()] == lg[emu_out["policy"][i, lg].argmax()] for i, lg in enumerate(legal)])
+    top_o = np.mean([lg[res["policy"][i, lg].argmax()] == lg[oracle_out["policy"][i, lg].argmax()] for i, lg in enumerate(legal)])
+    q_e = float(np.abs(res["q"] - (emu_out["wdl"][:, 0] - emu_out["wdl"][:, 2])).max())
+    print("fp8 vs emulation (%s): logit rms %.2e against %.2e vs the fp32 oracle (ratio %.2f); top-1 %.3f vs emulation, "
+          "%.3f vs oracle; q %.2e" % (what, diff, noise, diff / noise, top_e, top_o, q_e))
+    assert diff <= 0.8 * noise, (what, diff, noise)
+    return diff, noise, float(top_e), float(top_o)
+
+
 @pytest.mark.timeout(900)
 def test_bt4_shape_fp8_batch_sweep(positions):
-    """configs[4]: the BT4-shape net with e4m3 GEMM operands. Oracle comparison on 64 positions,
-    then the batch sweep 1/16/64/256/1024: rows are independent, so every batch size must
-    reproduce the rows of the 64-position run."""
+    """configs[4]: the BT4-shape net with e4m3 GEMM operands. 64 positions against the fp32 oracle (KL, W/D/L, top-1)
+    and against the emulation of the fp8 arithmetic; then the batch sweep 1/16/64/256/1024, whose rows are
+    independent and must reproduce the 64-position run, with rows of the first, a middle and the last 256-row tile
+    of the largest batch against the emulation as well."""
     path = netgen.cached_config("c2_bt4_15x1024")
     masks, values, legal = positions["masks"][:64], positions["values"][:64], positions["legal"][:64]
     want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
@@ -386,16 +429,30 @@ def test_bt4_shape_fp8_batch_sweep(positions):
     s = _fp8_report(res, want, legal)
     assert s["kl_max"] <= 1e-4 and s["softmax_maxabs"] <= 1e-3
     assert s["q"] <= 1e-2 and s["d"] <= 1e-2 and s["mlh_rel"] <= 2e-2
-    # The bar is top-1 agreement >= 0.99. fp16 on the same positions is the floor any quantisation starts from.
+    emu = _emulation_of(path, net)
+    emu64 = emu.forward(masks, values)
+    _check_fp8_against_emulation(res, emu64, want, legal, "64 positions")
+    # A mis-wired activation scale is what such a comparison must notice: the emulation with the Q/K/V and FFN1
+    # products scaled back by each other's scale, and with every layer using the scales of the layer before it,
+    # is further from the GPU than the faithful one.
+    for fault in ("swap_x_x1", "stale_layer"):
+        bad = _emulation_of(path, net, perturb=fault).forward(masks[:32], values[:32])
+        d_bad = _legal_logit_rms(res["policy"][:32], bad["policy"], legal[:32])
+        d_ok = _legal_logit_rms(res["policy"][:32], emu64["policy"][:32], legal[:32])
+        print("emulation with fault %s: logit rms %.2e against %.2e without" % (fault, d_bad, d_ok))
+        assert d_bad > 1.5 * d_ok, fault   # measured 1.75x and 3.4x
+    # fp16 on the same positions is the floor any quantisation starts from.
     _, res16 = _run_gpu(path, masks, values, "")
     s16 = _fp8_report(res16, want, legal)
     print("top-1 agreement with the fp32 oracle on %d positions: fp16 %.3f, fp8 %.3f (decisive positions: %.3f of %d)"
           % (len(legal), s16["top1"], s["top1"], s["top1_decisive"], s["decisive"]))
     assert s16["top1"] >= 0.99
     assert s["top1_decisive"] >= 0.99
+    assert s["top1"] >= 0.88   # measured 0.92 to 0.94: a fall below that is a regression, not format noise
     reps = -(-1024 // 320)
     big_m = np.tile(positions["masks"], (reps, 1))[:1024]
     big_v = np.tile(positions["values"], (reps, 1))[:1024]
+    big_legal = (positions["legal"] * reps)[:1024]
     for n in (1, 16, 64, 256, 1024):
         comp = net.NewComputation()
         comp.AddInputs(big_m[:n], big_v[:n])
@@ -410,12 +467,68 @@ def test_bt4_shape_fp8_batch_sweep(positions):
         assert np.sqrt(np.mean(diff * diff)) <= 2 * s["logit_rms"]
         assert np.abs(diff).max() <= 10 * s["logit_rms"] + 5e-3
         np.testing.assert_allclose(r["q"][:k], res["q"][:k], rtol=0, atol=1e-2)
+        if n == 1024:
+            rows = np.r_[0:8, 504:520, 1016:1024]
+            want_rows = onn.BlasNetwork(nr.load(path)).forward(big_m[rows], big_v[rows])
+            emu_rows = emu.forward(big_m[rows], big_v[rows])
+            _check_fp8_against_emulation({key: val[rows] for key, val in r.items()}, emu_rows, want_rows,
+                                         [big_legal[i] for i in rows], "rows of three tiles at batch 1024")
     if s["top1"] < 0.99:
-        # Everything above holds; the stated bar does not on this net. e4m3 keeps 3 mantissa bits: the rms logit
-        # error is ~5 % of the logit spread of an N(0, 0.02)-initialised net (std 0.07 over ~30 legal moves), and
-        # no configuration measured (fewer fp8 GEMMs, fp16 last layers, per-row activation scales) reaches 0.99.
+        # Everything above holds; the stated bar (top-1 agreement >= 0.99 with the fp32 reference) does not on this
+        # net. e4m3 keeps 3 mantissa bits: the rms logit error is ~5 % of the logit spread of an N(0, 0.02)-initialised
+        # net (std 0.07 over ~30 legal moves). Measured and short of 0.99 as well: fp8 in a subset of the four GEMMs,
+        # the last 1 to 8 layers in fp16. Per-row activation scales were not built (a floating-point format gains
+        # nothing from them above its subnormal range).
         pytest.xfail("fp8 top-1 agreement %.3f is below the 0.99 bar (fp16: %.3f; decisive positions: %.3f)"
                      % (s["top1"], s16["top1"], s["top1_decisive"]))
+
+
+@pytest.mark.parametrize("name,batch", [("tiny_attn_f8_sg", 40), ("c2_bt4_15x1024", 33)])
+def test_fp8_smolgen_chain_in_e4m3(name, batch, positions):
+    """fp8_gemms=...+smolgen (configs[4] lists the smolgen GEMMs among the e4m3 ones): compression, both dense layers
+    and the shared generator run on e4m3 operands. Against the emulation of the same arithmetic and, by noise
+    level, against the fp32 oracle; the profile must show the chain's fp8 kernels."""
+    path = netgen.cached_config(name)
+    masks, values, legal = positions["masks"][:batch], positions["values"][:batch], positions["legal"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    gemms = ALL_FP8_GEMMS + ("smolgen",)
+    net, res = _run_gpu(path, masks, values, "precision=fp8,fp8_gemms=" + "+".join(gemms))
+    s = _fp8_report(res, want, legal)
+    assert s["logit_rms"] <= 0.1 * s["logit_std"] and s["kl_max"] <= 1e-3 and s["top1_decisive"] >= 0.99
+    sc = net.Fp8Scales()
+    assert sc.shape[1] == 7 and (sc[:, 4:] != 1.0).all()
+    _check_fp8_against_emulation(res, _emulation_of(path, net, gemms=gemms).forward(masks, values), want, legal,
+                                 name + " with the smolgen chain in e4m3")
+    net.SetProfiling(True)
+    comp = net.NewComputation()
+    comp.AddInputs(masks, values)
+    comp.ComputeBlocking()
+    names = [k.name for k in net.TakeProfile()]
+    net.SetProfiling(False)
+    for layer in ("compress", "dense1", "dense2", "global"):
+        assert any(n.startswith("gemm_smolgen_%s|gemm_f8" % layer) for n in names), (layer, names)
+
+
+def test_fp8_activation_scales_match_the_calibration_rule(positions):
+    """Every activation scale the backend derives from caller-supplied positions (lc0mi_net_calibrate_fp8) against
+    the emulation's own calibration on the same positions: the largest magnitude of the right tensor maps to 224.
+    A scale taken at the wrong point of the layer, or from the wrong layer, shows here tensor by tensor."""
+    from oracle import fp8_net
+    for name, gemms in (("tiny_attn_f8_sg", ALL_FP8_GEMMS + ("smolgen",)), ("tiny_attn_f8", ALL_FP8_GEMMS)):
+        path = netgen.cached_config(name)
+        masks, values = positions["masks"][:96], positions["values"][:96]
+        from lc0_amd import Network
+        net = Network(path, "precision=fp8,fp8_gemms=" + "+".join(gemms))
+        net.CalibrateFp8(masks, values)
+        got = net.Fp8Scales()
+        want, want_sg = fp8_net.Fp8BlasNetwork(nr.load(path), quantize=False).calibrate(masks, values)
+        np.testing.assert_allclose(got[:, :4], want, rtol=5e-3, err_msg=name)
+        if "smolgen" in gemms:
+            np.testing.assert_allclose(got[:, 4:], want_sg, rtol=5e-3, err_msg=name)
+        else:
+            assert (got[:, 4:] == 1.0).all()
+        # distinct tensors have distinct scales on this net: equal entries would make the check above blind
+        assert len(np.unique(np.round(got[:, :4] / got[:, :4].max(), 3))) >= got[:, :4].size // 2
 
 
 # ---- modern net format: PE_DENSE embedding, input gating, multi-head format ---------------
@@ -548,7 +661,9 @@ def test_head_depth_64_policy_encoders_and_attention_policy_on_a_tower(name, bat
     masks, values = positions["masks"][:batch], positions["values"][:batch]
     want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
     _, res = _run_gpu(path, masks, values)
-    _compare(res, want, positions["legal"][:batch])
+    # (the tower's winograd products are halves and the policy embedding takes SELU of them: the worst logit of
+    # tiny_resnet_attnpolicy is 6 % of the spread off, measured 0.044 at spread 0.61; attention bodies stay at 5 %)
+    _compare(res, want, positions["legal"][:batch], logit_frac=0.08 if name == "tiny_resnet_attnpolicy" else None)
 
 
 def test_attention_policy_on_a_tower_needs_fp16():
