@@ -159,6 +159,11 @@ def main():
         masks, values = np.tile(masks, (reps, 1)), np.tile(values, (reps, 1))
     net = Network(path, "gpu=0,max_batch=%d" % max([batch, 16] + sweep) + ("," + wl["options"] if wl.get("options") else "") +
                   ("," + args.options if args.options else ""))
+    # Arithmetic type of the pass: the workload's own, or what a precision= option given on the command line says.
+    dtype = wl.get("dtype", "fp16")
+    for item in args.options.split(","):
+        if item.startswith("precision="):
+            dtype = {"fp8": "fp8_e4m3"}.get(item.split("=", 1)[1], item.split("=", 1)[1])
     comp = net.NewComputation()
     comp.AddInputs(masks[:batch], values[:batch])
     comp.ComputeBlocking()          # stages the batch into HBM and warms everything up
@@ -255,7 +260,7 @@ def main():
         groups[variant] = Agg(variant, g.ms + k.ms, g.launches + k.launches, g.flops + k.flops, g.bytes + k.bytes)
     dom = max(groups.values(), key=lambda g: g.ms)
     peak = (PEAK_FP8_TFLOPS if dom.name.startswith("gemm_f8") else
-            PEAK_FP32_TFLOPS if dom.name.startswith("gemm_f32") else PEAK_FP16_TFLOPS)
+            PEAK_FP32_TFLOPS if dom.name.startswith("gemm_f32") else PEAK_FP16_TFLOPS)   # (bf16 has the fp16 peak)
     # A matrix kernel is priced against the MFMA peak only when its flops per algorithmic byte lie above the ridge
     # point peak flops / peak bandwidth (fp16: 312 flop/B); below it the memory roofline is the one that bounds it
     # (the 36 batched winograd-domain GEMMs of a 256-filter convolution: 121 flop/B).
@@ -280,7 +285,7 @@ def main():
         "unit": "evals/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": wl.get("dtype", "fp16"), "data": "synthetic",
+        "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": {"workload": args.config, "description": wl["desc"], "batch": batch,
                    "inputs": "seeded random-playout positions, classical 112 planes",
                    **({"extra_options": args.options} if args.options else {})},

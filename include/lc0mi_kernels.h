@@ -127,12 +127,14 @@ int lc0mi_k_expand_planes_nhwc(const uint64_t* masks, const float* values, int b
 
 /* lc0mi_k_gemm_splitk for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. dA, dW, dbias (may be
- * NULL) and dC are DEVICE pointers (dA, dW 16-byte aligned); the work is enqueued on `stream` (a hipStream_t, NULL =
+ * NULL) and dC are DEVICE pointers (device or managed memory; dA, dW and dbias 16-byte aligned); the work is enqueued on `stream` (a hipStream_t, NULL =
  * the default stream) and the call returns without waiting. The partial sums of the K slices go to a fixed 16 MiB
  * array inside the library (one per GPU, held until the process ends): M * ldc * split_k may be at most 4194304
  * floats, larger requests fail with an error. The call uses no hipMalloc / hipFree. All calls on one GPU share that
  * array, so two calls that overlap in time on one GPU (different streams or threads) race; calls on one stream do
- * not. The first call on a device looks up the array's address and should be made outside graph capture. */
+ * not. The first call on a device looks up the array's address and should be made outside graph capture. The kernel
+ * variant is the automatic choice unless lc0mi_k_set_gemm_variant, a process-wide test hook, has forced another:
+ * do not change that setting while calls are in flight. */
 int lc0mi_k_gemm_splitk_noalloc(const uint16_t* dA, int lda, const uint16_t* dW, int ldw, const float* dbias, int M,
                                 int N, int K, int split_k, float scale, float* dC, int ldc, void* stream);
 

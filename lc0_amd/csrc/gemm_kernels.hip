@@ -27,8 +27,10 @@ namespace {
 // for one m and stores 8 bytes at a time. Global tiles are fetched as 16-byte
 // vectors into registers one k-tile ahead and staged through padded LDS.
 // ---------------------------------------------------------------------------
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, typename OutT>
+// ET: type of the operands (half_t or bf16_t); OutT: float, or ET.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, typename OutT, typename ET = half_t>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
+  using ev8 = typename Vec16<ET>::v8;
   static_assert(WAVES_M * WAVES_N == 4, "four waves per block");
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -102,18 +104,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     if (kt + 1 < nk) load_tile(k_begin + (kt + 1) * BK);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ks++) {
-      half8 af[TM], wf[TN];
+      ev8 af[TM], wf[TN];
 #pragma unroll
       for (int i = 0; i < TM; i++)
-        af[i] = *reinterpret_cast<const half8*>(&As[(wm * WM + i * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+        af[i] = *reinterpret_cast<const ev8*>(&As[(wm * WM + i * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
 #pragma unroll
       for (int j = 0; j < TN; j++)
-        wf[j] = *reinterpret_cast<const half8*>(&Ws[(wn * WN + j * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+        wf[j] = *reinterpret_cast<const ev8*>(&Ws[(wn * WN + j * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
 #pragma unroll
       for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; j++) acc[i][j] = Mfma32(wf[j], af[i], acc[i][j]);
     }
     __syncthreads();
   }
@@ -176,8 +177,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
           OutT* dst = C + (long long)m * p.ldc + n;
           if (vec_ok && n + 3 < N) {
             if constexpr (sizeof(OutT) == 2) {
-              half4 h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-              *reinterpret_cast<half4*>(dst) = h;
+              using ov4 = typename Vec16<OutT>::v4;
+              ov4 h = {(OutT)v[0], (OutT)v[1], (OutT)v[2], (OutT)v[3]};
+              *reinterpret_cast<ov4*>(dst) = h;
             } else {
               floatx4 f = {v[0], v[1], v[2], v[3]};
               *reinterpret_cast<floatx4*>(dst) = f;
@@ -206,8 +208,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 // eight partial sums are added in wave order through LDS, so results do not depend on
 // timing.
 // ---------------------------------------------------------------------------
-template <int RT, int CT, int U, typename OutT>
+template <int RT, int CT, int U, typename OutT, typename ET = half_t>
 __global__ __launch_bounds__(512) void gemm_rowpanel_kernel(GemmArgs p) {
+  using ev8 = typename Vec16<ET>::v8;
   constexpr int NW = 8, ROWS = 16 * RT, COLS = 16 * CT, LD = COLS + 1;
   __shared__ float part[NW][ROWS * LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -233,14 +236,14 @@ __global__ __launch_bounds__(512) void gemm_rowpanel_kernel(GemmArgs p) {
     for (int c = 0; c < CT; c++) acc[t][c] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
   // Loads carry no predicate, so that the compiler can put the loads of U steps in flight at once.
   for (int st = s_begin; st < s_end; st += U) {
-    half8 fa[RT][U], fw[CT][U];
+    ev8 fa[RT][U], fw[CT][U];
 #pragma unroll
     for (int u = 0; u < U; u++) {   // steps past the end re-read the last one (never used)
       const int k = min(st + u, s_end - 1) * 32;
 #pragma unroll
-      for (int t = 0; t < RT; t++) fa[t][u] = *reinterpret_cast<const half8*>(a_row[t] + k);
+      for (int t = 0; t < RT; t++) fa[t][u] = *reinterpret_cast<const ev8*>(a_row[t] + k);
 #pragma unroll
-      for (int c = 0; c < CT; c++) fw[c][u] = *reinterpret_cast<const half8*>(w_row[c] + k);
+      for (int c = 0; c < CT; c++) fw[c][u] = *reinterpret_cast<const ev8*>(w_row[c] + k);
     }
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -249,23 +252,23 @@ __global__ __launch_bounds__(512) void gemm_rowpanel_kernel(GemmArgs p) {
         for (int t = 0; t < RT; t++)
 #pragma unroll
           for (int c = 0; c < CT; c++)
-            acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[c][u], fa[t][u], acc[t][c], 0, 0, 0);
+            acc[t][c] = Mfma16(fw[c][u], fa[t][u], acc[t][c]);
       }
     }
   }
   if (wave == NW - 1 && K % 32 != 0) {   // K is a multiple of 8: the missing part of the last step is zero-filled
     const int k = steps * 32;
-    const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const ev8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     const bool in = k + 8 * g < K;
-    half8 fa[RT], fw[CT];
+    ev8 fa[RT], fw[CT];
 #pragma unroll
-    for (int t = 0; t < RT; t++) fa[t] = in ? *reinterpret_cast<const half8*>(a_row[t] + k) : zero;
+    for (int t = 0; t < RT; t++) fa[t] = in ? *reinterpret_cast<const ev8*>(a_row[t] + k) : zero;
 #pragma unroll
-    for (int c = 0; c < CT; c++) fw[c] = in ? *reinterpret_cast<const half8*>(w_row[c] + k) : zero;
+    for (int c = 0; c < CT; c++) fw[c] = in ? *reinterpret_cast<const ev8*>(w_row[c] + k) : zero;
 #pragma unroll
     for (int t = 0; t < RT; t++)
 #pragma unroll
-      for (int c = 0; c < CT; c++) acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[c], fa[t], acc[t][c], 0, 0, 0);
+      for (int c = 0; c < CT; c++) acc[t][c] = Mfma16(fw[c], fa[t], acc[t][c]);
   }
   // Accumulator lane (r, g) of tile (t, c) holds row m = 16 t + r, columns n = 16 c + 4 g + e.
   float* mine = part[wave];
@@ -423,8 +426,9 @@ __device__ __forceinline__ void DmaToLds16(const void* gptr, void* lds_base) {
 // operands come from L2; with small tiles and operands that come from memory (a few hundred to a few thousand rows:
 // every workgroup streams weights nobody has touched since the previous pass) a k-tile takes longer to arrive than
 // to consume, and more stages hide that.
+// ET (fp16-type operands only): half_t or bf16_t; the output type is then ET as well.
 template <int BM, int BN, int BKB, int WAVES_M, int WAVES_N, typename Args, typename OutT, bool STREAM = false,
-          int EPI = 0, int NSTAGES = 2>
+          int EPI = 0, int NSTAGES = 2, typename ET = half_t>
 // Second launch bound = waves per SIMD: with small wave tiles two workgroups share a CU
 // (4 waves per SIMD, at most 128 VGPRs) and overlap each other's prologue and epilogue.
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64,
@@ -454,7 +458,10 @@ void gemm_dma_kernel(Args p) {
   constexpr int EPI_TOTAL = EPI_BYTES + STAT_BYTES + PART_BYTES;
   constexpr int SMEM = (NSTAGES * STAGE > EPI_TOTAL) ? NSTAGES * STAGE : EPI_TOTAL;
   static_assert(NSTAGES >= 2 && (NSTAGES - 2) * (A_CPW + W_CPW) <= 63, "transfers in flight must fit the counter");
-  static_assert(EPI == 0 || (!F8 && sizeof(OutT) == 2), "folded layer norm: fp16 operands and output");
+  static_assert(EPI == 0 || (!F8 && std::is_same<OutT, half_t>::value && std::is_same<ET, half_t>::value),
+                "folded layer norm: fp16 operands and output");
+  static_assert(std::is_same<ET, half_t>::value || (!F8 && std::is_same<OutT, ET>::value),
+                "bfloat16 operands go with bfloat16 output");
   // The tile's bias (and per-column scale, fp8 operands) waits in LDS behind the stages: fetched with the first k-tile,
   // so that the epilogue does not start with a round trip to memory.
   constexpr int COLV_BYTES = (F8 ? 2 : 1) * BN * 4;
@@ -596,16 +603,16 @@ void gemm_dma_kernel(Args p) {
 #pragma unroll
       for (int ks = 0; ks < BKB / 32; ks++) {
         const int coff = ((2 * ks + g) ^ swz) * 16;
-        half8 af[TM], wf[TN];
+        using ev8 = typename Vec16<ET>::v8;
+        ev8 af[TM], wf[TN];
 #pragma unroll
-        for (int i = 0; i < TM; i++) af[i] = *reinterpret_cast<const half8*>(As + a_row + i * 32 * BKB + coff);
+        for (int i = 0; i < TM; i++) af[i] = *reinterpret_cast<const ev8*>(As + a_row + i * 32 * BKB + coff);
 #pragma unroll
-        for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const half8*>(Ws + w_row + j * 32 * BKB + coff);
+        for (int j = 0; j < TN; j++) wf[j] = *reinterpret_cast<const ev8*>(Ws + w_row + j * 32 * BKB + coff);
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-          for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < TN; j++) acc[i][j] = Mfma32(wf[j], af[i], acc[i][j]);
       }
       if constexpr ((BM / WAVES_M / 32) * (BN / WAVES_N / 32) >= (BM / WAVES_M / 32) + (BN / WAVES_N / 32) && EPI == 0) {
         // Order of the k-tile's 32 MFMAs and 24 fragment reads: the reads of a k-step one by one between the MFMAs
@@ -731,10 +738,11 @@ void gemm_dma_kernel(Args p) {
             *reinterpret_cast<unsigned*>(dst) =
                 PackFp8x4(v[0] * p.out_mul, v[1] * p.out_mul, v[2] * p.out_mul, v[3] * p.out_mul);
           } else {
-            half4 h;
+            using ov4 = typename Vec16<OutT>::v4;
+            ov4 h;
 #pragma unroll
-            for (int rr = 0; rr < 4; rr++) h[rr] = (half_t)v[rr];
-            *reinterpret_cast<half4*>(dst) = h;
+            for (int rr = 0; rr < 4; rr++) h[rr] = (OutT)v[rr];
+            *reinterpret_cast<ov4*>(dst) = h;
           }
         }
       }
@@ -859,6 +867,9 @@ void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
         hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 1, 2>), grid, block, 0,
                            stream, a);
       }
+    } else if (a.bf16) {
+      hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, bf16_t, S, 0, NSTAGES, bf16_t>), grid,
+                         block, 0, stream, a);
     } else {
       hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 0, NSTAGES>), grid, block, 0,
                          stream, a);
@@ -933,7 +944,13 @@ void LaunchGemmDmaF8Staged(const GemmF8Args& a, hipStream_t stream) {
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 void LaunchGemmTile(const GemmArgs& a, hipStream_t stream) {
   dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch * a.split_k);
-  if (a.out_f32) {
+  if (a.bf16) {
+    if (a.out_f32) {
+      hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, float, bf16_t>), grid, dim3(256), 0, stream, a);
+    } else {
+      hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, bf16_t, bf16_t>), grid, dim3(256), 0, stream, a);
+    }
+  } else if (a.out_f32) {
     hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, float>), grid, dim3(256), 0, stream, a);
   } else {
     hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, half_t>), grid, dim3(256), 0, stream, a);
@@ -1009,7 +1026,16 @@ enum GemmVariant { kDma256x256, kDma256x192, kDma256x128, kTile128, kTile64, kDm
 
 int g_variant_override = -1;
 
+GemmVariant PickGemmVariantHalf(const GemmArgs& a);
+
+// bfloat16 operands run every variant except the row panels (kept out to bound the number of kernel instances):
+// such shapes take the register-staged 64x64 tiles.
 GemmVariant PickGemmVariant(const GemmArgs& a) {
+  const GemmVariant v = PickGemmVariantHalf(a);
+  return (a.bf16 && v == kRowPanel) ? kTile64 : v;
+}
+
+GemmVariant PickGemmVariantHalf(const GemmArgs& a) {
   if (g_variant_override >= 0) {
     const bool dma_ok = !a.out_f32 && a.split_k == 1 && a.K % 64 == 0;
     const bool is_dma = g_variant_override <= kDma256x128 || g_variant_override == kDma128x128 ||
@@ -1104,6 +1130,7 @@ int DmaTileN(GemmVariant v) {
 }  // namespace
 
 bool GemmSupportsNormFolding(const GemmArgs& a) {
+  if (a.bf16 && (a.skip != nullptr || a.row_stats != nullptr)) return false;
   const GemmVariant v = PickGemmVariant(a);
   if (a.skip != nullptr) {
     return DmaTileN(v) != 0 && v != kDma256x192 && !a.out_f32 && a.act == 3 && a.batch == 1 && a.N % 8 == 0 &&

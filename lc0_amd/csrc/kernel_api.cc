@@ -683,7 +683,8 @@ __global__ __launch_bounds__(256) void sum_slices_kernel(const float* __restrict
 
 void RequireDevicePointer(const void* p, const char* what) {
   hipPointerAttribute_t attr;
-  if (hipPointerGetAttributes(&attr, p) != hipSuccess || attr.type != hipMemoryTypeDevice) {
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess ||
+      (attr.type != hipMemoryTypeDevice && attr.type != hipMemoryTypeManaged)) {
     (void)hipGetLastError();
     throw Error(std::string(what) + " is not a device pointer");
   }
@@ -708,6 +709,7 @@ int lc0mi_k_gemm_splitk_noalloc(const uint16_t* dA, int lda, const uint16_t* dW,
     RequireDevicePointer(dC, "C");
     if (dbias) RequireDevicePointer(dbias, "bias");
     if ((reinterpret_cast<uintptr_t>(dA) | reinterpret_cast<uintptr_t>(dW)) & 15) throw Error("A and W must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(dbias) & 15) throw Error("bias must be 16-byte aligned");   // read four floats at a time
     float* part = ScratchOfCurrentDevice();
     hipStream_t st = static_cast<hipStream_t>(stream);
     lc0mi::GemmArgs g;

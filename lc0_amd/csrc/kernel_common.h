@@ -15,7 +15,28 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx8 __attribute__((ext_vector_type(8)));
 
+// 16-bit element types of activations and weights: IEEE half and bfloat16 (the same storage, kernels are
+// instantiated for either). Vector forms and the 32x32x16 / 16x16x32 matrix instructions per type.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+template <typename T> struct Vec16;
+template <> struct Vec16<half_t> { using v8 = half8; using v4 = half4; };
+template <> struct Vec16<bf16_t> { using v8 = bf16x8; using v4 = bf16x4; };
+
 namespace {
+
+__device__ __forceinline__ floatx16 Mfma32(half8 a, half8 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx16 Mfma32(bf16x8 a, bf16x8 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx4 Mfma16(half8 a, half8 b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx4 Mfma16(bf16x8 a, bf16x8 b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
 
 // Calls f with a branch-free functor for the activation, so that unrolled
 // epilogue loops do not carry a per-element switch.

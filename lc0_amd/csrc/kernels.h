@@ -10,6 +10,10 @@
 namespace lc0mi {
 
 using half_t = _Float16;
+using bf16_t = __bf16;
+// Element type of a network's activations and weights. The 16-bit launchers below take half_t pointers for either
+// 16-bit type (same storage); a `bf16` argument or field says which arithmetic the bits mean.
+enum class Dtype { kHalf, kBf16, kFloat };
 
 // C[b][m][n] = act(scale * sum_k A[b][m][k] * W[b][n][k] + bias[n]),  b < batch.
 // A and W are K-contiguous (row-major activations, lc0's [out][in] weights).
@@ -25,6 +29,8 @@ struct GemmArgs {
   float scale = 1.0f;
   int act = 3;  // Activation enum value (3 = none)
   bool out_f32 = false;
+  // A, W and (unless out_f32) C hold bfloat16 instead of half values. Not with the folded layer-norm fields.
+  bool bf16 = false;
   // split_k > 1: the K range is cut into split_k slices computed by different
   // workgroups; slice s stores its partial sums (float, out_f32 required, no
   // activation, bias only in slice 0) at C + s * split_stride. The consumer adds
@@ -115,13 +121,16 @@ template <typename T>
 void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T* pos_enc /*[64][64]*/,
                             T* out, int ld, int batch, hipStream_t stream);
 // Same with per-sample extra channels (the dense position encoding): out[b*64+sq][112 + c] =
-// extra[b][sq][c], c < n_extra.
-void LaunchExpandPlanesDense(const uint64_t* masks, const float* values, const half_t* extra, int n_extra,
-                             half_t* out, int ld, int batch, hipStream_t stream);
+// extra[b][sq][c], c < n_extra. T = half_t, bf16_t or float (also for the two launchers below and the one above).
+template <typename T>
+void LaunchExpandPlanesDense(const uint64_t* masks, const float* values, const T* extra, int n_extra, T* out, int ld,
+                             int batch, hipStream_t stream);
 // First 12 input planes, square-major: out[b][sq * 12 + j] (input of the dense position-encoding layer).
-void LaunchPiecePlanes(const uint64_t* masks, const float* values, half_t* out, int batch, hipStream_t stream);
+template <typename T>
+void LaunchPiecePlanes(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream);
 // Input gating: x[b][i] = x[b][i] * mult[i] + add[i], i < per_sample (= 64 * channels, square-major).
-void LaunchInputGating(half_t* x, const float* mult, const float* add, int batch, int per_sample, hipStream_t stream);
+template <typename T>
+void LaunchInputGating(T* x, const float* mult, const float* add, int batch, int per_sample, hipStream_t stream);
 // Input planes -> NCHW dense planes out[b][c][sq] (T = half_t or float).
 template <typename T>
 void LaunchExpandPlanesNchw(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream);
@@ -142,26 +151,37 @@ void SetGemmVariantOverride(int variant);
 // Activation enum value applied before the norm. C % 8 == 0, C <= 8192.
 void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_stride, const half_t* x_f16,
                          int pre_act, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows,
-                         int C, float alpha, float eps, hipStream_t stream);
+                         int C, float alpha, float eps, hipStream_t stream, bool bf16 = false);
 
 // rows x C layer norm: y = beta + gamma * (t - mean) / sqrt(var + eps) with
 // t = x * alpha + skip (skip may be null). x, skip, y may alias. C % 8 == 0, C <= 8192.
 // y_f8 (optional): also receives e4m3(y * f8_mul), saturating, the operand of a following fp8 GEMM.
 void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
                      int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8 = nullptr,
-                     float f8_mul = 1.0f);
+                     float f8_mul = 1.0f, bool bf16 = false);
+// The same for any element type (half_t, bf16_t, float) and any row length, with an activation applied to x first:
+// y = norm(act(x) * alpha + skip). One workgroup per row, scalar accesses.
+template <typename T>
+void LaunchLayerNormGeneric(const T* x, const T* skip, T* y, const float* gamma, const float* beta, int rows, int C,
+                            float alpha, float eps, int pre_act, hipStream_t stream);
 
 // Fused multi-head attention over 64 tokens, head depth 32, 64 or 128 (d_model = heads * depth).
 // qkv: [B*64][3*d_model] (q | k | v column blocks), bias: smolgen logits in the
 // tile-native layout produced by SmolgenBiasIndex (may be null), out: [B*64][d_model].
 void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int batch, int heads,
-                     float scale, hipStream_t stream, int depth = 32);
+                     float scale, hipStream_t stream, int depth = 32, bool bf16 = false);
 bool AttentionDepthSupported(int depth);
+// The same contract (bias in the SmolgenBiasIndex layout, may be null) for any element type and any head depth up to
+// 128, on the vector ALUs: the float configuration, and head depths the kernel above does not take.
+template <typename T>
+void LaunchAttentionGeneric(const T* qkv, const T* bias, T* out, int batch, int heads, int depth, float scale,
+                            hipStream_t stream);
+bool AttentionGenericDepthSupported(int depth);
 // Same with e4m3 output: out[...] = e4m3(result * out_mul), saturating.
 void LaunchAttentionF8Out(const half_t* qkv, const half_t* bias, uint8_t* out, float out_mul, int batch, int heads,
                           float scale, hipStream_t stream, int depth = 32);
 // Position inside one head's 4096-entry bias block of logit (query q, key k).
-int SmolgenBiasIndex(int q, int k);
+__host__ __device__ int SmolgenBiasIndex(int q, int k);
 
 // Smolgen generator layer and attention in one kernel (smolgen_attention.hip): the logits
 //   sum_j W[q*64+k][j] * gen[b][h][j]   (W: the shared smolgen_w layer [4096][gen_sz], gen: [B][heads][gen_sz])
@@ -180,7 +200,8 @@ void LaunchSmolgenAttentionF8Out(const half_t* qkv, const half_t* gen, const hal
 // logits: [B][64*64] float (already scaled), kq: [B*64][ld_kq] with keys at column
 // offset key_off, ppo: [4][pd] float, inv_map: [1858] source index into the
 // 4096+192 virtual buffer. out: [B][1858] float.
-void LaunchAttnPolicyGather(const float* logits, const half_t* kq, int ld_kq, int key_off, const float* ppo,
+template <typename T>   // T: element type of kq (half_t, bf16_t, float)
+void LaunchAttnPolicyGather(const float* logits, const T* kq, int ld_kq, int key_off, const float* ppo,
                             int pd, const int16_t* inv_map, float* out, int batch, hipStream_t stream);
 
 // Most legal moves one sample may list for LaunchLegalSoftmax (chess positions have at most 218).

@@ -64,25 +64,27 @@ __global__ __launch_bounds__(256) void expand_planes_attn_kernel(const uint64_t*
 }
 
 // First 12 planes (the current position's pieces) square-major: out[b][sq * 12 + j].
+template <typename T>
 __global__ __launch_bounds__(256) void piece_planes_kernel(const uint64_t* __restrict__ masks,
                                                            const float* __restrict__ values,
-                                                           half_t* __restrict__ out) {
+                                                           T* __restrict__ out) {
   const int b = blockIdx.x;
   for (int i = threadIdx.x; i < 64 * 12; i += 256) {
     const int sq = i / 12, j = i - sq * 12;
     const bool bit = (masks[(long long)b * 112 + j] >> sq) & 1ull;
-    out[(long long)b * 768 + i] = bit ? (half_t)values[(long long)b * 112 + j] : (half_t)0.0f;
+    out[(long long)b * 768 + i] = bit ? (T)values[(long long)b * 112 + j] : (T)0.0f;
   }
 }
 
 // x[b][sq][c] = x * mult[sq][c] + add[sq][c]
-__global__ __launch_bounds__(256) void input_gating_kernel(half_t* __restrict__ x, const float* __restrict__ mult,
+template <typename T>
+__global__ __launch_bounds__(256) void input_gating_kernel(T* __restrict__ x, const float* __restrict__ mult,
                                                            const float* __restrict__ add, int per_sample,
                                                            long long total) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
   const int j = (int)(i % per_sample);
-  x[i] = (half_t)((float)x[i] * mult[j] + add[j]);
+  x[i] = (T)((float)x[i] * mult[j] + add[j]);
 }
 
 template <typename T>
@@ -110,33 +112,41 @@ void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T*
   }
 }
 
-void LaunchExpandPlanesDense(const uint64_t* masks, const float* values, const half_t* extra, int n_extra,
-                             half_t* out, int ld, int batch, hipStream_t stream) {
+template <typename T>
+void LaunchExpandPlanesDense(const uint64_t* masks, const float* values, const T* extra, int n_extra, T* out, int ld,
+                             int batch, hipStream_t stream) {
   if (batch <= 0) return;
   if (ld % 8 == 0) {
-    hipLaunchKernelGGL((expand_planes_attn_kernel<half_t, 8>), dim3(batch), dim3(256), 0, stream, masks, values, extra,
+    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 8>), dim3(batch), dim3(256), 0, stream, masks, values, extra,
                        n_extra, 64LL * n_extra, out, ld);
   } else {
-    hipLaunchKernelGGL((expand_planes_attn_kernel<half_t, 1>), dim3(batch), dim3(256), 0, stream, masks, values, extra,
+    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 1>), dim3(batch), dim3(256), 0, stream, masks, values, extra,
                        n_extra, 64LL * n_extra, out, ld);
   }
 }
 
-void LaunchPiecePlanes(const uint64_t* masks, const float* values, half_t* out, int batch, hipStream_t stream) {
+template <typename T>
+void LaunchPiecePlanes(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream) {
   if (batch <= 0) return;
-  hipLaunchKernelGGL(piece_planes_kernel, dim3(batch), dim3(256), 0, stream, masks, values, out);
+  hipLaunchKernelGGL(piece_planes_kernel<T>, dim3(batch), dim3(256), 0, stream, masks, values, out);
 }
 
-void LaunchInputGating(half_t* x, const float* mult, const float* add, int batch, int per_sample, hipStream_t stream) {
+template <typename T>
+void LaunchInputGating(T* x, const float* mult, const float* add, int batch, int per_sample, hipStream_t stream) {
   const long long total = (long long)batch * per_sample;
   if (total <= 0) return;
-  hipLaunchKernelGGL(input_gating_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, mult, add,
+  hipLaunchKernelGGL(input_gating_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, mult, add,
                      per_sample, total);
 }
-template void LaunchExpandPlanesAttn<half_t>(const uint64_t*, const float*, const half_t*, half_t*, int, int,
-                                             hipStream_t);
-template void LaunchExpandPlanesAttn<float>(const uint64_t*, const float*, const float*, float*, int, int,
-                                            hipStream_t);
+#define LC0MI_INSTANTIATE_PLANES(T)                                                                                  \
+  template void LaunchExpandPlanesAttn<T>(const uint64_t*, const float*, const T*, T*, int, int, hipStream_t);       \
+  template void LaunchExpandPlanesDense<T>(const uint64_t*, const float*, const T*, int, T*, int, int, hipStream_t); \
+  template void LaunchPiecePlanes<T>(const uint64_t*, const float*, T*, int, hipStream_t);                           \
+  template void LaunchInputGating<T>(T*, const float*, const float*, int, int, hipStream_t);
+LC0MI_INSTANTIATE_PLANES(half_t)
+LC0MI_INSTANTIATE_PLANES(bf16_t)
+LC0MI_INSTANTIATE_PLANES(float)
+#undef LC0MI_INSTANTIATE_PLANES
 
 template <typename T>
 void LaunchExpandPlanesNchw(const uint64_t* masks, const float* values, T* out, int batch, hipStream_t stream) {
@@ -152,12 +162,13 @@ template void LaunchExpandPlanesNchw<float>(const uint64_t*, const float*, float
 // Layer norm with optional skip: one wave per row, the row held in registers.
 // ---------------------------------------------------------------------------
 namespace {
-template <int NV>  // 16-byte vectors per lane; covers C <= 512 * NV
+template <int NV, typename ET>  // 16-byte vectors per lane, covers C <= 512 * NV; ET: half_t or bf16_t (bits in half_t storage)
 __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restrict__ x, const half_t* skip,
                                                          half_t* y, uint8_t* yq, float q_mul,
                                                          const float* __restrict__ gamma,
                                                          const float* __restrict__ beta, int rows, int C,
                                                          float alpha, float eps) {
+  using ev8 = typename Vec16<ET>::v8;
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -170,9 +181,9 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restric
   for (int i = 0; i < NV; i++) {
     int v = lane + i * 64;
     if (v < nvec) {
-      half8 hx = *reinterpret_cast<const half8*>(xr + v * 8);
+      ev8 hx = *reinterpret_cast<const ev8*>(xr + v * 8);
       if (sr) {
-        half8 hs = *reinterpret_cast<const half8*>(sr + v * 8);
+        ev8 hs = *reinterpret_cast<const ev8*>(sr + v * 8);
 #pragma unroll
         for (int e = 0; e < 8; e++) t[i][e] = (float)hx[e] * alpha + (float)hs[e];
       } else {
@@ -202,14 +213,14 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restric
   for (int i = 0; i < NV; i++) {
     int v = lane + i * 64;
     if (v < nvec) {
-      half8 o;
+      ev8 o;
       float f[8];
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         f[e] = beta[v * 8 + e] + gamma[v * 8 + e] * (t[i][e] - mean) * den;
-        o[e] = (half_t)f[e];
+        o[e] = (ET)f[e];
       }
-      *reinterpret_cast<half8*>(yr + v * 8) = o;
+      *reinterpret_cast<ev8*>(yr + v * 8) = o;
       if (yq) {  // e4m3 copy of the same row for the next fp8 GEMM
         uint2 q;
         q.x = PackFp8x4(f[0] * q_mul, f[1] * q_mul, f[2] * q_mul, f[3] * q_mul);
@@ -242,13 +253,14 @@ __global__ __launch_bounds__(256) void zero_kernel(float* p, long long n) {
 // EARLY (few rows, where the kernel's latency is the pass's): gamma and beta, which nobody has touched since the
 // previous pass, are asked for first and arrive while the row is reduced; otherwise they are read where they are
 // used, which leaves more of the CU to a GEMM on the other stream.
-template <bool EARLY>
+template <bool EARLY, typename ET>
 __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __restrict__ xf, int n_partials,
                                                               long long partial_stride, const half_t* xh,
                                                               int pre_act, const half_t* skip, half_t* y,
                                                               const float* __restrict__ gamma,
                                                               const float* __restrict__ beta, int C, float alpha,
                                                               float eps) {
+  using ev8 = typename Vec16<ET>::v8;
   __shared__ float red[4];
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int nvec = C / 8;
@@ -282,14 +294,14 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __res
             for (int e = 0; e < 4; e++) { t[i][e] += a[e]; t[i][4 + e] += b[e]; }
           }
         } else {
-          half8 h = *reinterpret_cast<const half8*>(xh + off);
+          ev8 h = *reinterpret_cast<const ev8*>(xh + off);
 #pragma unroll
           for (int e = 0; e < 8; e++) t[i][e] = (float)h[e];
         }
 #pragma unroll
         for (int e = 0; e < 8; e++) t[i][e] = act_fn(t[i][e]) * alpha;
         if (skip != nullptr) {
-          half8 hs = *reinterpret_cast<const half8*>(skip + off);
+          ev8 hs = *reinterpret_cast<const ev8*>(skip + off);
 #pragma unroll
           for (int e = 0; e < 8; e++) t[i][e] += (float)hs[e];
         }
@@ -324,10 +336,10 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __res
         bt[i][0] = *reinterpret_cast<const floatx4*>(beta + v * 8);
         bt[i][1] = *reinterpret_cast<const floatx4*>(beta + v * 8 + 4);
       }
-      half8 o;
+      ev8 o;
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = (half_t)(bt[i][e / 4][e % 4] + gm[i][e / 4][e % 4] * (t[i][e] - mean) * den);
-      *reinterpret_cast<half8*>(y + (long long)row * C + v * 8) = o;
+      for (int e = 0; e < 8; e++) o[e] = (ET)(bt[i][e / 4][e % 4] + gm[i][e / 4][e % 4] * (t[i][e] - mean) * den);
+      *reinterpret_cast<ev8*>(y + (long long)row * C + v * 8) = o;
     }
   }
 }
@@ -353,34 +365,38 @@ void LaunchZero(float* p, long long n, hipStream_t stream) {
 
 void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_stride, const half_t* x_f16,
                          int pre_act, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows,
-                         int C, float alpha, float eps, hipStream_t stream) {
+                         int C, float alpha, float eps, hipStream_t stream, bool bf16) {
   if (rows <= 0) return;
-  if (rows <= 64) {
-    hipLaunchKernelGGL(layer_norm_rows_kernel<true>, dim3(rows), dim3(256), 0, stream, x_f32, n_partials,
-                       partial_stride, x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps);
+  auto launch = [&](auto early_tag, auto elem_tag) {
+    using ET = decltype(elem_tag);
+    hipLaunchKernelGGL((layer_norm_rows_kernel<decltype(early_tag)::value, ET>), dim3(rows), dim3(256), 0, stream, x_f32,
+                       n_partials, partial_stride, x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps);
+  };
+  if (bf16) {
+    if (rows <= 64) launch(std::true_type{}, bf16_t{});
+    else launch(std::false_type{}, bf16_t{});
   } else {
-    hipLaunchKernelGGL(layer_norm_rows_kernel<false>, dim3(rows), dim3(256), 0, stream, x_f32, n_partials,
-                       partial_stride, x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps);
+    if (rows <= 64) launch(std::true_type{}, half_t{});
+    else launch(std::false_type{}, half_t{});
   }
 }
 
 void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
-                     int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8, float f8_mul) {
+                     int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8, float f8_mul, bool bf16) {
   if (rows <= 0) return;
   dim3 grid((rows + 3) / 4), block(256);
-  if (C <= 512) {
-    hipLaunchKernelGGL(layer_norm_kernel<1>, grid, block, 0, stream, x, skip, y, y_f8, f8_mul, gamma, beta, rows, C,
-                       alpha, eps);
-  } else if (C <= 1024) {
-    hipLaunchKernelGGL(layer_norm_kernel<2>, grid, block, 0, stream, x, skip, y, y_f8, f8_mul, gamma, beta, rows, C,
-                       alpha, eps);
-  } else if (C <= 2048) {
-    hipLaunchKernelGGL(layer_norm_kernel<4>, grid, block, 0, stream, x, skip, y, y_f8, f8_mul, gamma, beta, rows, C,
-                       alpha, eps);
-  } else {  // callers guarantee C <= 8192
-    hipLaunchKernelGGL(layer_norm_kernel<16>, grid, block, 0, stream, x, skip, y, y_f8, f8_mul, gamma, beta, rows, C,
-                       alpha, eps);
-  }
+  auto launch = [&](auto nv_tag, auto elem_tag) {
+    hipLaunchKernelGGL((layer_norm_kernel<decltype(nv_tag)::value, decltype(elem_tag)>), grid, block, 0, stream, x, skip,
+                       y, y_f8, f8_mul, gamma, beta, rows, C, alpha, eps);
+  };
+  auto by_width = [&](auto elem_tag) {
+    if (C <= 512) launch(std::integral_constant<int, 1>{}, elem_tag);
+    else if (C <= 1024) launch(std::integral_constant<int, 2>{}, elem_tag);
+    else if (C <= 2048) launch(std::integral_constant<int, 4>{}, elem_tag);
+    else launch(std::integral_constant<int, 16>{}, elem_tag);   // callers guarantee C <= 8192
+  };
+  if (bf16) by_width(bf16_t{});
+  else by_width(half_t{});
 }
 
 namespace {
@@ -425,11 +441,13 @@ namespace {
 // DEPTH = head depth (32, 64 or 128); OutT = half_t, or uint8_t for e4m3 output scaled by out_mul.
 // Second launch bound = waves per SIMD the register allocation must allow: the kernel is a chain of
 // dependent memory phases (q/k/v loads, bias loads, stores), so resident waves are what hides latency.
-template <int DEPTH, typename OutT>
+// ET: half_t or bf16_t (inputs, bias and a 16-bit output, all in half_t storage).
+template <int DEPTH, typename OutT, typename ET>
 __global__ __launch_bounds__(256, DEPTH == 32 ? 4 : DEPTH == 64 ? 3 : 1) void attention_kernel(const half_t* __restrict__ qkv,
                                                         const half_t* __restrict__ bias,
                                                         OutT* __restrict__ out, int total_heads, int heads,
                                                         float scale, float out_mul) {
+  using ev8 = typename Vec16<ET>::v8;
   constexpr int kVStride = DEPTH + 8;  // halves per key row of V in LDS
   constexpr int DT = DEPTH / 32;       // 32-wide depth tiles of the output
   __shared__ __attribute__((aligned(16))) half_t Vs[4][64 * kVStride];
@@ -464,17 +482,17 @@ __global__ __launch_bounds__(256, DEPTH == 32 ? 4 : DEPTH == 64 ? 3 : 1) void at
       for (int e = 0; e < 16; e++) st[mt][nt][e] = 0.0f;
 #pragma unroll
   for (int ks = 0; ks < DEPTH / 16; ks++) {
-    half8 kf[2], qf[2];
+    ev8 kf[2], qf[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-      kf[t] = *reinterpret_cast<const half8*>(Kp + (long long)(32 * t + r) * ld + 16 * ks + 8 * g);
-      qf[t] = *reinterpret_cast<const half8*>(Q + (long long)(32 * t + r) * ld + 16 * ks + 8 * g);
+      kf[t] = *reinterpret_cast<const ev8*>(Kp + (long long)(32 * t + r) * ld + 16 * ks + 8 * g);
+      qf[t] = *reinterpret_cast<const ev8*>(Q + (long long)(32 * t + r) * ld + 16 * ks + 8 * g);
     }
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
 #pragma unroll
       for (int nt = 0; nt < 2; nt++)
-        st[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[mt], qf[nt], st[mt][nt], 0, 0, 0);
+        st[mt][nt] = Mfma32(kf[mt], qf[nt], st[mt][nt]);
   }
 
   // Scale, add the smolgen logits, softmax over keys per query column.
@@ -486,8 +504,8 @@ __global__ __launch_bounds__(256, DEPTH == 32 ? 4 : DEPTH == 64 ? 3 : 1) void at
     for (int mt = 0; mt < 2; mt++) {
 #pragma unroll
       for (int bp = 0; bp < 2; bp++) {
-        half8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (bh) bv = *reinterpret_cast<const half8*>(bh + ((nt * 2 + mt) * 2 + bp) * 512 + lane * 8);
+        ev8 bv = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (bh) bv = *reinterpret_cast<const ev8*>(bh + ((nt * 2 + mt) * 2 + bp) * 512 + lane * 8);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           float s = st[mt][nt][bp * 8 + e] * scale + (float)bv[e];
@@ -526,18 +544,18 @@ __global__ __launch_bounds__(256, DEPTH == 32 ? 4 : DEPTH == 64 ? 3 : 1) void at
       for (int e = 0; e < 16; e++) o[nt][dt][e] = 0.0f;
 #pragma unroll
   for (int s = 0; s < 4; s++) {
-    half8 pf[2];
+    ev8 pf[2];
 #pragma unroll
     for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-      for (int e = 0; e < 8; e++) pf[nt][e] = (half_t)st[s / 2][nt][8 * (s % 2) + e];
+      for (int e = 0; e < 8; e++) pf[nt][e] = (ET)st[s / 2][nt][8 * (s % 2) + e];
 #pragma unroll
     for (int dt = 0; dt < DT; dt++) {
-      half8 vf;
+      ev8 vf;
 #pragma unroll
-      for (int e = 0; e < 8; e++) vf[e] = vs[(16 * s + 8 * (e / 4) + 4 * g + (e % 4)) * kVStride + dt * 32 + r];
+      for (int e = 0; e < 8; e++) vf[e] = __builtin_bit_cast(ET, vs[(16 * s + 8 * (e / 4) + 4 * g + (e % 4)) * kVStride + dt * 32 + r]);
 #pragma unroll
-      for (int nt = 0; nt < 2; nt++) o[nt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(pf[nt], vf, o[nt][dt], 0, 0, 0);
+      for (int nt = 0; nt < 2; nt++) o[nt][dt] = Mfma32(pf[nt], vf, o[nt][dt]);
     }
   }
   if (!live) return;
@@ -560,7 +578,7 @@ __global__ __launch_bounds__(256, DEPTH == 32 ? 4 : DEPTH == 64 ? 3 : 1) void at
         if constexpr (sizeof(OutT) == 1) {
           *dst = (uint8_t)(PackFp8x4(o[nt][dt][e] * out_mul, 0.0f, 0.0f, 0.0f) & 0xffu);
         } else {
-          *dst = (half_t)o[nt][dt][e];
+          *dst = __builtin_bit_cast(OutT, (ET)o[nt][dt][e]);
         }
       }
   __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the region is private to this wave
@@ -576,7 +594,7 @@ __global__ __launch_bounds__(256, DEPTH == 32 ? 4 : DEPTH == 64 ? 3 : 1) void at
 }
 }  // namespace
 
-int SmolgenBiasIndex(int q, int k) {
+__host__ __device__ int SmolgenBiasIndex(int q, int k) {
   int nt = q / 32, r = q % 32, mt = k / 32, kk = k % 32;
   int blk = kk / 8, g = (kk % 8) / 4, j = kk % 4;
   int lane = g * 32 + r;
@@ -586,29 +604,33 @@ int SmolgenBiasIndex(int q, int k) {
 namespace {
 template <typename OutT>
 void LaunchAttentionT(const half_t* qkv, const half_t* bias, OutT* out, float out_mul, int batch, int heads, int depth,
-                      float scale, hipStream_t stream) {
+                      float scale, hipStream_t stream, bool bf16 = false) {
   const int total = batch * heads;
   if (total <= 0) return;
   const dim3 grid((total + 3) / 4), block(256);
-  switch (depth) {
-    case 32:
-      hipLaunchKernelGGL((attention_kernel<32, OutT>), grid, block, 0, stream, qkv, bias, out, total, heads, scale, out_mul);
-      break;
-    case 64:
-      hipLaunchKernelGGL((attention_kernel<64, OutT>), grid, block, 0, stream, qkv, bias, out, total, heads, scale, out_mul);
-      break;
-    default:  // 128; callers check the depth
-      hipLaunchKernelGGL((attention_kernel<128, OutT>), grid, block, 0, stream, qkv, bias, out, total, heads, scale, out_mul);
-      break;
+  auto launch = [&](auto depth_tag, auto elem_tag) {
+    hipLaunchKernelGGL((attention_kernel<decltype(depth_tag)::value, OutT, decltype(elem_tag)>), grid, block, 0, stream, qkv,
+                       bias, out, total, heads, scale, out_mul);
+  };
+  auto by_depth = [&](auto elem_tag) {
+    switch (depth) {
+      case 32: launch(std::integral_constant<int, 32>{}, elem_tag); break;
+      case 64: launch(std::integral_constant<int, 64>{}, elem_tag); break;
+      default: launch(std::integral_constant<int, 128>{}, elem_tag); break;   // 128; callers check the depth
+    }
+  };
+  if constexpr (sizeof(OutT) == 2) {
+    if (bf16) return by_depth(bf16_t{});
   }
+  by_depth(half_t{});
 }
 }  // namespace
 
 bool AttentionDepthSupported(int depth) { return depth == 32 || depth == 64 || depth == 128; }
 
 void LaunchAttention(const half_t* qkv, const half_t* bias, half_t* out, int batch, int heads, float scale,
-                     hipStream_t stream, int depth) {
-  LaunchAttentionT<half_t>(qkv, bias, out, 1.0f, batch, heads, depth, scale, stream);
+                     hipStream_t stream, int depth, bool bf16) {
+  LaunchAttentionT<half_t>(qkv, bias, out, 1.0f, batch, heads, depth, scale, stream, bf16);
 }
 
 void LaunchAttentionF8Out(const half_t* qkv, const half_t* bias, uint8_t* out, float out_mul, int batch, int heads,
@@ -620,8 +642,9 @@ void LaunchAttentionF8Out(const half_t* qkv, const half_t* bias, uint8_t* out, f
 // Attention policy tail.
 // ---------------------------------------------------------------------------
 namespace {
+template <typename T>   // element type of kq: half_t, bf16_t or float
 __global__ __launch_bounds__(256) void attn_policy_gather_kernel(const float* __restrict__ logits,
-                                                                 const half_t* __restrict__ kq, int ld_kq,
+                                                                 const T* __restrict__ kq, int ld_kq,
                                                                  int key_off, const float* __restrict__ ppo, int pd,
                                                                  const int16_t* __restrict__ inv_map,
                                                                  float* __restrict__ out) {
@@ -631,20 +654,25 @@ __global__ __launch_bounds__(256) void attn_policy_gather_kernel(const float* __
   // with the loads of the eight products in flight together.
   {
     const int i = wave;
-    const half_t* krow = kq + (long long)(b * 64 + 56) * ld_kq + key_off;
+    const T* krow = kq + (long long)(b * 64 + 56) * ld_kq + key_off;
     float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-    if (((pd | ld_kq | key_off) & 7) == 0) {
+    bool done = false;
+    if constexpr (sizeof(T) == 2) {
+      if (((pd | ld_kq | key_off) & 7) == 0) {
+        done = true;
       for (int c = lane; c < pd / 8; c += 64) {
         const floatx4 p0 = *reinterpret_cast<const floatx4*>(ppo + (long long)i * pd + c * 8);
         const floatx4 p1 = *reinterpret_cast<const floatx4*>(ppo + (long long)i * pd + c * 8 + 4);
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-          const half8 kv = *reinterpret_cast<const half8*>(krow + (long long)j * ld_kq + c * 8);
+          const auto kv = *reinterpret_cast<const typename Vec16<T>::v8*>(krow + (long long)j * ld_kq + c * 8);
 #pragma unroll
           for (int e = 0; e < 4; e++) s[j] += (float)kv[e] * p0[e] + (float)kv[4 + e] * p1[e];
         }
       }
-    } else {
+      }
+    }
+    if (!done) {
       for (int k = lane; k < pd; k += 64) {
         const float pw = ppo[(long long)i * pd + k];
 #pragma unroll
@@ -674,12 +702,144 @@ __global__ __launch_bounds__(256) void attn_policy_gather_kernel(const float* __
 }
 }  // namespace
 
-void LaunchAttnPolicyGather(const float* logits, const half_t* kq, int ld_kq, int key_off, const float* ppo, int pd,
+template <typename T>
+void LaunchAttnPolicyGather(const float* logits, const T* kq, int ld_kq, int key_off, const float* ppo, int pd,
                             const int16_t* inv_map, float* out, int batch, hipStream_t stream) {
   if (batch <= 0) return;
-  hipLaunchKernelGGL(attn_policy_gather_kernel, dim3(batch), dim3(256), 0, stream, logits, kq, ld_kq, key_off, ppo,
+  hipLaunchKernelGGL(attn_policy_gather_kernel<T>, dim3(batch), dim3(256), 0, stream, logits, kq, ld_kq, key_off, ppo,
                      pd, inv_map, out);
 }
+template void LaunchAttnPolicyGather<half_t>(const float*, const half_t*, int, int, const float*, int, const int16_t*,
+                                             float*, int, hipStream_t);
+template void LaunchAttnPolicyGather<bf16_t>(const float*, const bf16_t*, int, int, const float*, int, const int16_t*,
+                                             float*, int, hipStream_t);
+template void LaunchAttnPolicyGather<float>(const float*, const float*, int, int, const float*, int, const int16_t*,
+                                            float*, int, hipStream_t);
+
+// ---------------------------------------------------------------------------
+// Layer norm and attention for any element type and any row length / head depth: the forms the float
+// configuration runs on, and what 16-bit networks fall back to for shapes the tuned kernels above do not take
+// (LayerNorm2DWithSkipConnection, blas/encoder.h:29-66; per-head attention, blas/network_blas.cc:352-439).
+// Plain vector-ALU arithmetic in float; written for generality, not for speed.
+// ---------------------------------------------------------------------------
+namespace {
+// One workgroup per row: y = beta + gamma * (t - mean) / sqrt(var + eps), t = act(x) * alpha + skip.
+template <typename T>
+__global__ __launch_bounds__(256) void layer_norm_generic_kernel(const T* __restrict__ x, const T* skip, T* y,
+                                                                 const float* __restrict__ gamma,
+                                                                 const float* __restrict__ beta, int C, float alpha,
+                                                                 float eps, int pre_act) {
+  __shared__ float red[4];
+  const long long row = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* xr = x + row * C;
+  const T* sr = skip != nullptr ? skip + row * C : nullptr;
+  auto value = [&](int c) {
+    const float t = Activate((float)xr[c], pre_act) * alpha;
+    return sr != nullptr ? t + (float)sr[c] : t;
+  };
+  float sum = 0.0f;
+  for (int c = tid; c < C; c += 256) sum += value(c);
+  sum = WaveSum(sum);
+  if (lane == 0) red[wave] = sum;
+  __syncthreads();
+  const float mean = (red[0] + red[1] + red[2] + red[3]) / (float)C;
+  __syncthreads();
+  float var = 0.0f;
+  for (int c = tid; c < C; c += 256) {
+    const float d = value(c) - mean;
+    var += d * d;
+  }
+  var = WaveSum(var);
+  if (lane == 0) red[wave] = var;
+  __syncthreads();
+  const float den = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)C + eps);
+  // (x, skip and y may alias: every element is read for the last time by the thread that writes it)
+  for (int c = tid; c < C; c += 256) y[row * C + c] = (T)(beta[c] + gamma[c] * (value(c) - mean) * den);
+}
+
+// One workgroup per (sample, head): Q, K, V of the head in LDS as floats, the 64 x 64 scores in LDS, softmax by
+// rows, then P.V. MAXD bounds the head depth (LDS: 64 x (3 MAXD + 66) floats).
+template <typename T, int MAXD>
+__global__ __launch_bounds__(256) void attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ bias,
+                                                                T* __restrict__ out, int heads, int depth,
+                                                                float scale) {
+  constexpr int LD = MAXD + 1;
+  __shared__ float Qs[64 * LD], Ks[64 * LD], Vs[64 * MAXD], S[64 * 65];
+  const int gh = blockIdx.x, b = gh / heads, h = gh - b * heads;
+  const int d_model = heads * depth, ld = 3 * d_model;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* base = qkv + (long long)b * 64 * ld + h * depth;
+  for (int i = tid; i < 64 * depth; i += 256) {
+    const int row = i / depth, d = i - row * depth;
+    const T* src = base + (long long)row * ld + d;
+    Qs[row * LD + d] = (float)src[0];
+    Ks[row * LD + d] = (float)src[d_model];
+    Vs[row * MAXD + d] = (float)src[2 * d_model];
+  }
+  __syncthreads();
+  const T* bh = bias != nullptr ? bias + (long long)gh * 4096 : nullptr;
+  for (int i = tid; i < 4096; i += 256) {
+    const int q = i >> 6, k = i & 63;
+    float acc = 0.0f;
+    for (int d = 0; d < depth; d++) acc = fmaf(Qs[q * LD + d], Ks[k * LD + d], acc);
+    acc *= scale;
+    if (bh != nullptr) acc += (float)bh[SmolgenBiasIndex(q, k)];
+    S[q * 65 + k] = acc;
+  }
+  __syncthreads();
+  for (int q = wave; q < 64; q += 4) {   // lane = key
+    const float v = S[q * 65 + lane];
+    float mx = v;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    const float e = expf(v - mx);
+    const float sum = WaveSum(e);
+    S[q * 65 + lane] = e / sum;
+  }
+  __syncthreads();
+  T* ob = out + (long long)b * 64 * d_model + h * depth;
+  for (int i = tid; i < 64 * depth; i += 256) {
+    const int q = i / depth, d = i - q * depth;
+    float acc = 0.0f;
+    for (int k = 0; k < 64; k++) acc = fmaf(S[q * 65 + k], Vs[k * MAXD + d], acc);
+    ob[(long long)q * d_model + d] = (T)acc;
+  }
+}
+}  // namespace
+
+template <typename T>
+void LaunchLayerNormGeneric(const T* x, const T* skip, T* y, const float* gamma, const float* beta, int rows, int C,
+                            float alpha, float eps, int pre_act, hipStream_t stream) {
+  if (rows <= 0) return;
+  hipLaunchKernelGGL(layer_norm_generic_kernel<T>, dim3(rows), dim3(256), 0, stream, x, skip, y, gamma, beta, C, alpha,
+                     eps, pre_act);
+}
+
+bool AttentionGenericDepthSupported(int depth) { return depth >= 1 && depth <= 128; }
+
+template <typename T>
+void LaunchAttentionGeneric(const T* qkv, const T* bias, T* out, int batch, int heads, int depth, float scale,
+                            hipStream_t stream) {
+  if (batch * heads <= 0) return;
+  if (!AttentionGenericDepthSupported(depth)) throw std::runtime_error("LaunchAttentionGeneric: head depth above 128");
+  const dim3 grid(batch * heads), block(256);
+  if (depth <= 32) {
+    hipLaunchKernelGGL((attention_generic_kernel<T, 32>), grid, block, 0, stream, qkv, bias, out, heads, depth, scale);
+  } else if (depth <= 64) {
+    hipLaunchKernelGGL((attention_generic_kernel<T, 64>), grid, block, 0, stream, qkv, bias, out, heads, depth, scale);
+  } else {
+    hipLaunchKernelGGL((attention_generic_kernel<T, 128>), grid, block, 0, stream, qkv, bias, out, heads, depth, scale);
+  }
+}
+#define LC0MI_INSTANTIATE_GENERIC(T)                                                                                   \
+  template void LaunchLayerNormGeneric<T>(const T*, const T*, T*, const float*, const float*, int, int, float, float, \
+                                          int, hipStream_t);                                                          \
+  template void LaunchAttentionGeneric<T>(const T*, const T*, T*, int, int, int, float, hipStream_t);
+LC0MI_INSTANTIATE_GENERIC(half_t)
+LC0MI_INSTANTIATE_GENERIC(bf16_t)
+LC0MI_INSTANTIATE_GENERIC(float)
+#undef LC0MI_INSTANTIATE_GENERIC
 
 // ---------------------------------------------------------------------------
 // Policy softmax over the legal moves of every sample: what lc0's search wrapper does on the host

@@ -114,8 +114,11 @@ class DeviceArena {
   size_t total_ = 0;
 };
 
+// (Weights and activations of an attention body are typed half_t* whatever the network's element type is: the same
+// storage holds bfloat16 bits with precision=bf16, and twice as many bytes holding floats with precision=fp32. The
+// launch helpers of Mi355xNetwork pick the kernels by dtype_; nothing else dereferences these pointers.)
 struct Linear {
-  half_t* w = nullptr;   // [out][ld] halves, K zero-padded to ld
+  half_t* w = nullptr;   // [out][ld] elements, K zero-padded to ld
   float* b = nullptr;    // [out] or null
   int out = 0, in = 0, ld = 0;
   float* c = nullptr;    // [out] row sums of w, for a layer whose input layer norm is folded into it (GemmArgs::col_c)
@@ -308,6 +311,8 @@ struct ModelState {
   // Policy-head encoder layers (network_blas.cc:836-842): post-LN layers without smolgen on the policy embedding.
   std::vector<EncoderDev> pol_encoders_;
   int pe_heads_ = 0, pe_dmodel_ = 0, pe_dff_ = 0, pe_depth_ = 32, pe_ffn_act_ = kActNone, pol_emb_act_ = kActNone;
+  bool pe_smolgen_ = false;                      // policy encoder layers with smolgen (network_blas.cc:836-842)
+  int pe_sg_hc_ = 0, pe_sg_hs_ = 0, pe_sg_gen_ = 0;
   half_t* pos_enc_ = nullptr;
   float* ppo_ = nullptr;
   int16_t* inv_map_ = nullptr;
@@ -319,6 +324,11 @@ struct ModelState {
   uint8_t* smolgen_w8_ = nullptr;        // e4m3 codes of the shared generator layer (rows in SmolgenBiasIndex order)
   std::vector<float> smolgen_w8_scale_;  // their per-row scales
   int fp8_fp16_layers_ = 0;   // option fp8_fp16_layers: the last that many encoder layers keep fp16 operands
+
+  // Element type of activations and weights (option precision: fp16, bf16, fp32; fp8 is fp16 with e4m3 operands in
+  // the large GEMMs) and its size in bytes.
+  Dtype dtype_ = Dtype::kHalf;
+  size_t es_ = 2;
 
   // Residual tower.
   bool fp32_ = false;
@@ -367,9 +377,13 @@ class Mi355xNetwork : public Network, protected ModelState {
   void BuildResnet(const WeightsFile& file);
   void ForwardDevice(int batch);
   void ForwardAttentionBody(int B);
-  void BuildAttentionPolicy(const PolicyHead& ph, int in_channels);
+  void BuildAttentionPolicy(const NetWeights& w, const PolicyHead& ph, int in_channels);
   void ForwardAttentionPolicy(const half_t* x, int ld_x, int B);
   EncoderDev MakeEncoderLayer(const EncoderLayer& l, int emb, int d_model, int dff);
+  // Smolgen weights of one encoder layer; hc / hs / gen receive (or are checked against) the chain's widths.
+  void LoadSmolgen(const Smolgen& s, int emb, int heads, EncoderDev* e, int* hc, int* hs, int* gen, bool* any);
+  // The shared generator layer smolgen_w (4096 x g), rows in the order the attention kernels read the logits.
+  void EnsureSmolgenGlobal(const NetWeights& w, int g);
   template <typename T>
   void ForwardResnet(int B);
   template <typename T>
@@ -401,7 +415,14 @@ class Mi355xNetwork : public Network, protected ModelState {
     }
     return arena_.Upload(v);
   }
-  half_t* AllocH(size_t n) { return static_cast<half_t*>(arena_.Alloc(n * sizeof(half_t))); }
+  // n elements of the network's element type.
+  half_t* AllocH(size_t n) { return static_cast<half_t*>(arena_.Alloc(n * es_)); }
+  // p advanced by n elements of the network's element type.
+  const half_t* ElemAt(const half_t* p, size_t n) const {
+    return reinterpret_cast<const half_t*>(reinterpret_cast<const char*>(p) + n * es_);
+  }
+  // Uploads values converted to the network's element type.
+  half_t* UploadElems(const std::vector<float>& v);
   float* AllocF(size_t n) { return static_cast<float*>(arena_.Alloc(n * sizeof(float))); }
 
   // Launch helpers (profiling aware).
@@ -412,6 +433,15 @@ class Mi355xNetwork : public Network, protected ModelState {
             const NormFold* fold = nullptr);
   GemmArgs MakeGemmArgs(const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act, bool out_f32,
                         int split_k, bool latency_first, const NormFold* fold) const;
+  // Kernels other than the dense layers, by the network's element type (and, for 16-bit types, by whether the tuned
+  // kernel takes the shape).
+  void LayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows, int C,
+                 float alpha, float eps, hipStream_t st = nullptr, uint8_t* y_f8 = nullptr, float f8_mul = 1.0f);
+  void LayerNormRows(const half_t* x, half_t* y, const float* gamma, const float* beta, int rows, int C,
+                     hipStream_t st);
+  void Attention(const half_t* qkv, const half_t* bias, half_t* out, int B, int heads, int depth, hipStream_t st);
+  void SmolgenChain(const EncoderDev& e, const half_t* x, int emb, int heads, int hc, int hs, int gen, half_t* sg1,
+                    half_t* sg2, half_t* sg3, half_t* sbias, int B, hipStream_t st, bool latency_first);
   bool CanFoldLayerNorms(int B) const;
 
   // ---- per-lane state: streams, activations, recorded graphs ----
@@ -433,6 +463,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   float *ln_stats_a_ = nullptr, *ln_stats_b_ = nullptr;
   half_t *pol_e_ = nullptr, *pol_qk_ = nullptr, *head1_ = nullptr, *head2_ = nullptr;
   half_t *pe_qkv_ = nullptr, *pe_att_ = nullptr, *pe_t_ = nullptr, *pe_ffn_ = nullptr;   // policy encoder scratch
+  half_t *pe_sg1_ = nullptr, *pe_sg2_ = nullptr, *pe_sg3_ = nullptr, *pe_sbias_ = nullptr;
   float *pol_logits_ = nullptr, *d_policy_ = nullptr, *d_wdl_ = nullptr, *d_mlh_ = nullptr;
   // Legal-move softmax: per-sample offsets, policy indices and probabilities.
   int* d_legal_off_ = nullptr;
@@ -544,12 +575,32 @@ Linear Mi355xNetwork::MakeLinear(const Vec& w, const Vec& b, int out, int in, in
   l.out = out;
   l.in = in;
   l.ld = RoundUp(in, pad_to);   // zero padding: the reduction may run over ld
-  std::vector<half_t> h(static_cast<size_t>(out) * l.ld, (half_t)0.0f);
+  std::vector<float> h(static_cast<size_t>(out) * l.ld, 0.0f);
   for (int o = 0; o < out; o++)
-    for (int i = 0; i < in; i++) h[static_cast<size_t>(o) * l.ld + i] = (half_t)w[static_cast<size_t>(o) * in + i];
-  l.w = arena_.Upload(h);
+    for (int i = 0; i < in; i++) h[static_cast<size_t>(o) * l.ld + i] = w[static_cast<size_t>(o) * in + i];
+  l.w = UploadElems(h);
   if (!b.empty()) l.b = arena_.Upload(b);
   return l;
+}
+
+half_t* Mi355xNetwork::UploadElems(const std::vector<float>& v) {
+  if (dtype_ == Dtype::kFloat) return reinterpret_cast<half_t*>(arena_.Upload(v));
+  std::vector<uint16_t> bits(v.size());
+  for (size_t i = 0; i < v.size(); i++) {
+    if (dtype_ == Dtype::kBf16) {   // round to nearest even on the upper 16 bits of the float
+      uint32_t u;
+      std::memcpy(&u, &v[i], 4);
+      if ((u & 0x7fffffffu) > 0x7f800000u) {
+        bits[i] = static_cast<uint16_t>((u >> 16) | 0x40);   // NaN stays NaN
+      } else {
+        bits[i] = static_cast<uint16_t>((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+      }
+    } else {
+      const half_t h = (half_t)v[i];
+      std::memcpy(&bits[i], &h, 2);
+    }
+  }
+  return reinterpret_cast<half_t*>(arena_.Upload(bits));
 }
 
 // A layer that reads layer-normalised rows, prepared for reading the un-normalised rows instead (the consumer
@@ -614,7 +665,23 @@ void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linea
                          int act, bool out_f32, hipStream_t st, int split_k, bool latency_first,
                          const NormFold* fold) {
   if (st == nullptr) st = stream_;
-  const GemmArgs g = MakeGemmArgs(A, lda, lin, C, ldc, M, act, out_f32, split_k, latency_first, fold);
+  if (dtype_ == Dtype::kFloat) {
+    if (split_k != 1 || fold != nullptr) throw Error("internal: split or folded GEMM requested in the float configuration");
+    GemmArgsF32 g;
+    g.A = reinterpret_cast<const float*>(A); g.lda = lda;
+    g.W = reinterpret_cast<const float*>(lin.w); g.ldw = lin.ld;
+    g.C = static_cast<float*>(C); g.ldc = ldc;
+    g.bias = lin.b;
+    g.M = M; g.N = lin.out; g.K = lin.ld;
+    g.act = act;
+    const std::string label = std::string(name) + "|gemm_f32_mfma_32x32x2";
+    Timed(label.c_str(), 2.0 * M * lin.out * lin.in,
+          4.0 * (static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in + static_cast<double>(M) * lin.out),
+          [&] { LaunchGemmF32(g, st); }, st);
+    return;
+  }
+  GemmArgs g = MakeGemmArgs(A, lda, lin, C, ldc, M, act, out_f32, split_k, latency_first, fold);
+  g.bf16 = dtype_ == Dtype::kBf16;
   if (fold != nullptr && fold->parts_out != nullptr) *fold->parts_out = GemmStatsParts(g);
   const double flops = 2.0 * M * lin.out * lin.in;
   const double bytes = 2.0 * (static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in) +
@@ -623,6 +690,60 @@ void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linea
   std::string label = std::string(name) + "|" + GemmVariantName(g);
   if (fold != nullptr) label += fold->skip != nullptr ? "+skip_stats" : "+row_norm";
   Timed(label.c_str(), flops, bytes, [&] { LaunchGemm(g, st); }, st);
+}
+
+void Mi355xNetwork::LayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
+                              int rows, int C, float alpha, float eps, hipStream_t st, uint8_t* y_f8, float f8_mul) {
+  if (st == nullptr) st = stream_;
+  if (dtype_ == Dtype::kFloat) {
+    LaunchLayerNormGeneric<float>(reinterpret_cast<const float*>(x), reinterpret_cast<const float*>(skip),
+                                  reinterpret_cast<float*>(y), gamma, beta, rows, C, alpha, eps, kActNone, st);
+  } else {
+    LaunchLayerNorm(x, skip, y, gamma, beta, rows, C, alpha, eps, st, y_f8, f8_mul, dtype_ == Dtype::kBf16);
+  }
+}
+
+// Layer norm of few, long rows (the two norms of the smolgen chain).
+void Mi355xNetwork::LayerNormRows(const half_t* x, half_t* y, const float* gamma, const float* beta, int rows, int C,
+                                  hipStream_t st) {
+  if (dtype_ == Dtype::kFloat) {
+    LaunchLayerNormGeneric<float>(reinterpret_cast<const float*>(x), nullptr, reinterpret_cast<float*>(y), gamma, beta,
+                                  rows, C, 1.0f, 1e-3f, kActNone, st);
+  } else {
+    LaunchLayerNormRows(nullptr, 0, 0, x, kActNone, nullptr, y, gamma, beta, rows, C, 1.0f, 1e-3f, st,
+                        dtype_ == Dtype::kBf16);
+  }
+}
+
+// Per-head attention: the matrix-core kernel for 16-bit elements and head depth 32, 64 or 128, the general one else.
+void Mi355xNetwork::Attention(const half_t* qkv, const half_t* bias, half_t* out, int B, int heads, int depth,
+                              hipStream_t st) {
+  const float scale = 1.0f / std::sqrt(static_cast<float>(depth));
+  if (dtype_ == Dtype::kFloat) {
+    LaunchAttentionGeneric<float>(reinterpret_cast<const float*>(qkv), reinterpret_cast<const float*>(bias),
+                                  reinterpret_cast<float*>(out), B, heads, depth, scale, st);
+  } else if (AttentionDepthSupported(depth)) {
+    LaunchAttention(qkv, bias, out, B, heads, scale, st, depth, dtype_ == Dtype::kBf16);
+  } else if (dtype_ == Dtype::kBf16) {
+    LaunchAttentionGeneric<bf16_t>(reinterpret_cast<const bf16_t*>(qkv), reinterpret_cast<const bf16_t*>(bias),
+                                   reinterpret_cast<bf16_t*>(out), B, heads, depth, scale, st);
+  } else {
+    LaunchAttentionGeneric<half_t>(qkv, bias, out, B, heads, depth, scale, st);
+  }
+}
+
+// The smolgen chain of one encoder layer, unfused (network_blas.cc:283-347): compression, two dense layers with
+// their row norms, then the shared generator layer, which leaves the logits in sbias (SmolgenBiasIndex order).
+void Mi355xNetwork::SmolgenChain(const EncoderDev& e, const half_t* x, int emb, int heads, int hc, int hs, int gen,
+                                 half_t* sg1, half_t* sg2, half_t* sg3, half_t* sbias, int B, hipStream_t st,
+                                 bool latency_first) {
+  const int T = B * 64;
+  Gemm("gemm_smolgen_compress", x, emb, e.sg_compress, sg1, hc, T, kActNone, false, st, 1, latency_first);
+  Gemm("gemm_smolgen_dense1", sg1, 64 * hc, e.sg_dense1, sg2, hs, B, smolgen_act_, false, st, 1, latency_first);
+  Timed("layer_norm_rows", 0.0, 2.0 * es_ * B * hs, [&] { LayerNormRows(sg2, sg2, e.sg_ln1_g, e.sg_ln1_b, B, hs, st); }, st);
+  Gemm("gemm_smolgen_dense2", sg2, hs, e.sg_dense2, sg3, gen, B, smolgen_act_, false, st, 1, latency_first);
+  Timed("layer_norm_rows", 0.0, 2.0 * es_ * B * gen, [&] { LayerNormRows(sg3, sg3, e.sg_ln2_g, e.sg_ln2_b, B, gen, st); }, st);
+  Gemm("gemm_smolgen_global", sg3, gen / heads, smolgen_w_, sbias, 4096, B * heads, kActNone, false, st, 1, latency_first);
 }
 
 // Whether a pass over B positions can run the encoder stack with its layer norms folded into the GEMMs around
@@ -882,11 +1003,13 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   max_batch_ = options.GetInt("max_batch", 1024);
   if (max_batch_ < 1 || max_batch_ > 4096) throw Error("max_batch must be in 1..4096.");
   const std::string precision = options.GetString("precision", "fp16");
-  if (precision != "fp16" && precision != "fp32" && precision != "fp8") {
-    throw Error("Precision '" + precision + "' is not supported (fp16, fp32 or fp8).");
+  if (precision != "fp16" && precision != "fp32" && precision != "fp8" && precision != "bf16") {
+    throw Error("Precision '" + precision + "' is not supported (fp16, bf16, fp32 or fp8).");
   }
   fp32_ = precision == "fp32";
   fp8_ = precision == "fp8";
+  dtype_ = fp32_ ? Dtype::kFloat : precision == "bf16" ? Dtype::kBf16 : Dtype::kHalf;
+  es_ = fp32_ ? 4 : 2;
   {
     // Which of the four encoder GEMMs use e4m3 operands: names joined by '+'.
     const std::string which = options.GetString("fp8_gemms", "qkv+dense+ffn1+ffn2");
@@ -953,10 +1076,11 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   if (device_ < 0 || device_ >= count) throw Error("Invalid GPU id " + std::to_string(device_) + ".");
   CreateStreams();
   if (attn_body_) {
-    if (fp32_) throw Error("precision=fp32 is available for residual-tower networks only.");
     BuildAttentionBody(file);
   } else if (fp8_) {
     throw Error("precision=fp8 is available for attention-body networks only.");
+  } else if (dtype_ == Dtype::kBf16) {
+    throw Error("precision=bf16 is available for attention-body networks only.");
   } else if (fp32_) {
     BuildResnet<float>(file);
   } else {
@@ -1028,6 +1152,12 @@ void Mi355xNetwork::AllocActivations() {
       pe_att_ = AllocH(T * pe_dmodel_);
       pe_t_ = AllocH(T * pol_emb_);
       pe_ffn_ = AllocH(T * pe_dff_);
+      if (pe_smolgen_) {
+        pe_sg1_ = AllocH(T * pe_sg_hc_);
+        pe_sg2_ = AllocH(static_cast<size_t>(max_batch_) * pe_sg_hs_);
+        pe_sg3_ = AllocH(static_cast<size_t>(max_batch_) * pe_sg_gen_);
+        pe_sbias_ = AllocH(static_cast<size_t>(max_batch_) * pe_heads_ * 4096);
+      }
     }
   }
   if (!attn_body_) {
@@ -1108,8 +1238,49 @@ EncoderDev Mi355xNetwork::MakeEncoderLayer(const EncoderLayer& l, int emb, int d
   return e;
 }
 
+void Mi355xNetwork::LoadSmolgen(const Smolgen& s, int emb, int heads, EncoderDev* e, int* hc_io, int* hs_io, int* gen_io,
+                                bool* any) {
+  const int hc = static_cast<int>(s.compress.size()) / emb;
+  const int hs = static_cast<int>(s.dense1_b.size());
+  const int gen = static_cast<int>(s.dense2_b.size());
+  if (!*any) {
+    *hc_io = hc; *hs_io = hs; *gen_io = gen;
+  } else if (hc != *hc_io || hs != *hs_io || gen != *gen_io) {
+    throw Error("Smolgen layers of different sizes are not supported.");
+  }
+  *any = true;
+  if (hc <= 0 || hc % 8 || hs <= 0 || hs % 8 || gen % heads || (gen / heads) % 8 || hs > 8192 || gen > 8192) {
+    throw Error("Unsupported smolgen sizes.");
+  }
+  e->has_smolgen = true;
+  e->sg_compress = MakeLinear(s.compress, Vec(), hc, emb);
+  e->sg_dense1 = MakeLinear(s.dense1_w, s.dense1_b, hs, 64 * hc);
+  e->sg_dense2 = MakeLinear(s.dense2_w, s.dense2_b, gen, hs);
+  e->sg_ln1_g = UploadN(s.ln1_gammas, hs, "Smolgen layer norm gamma"); e->sg_ln1_b = UploadN(s.ln1_betas, hs, "Smolgen layer norm beta");
+  e->sg_ln2_g = UploadN(s.ln2_gammas, gen, "Smolgen layer norm gamma"); e->sg_ln2_b = UploadN(s.ln2_betas, gen, "Smolgen layer norm beta");
+}
+
+void Mi355xNetwork::EnsureSmolgenGlobal(const NetWeights& w, int g) {
+  if (w.smolgen_w.size() != static_cast<size_t>(4096) * g) throw Error("Global smolgen weights have a wrong size.");
+  if (smolgen_w_.w != nullptr) return;
+  // Rows permuted so that the generated logits come out in the layout the
+  // attention kernel reads with one 16-byte load per lane.
+  Vec perm(w.smolgen_w.size());
+  for (int q = 0; q < 64; q++)
+    for (int k = 0; k < 64; k++)
+      std::memcpy(&perm[static_cast<size_t>(SmolgenBiasIndex(q, k)) * g], &w.smolgen_w[static_cast<size_t>(q * 64 + k) * g],
+                  sizeof(float) * g);
+  smolgen_w_ = MakeLinear(perm, Vec(), 4096, g);
+  if (fp8_ && q_smolgen_) {
+    // One set of codes for all layers; every layer brings the scale of its own operand.
+    LinearF8 shared = MakeLinearF8(perm, 4096, g);
+    smolgen_w8_ = shared.w;
+    smolgen_w8_scale_ = shared.wscale;
+  }
+}
+
 // Attention policy head (network_blas.cc:806-914) on token-major input of in_channels channels.
-void Mi355xNetwork::BuildAttentionPolicy(const PolicyHead& ph, int in_channels) {
+void Mi355xNetwork::BuildAttentionPolicy(const NetWeights& w, const PolicyHead& ph, int in_channels) {
   pol_emb_ = static_cast<int>(ph.ip_pol_b.size());
   pol_d_ = static_cast<int>(ph.ip2_pol_b.size());
   if (pol_emb_ <= 0 || pol_emb_ % 8 || pol_d_ % 8 || pol_d_ <= 0 || in_channels % 8) {
@@ -1124,11 +1295,15 @@ void Mi355xNetwork::BuildAttentionPolicy(const PolicyHead& ph, int in_channels) 
       throw Error("Unsupported policy encoder sizes.");
     }
     pe_depth_ = pe_dmodel_ / pe_heads_;
-    if (!AttentionDepthSupported(pe_depth_)) throw Error("Policy encoder head depth must be 32, 64 or 128.");
+    if (!AttentionGenericDepthSupported(pe_depth_)) throw Error("Policy encoder head depth must be at most 128.");
     for (const EncoderLayer& l : ph.pol_encoder) {
-      if (l.mha.has_smolgen) throw Error("Smolgen in policy encoder layers is not supported.");
-      pol_encoders_.push_back(MakeEncoderLayer(l, pol_emb_, pe_dmodel_, pe_dff_));
+      EncoderDev e = MakeEncoderLayer(l, pol_emb_, pe_dmodel_, pe_dff_);
+      // The reference runs policy encoder layers through the same ForwardEncoderLayer as the body's
+      // (network_blas.cc:836-842), smolgen and the shared generator layer included.
+      if (l.mha.has_smolgen) LoadSmolgen(l.mha.smolgen, pol_emb_, pe_heads_, &e, &pe_sg_hc_, &pe_sg_hs_, &pe_sg_gen_, &pe_smolgen_);
+      pol_encoders_.push_back(e);
     }
+    if (pe_smolgen_) EnsureSmolgenGlobal(w, pe_sg_gen_ / pe_heads_);
   }
   {
     Vec qk_w(ph.ip2_pol_w), qk_b(ph.ip2_pol_b);
@@ -1145,37 +1320,60 @@ void Mi355xNetwork::ForwardAttentionPolicy(const half_t* x, int ld_x, int B) {
   const int T = B * 64;
   Gemm("gemm_policy_embed", x, ld_x, pol_emb_lin_, pol_e_, pol_emb_, T, pol_emb_act_);
   for (const EncoderDev& e : pol_encoders_) {   // alpha 1, eps 1e-6 (network_blas.cc:836-842)
+    const half_t* bias = nullptr;
+    if (e.has_smolgen) {
+      SmolgenChain(e, pol_e_, pol_emb_, pe_heads_, pe_sg_hc_, pe_sg_hs_, pe_sg_gen_, pe_sg1_, pe_sg2_, pe_sg3_, pe_sbias_, B,
+                   stream_, true);
+      bias = pe_sbias_;
+    }
     Gemm("gemm_pol_qkv", pol_e_, pol_emb_, e.qkv, pe_qkv_, 3 * pe_dmodel_, T, kActNone);
-    Timed("attention", 4.0 * 64 * 64 * pe_depth_ * B * pe_heads_, B * pe_heads_ * 2.0 * 4 * 64 * pe_depth_, [&] {
-      LaunchAttention(pe_qkv_, nullptr, pe_att_, B, pe_heads_, 1.0f / std::sqrt(static_cast<float>(pe_depth_)), stream_,
-                      pe_depth_);
-    });
+    Timed("attention", 4.0 * 64 * 64 * pe_depth_ * B * pe_heads_,
+          B * pe_heads_ * (static_cast<double>(es_) * 4 * 64 * pe_depth_ + (bias ? es_ * 4096.0 : 0.0)),
+          [&] { Attention(pe_qkv_, bias, pe_att_, B, pe_heads_, pe_depth_, stream_); });
     Gemm("gemm_pol_dense", pe_att_, pe_dmodel_, e.dense, pe_t_, pol_emb_, T, kActNone);
-    Timed("layer_norm_skip", 0.0, 6.0 * T * pol_emb_, [&] {
-      LaunchLayerNorm(pe_t_, pol_e_, pol_e_, e.ln1_g, e.ln1_b, T, pol_emb_, 1.0f, 1e-6f, stream_);
-    });
+    Timed("layer_norm_skip", 0.0, 3.0 * es_ * T * pol_emb_,
+          [&] { LayerNorm(pe_t_, pol_e_, pol_e_, e.ln1_g, e.ln1_b, T, pol_emb_, 1.0f, 1e-6f); });
     Gemm("gemm_pol_ffn1", pol_e_, pol_emb_, e.ffn1, pe_ffn_, pe_dff_, T, pe_ffn_act_);
     Gemm("gemm_pol_ffn2", pe_ffn_, pe_dff_, e.ffn2, pe_t_, pol_emb_, T, kActNone);
-    Timed("layer_norm_skip", 0.0, 6.0 * T * pol_emb_, [&] {
-      LaunchLayerNorm(pe_t_, pol_e_, pol_e_, e.ln2_g, e.ln2_b, T, pol_emb_, 1.0f, 1e-6f, stream_);
-    });
+    Timed("layer_norm_skip", 0.0, 3.0 * es_ * T * pol_emb_,
+          [&] { LayerNorm(pe_t_, pol_e_, pol_e_, e.ln2_g, e.ln2_b, T, pol_emb_, 1.0f, 1e-6f); });
   }
   Gemm("gemm_policy_qk", pol_e_, pol_emb_, pol_qk_lin_, pol_qk_, 2 * pol_d_, T, kActNone);
-  {
+  // Per-sample Q.K^T / sqrt(d): 64 x 64 logits, float (network_blas.cc:850-872).
+  const float logit_scale = 1.0f / std::sqrt(static_cast<float>(pol_d_));
+  const double logit_flops = 2.0 * 64 * 64 * pol_d_ * B, logit_bytes = B * (2.0 * es_ * 64 * pol_d_ + 4.0 * 4096);
+  if (dtype_ == Dtype::kFloat) {
+    GemmArgsF32 g;
+    g.A = reinterpret_cast<const float*>(pol_qk_); g.lda = 2 * pol_d_; g.strideA = 64LL * 2 * pol_d_;
+    g.W = reinterpret_cast<const float*>(ElemAt(pol_qk_, pol_d_)); g.ldw = 2 * pol_d_; g.strideW = 64LL * 2 * pol_d_;
+    g.C = pol_logits_; g.ldc = 64; g.strideC = 4096;
+    g.M = 64; g.N = 64; g.K = pol_d_; g.batch = B;
+    g.scale = logit_scale;
+    g.act = kActNone;
+    Timed("gemm_policy_logits|gemm_f32_mfma_32x32x2", logit_flops, logit_bytes, [&] { LaunchGemmF32(g, stream_); });
+  } else {
     GemmArgs g;
     g.A = pol_qk_; g.lda = 2 * pol_d_; g.strideA = 64LL * 2 * pol_d_;
     g.W = pol_qk_ + pol_d_; g.ldw = 2 * pol_d_; g.strideW = 64LL * 2 * pol_d_;
     g.C = pol_logits_; g.ldc = 64; g.strideC = 4096;
     g.M = 64; g.N = 64; g.K = pol_d_; g.batch = B;
-    g.scale = 1.0f / std::sqrt(static_cast<float>(pol_d_));
+    g.scale = logit_scale;
     g.act = kActNone;
     g.out_f32 = true;
+    g.bf16 = dtype_ == Dtype::kBf16;
     const std::string label = std::string("gemm_policy_logits|") + GemmVariantName(g);
-    Timed(label.c_str(), 2.0 * 64 * 64 * pol_d_ * B, B * (2.0 * 2 * 64 * pol_d_ + 4.0 * 4096),
-          [&] { LaunchGemm(g, stream_); });
+    Timed(label.c_str(), logit_flops, logit_bytes, [&] { LaunchGemm(g, stream_); });
   }
   Timed("policy_gather", 0.0, B * (4.0 * 4288 + 4.0 * 1858), [&] {
-    LaunchAttnPolicyGather(pol_logits_, pol_qk_, 2 * pol_d_, pol_d_, ppo_, pol_d_, inv_map_, d_policy_, B, stream_);
+    if (dtype_ == Dtype::kFloat) {
+      LaunchAttnPolicyGather(pol_logits_, reinterpret_cast<const float*>(pol_qk_), 2 * pol_d_, pol_d_, ppo_, pol_d_,
+                             inv_map_, d_policy_, B, stream_);
+    } else if (dtype_ == Dtype::kBf16) {
+      LaunchAttnPolicyGather(pol_logits_, reinterpret_cast<const bf16_t*>(pol_qk_), 2 * pol_d_, pol_d_, ppo_, pol_d_,
+                             inv_map_, d_policy_, B, stream_);
+    } else {
+      LaunchAttnPolicyGather(pol_logits_, pol_qk_, 2 * pol_d_, pol_d_, ppo_, pol_d_, inv_map_, d_policy_, B, stream_);
+    }
   });
 }
 
@@ -1199,10 +1397,11 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   d_model_ = static_cast<int>(w.encoder[0].mha.q_b.size());
   dff_ = static_cast<int>(w.encoder[0].ffn.dense1_b.size());
   depth_ = d_model_ / heads_;
-  if (d_model_ != heads_ * depth_ || !AttentionDepthSupported(depth_)) {
-    throw Error("Attention head depth must be 32, 64 or 128 (got " + std::to_string(d_model_) + " / " +
+  if (d_model_ != heads_ * depth_ || !AttentionGenericDepthSupported(depth_)) {
+    throw Error("Attention head depth must be a whole number up to 128 (got " + std::to_string(d_model_) + " / " +
                 std::to_string(heads_) + ").");
   }
+  if (fp8_ && !AttentionDepthSupported(depth_)) throw Error("precision=fp8 needs an attention head depth of 32, 64 or 128.");
   if (dff_ % 8 != 0) throw Error("FFN width must be a multiple of 8.");
   alpha_ = static_cast<float>(std::pow(2.0 * w.encoder.size(), -0.25));
   eps_ = pe_dense_ ? 1e-3f : 1e-6f;   // src/neural/backends/blas/network_blas.cc:719
@@ -1244,10 +1443,7 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     gate_mult_ = UploadF(mult); gate_add_ = UploadF(add);
   }
   {
-    const std::vector<float>& pe = PosEncoding();
-    std::vector<half_t> h(pe.size());
-    for (size_t i = 0; i < pe.size(); i++) h[i] = (half_t)pe[i];
-    pos_enc_ = arena_.Upload(h);
+    pos_enc_ = UploadElems(PosEncoding());
   }
 
   for (const EncoderLayer& l : w.encoder) {
@@ -1277,37 +1473,20 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     if (static_cast<int>(l.ln1_gammas.size()) != emb_ || static_cast<int>(l.ln2_gammas.size()) != emb_) {
       throw Error("Layer norm parameters do not match the embedding size.");
     }
-    e.has_smolgen = l.mha.has_smolgen;
-    if (e.has_smolgen) {
+    if (l.mha.has_smolgen) {
       const Smolgen& s = l.mha.smolgen;
-      const int hc = static_cast<int>(s.compress.size()) / emb_;
-      const int hs = static_cast<int>(s.dense1_b.size());
-      const int gen = static_cast<int>(s.dense2_b.size());
-      if (!any_smolgen_) {
-        sg_hc_ = hc; sg_hs_ = hs; sg_gen_ = gen;
-      } else if (hc != sg_hc_ || hs != sg_hs_ || gen != sg_gen_) {
-        throw Error("Smolgen layers of different sizes are not supported.");
-      }
-      any_smolgen_ = true;
-      if (hc % 8 || hs % 8 || gen % heads_ || (gen / heads_) % 8 || hs > 8192 || gen > 8192) {
-        throw Error("Unsupported smolgen sizes.");
-      }
-      e.sg_compress = MakeLinear(s.compress, Vec(), hc, emb_);
-      e.sg_dense1 = MakeLinear(s.dense1_w, s.dense1_b, hs, 64 * hc);
-      e.sg_dense2 = MakeLinear(s.dense2_w, s.dense2_b, gen, hs);
-      e.sg_ln1_g = UploadN(s.ln1_gammas, hs, "Smolgen layer norm gamma"); e.sg_ln1_b = UploadN(s.ln1_betas, hs, "Smolgen layer norm beta");
-      e.sg_ln2_g = UploadN(s.ln2_gammas, gen, "Smolgen layer norm gamma"); e.sg_ln2_b = UploadN(s.ln2_betas, gen, "Smolgen layer norm beta");
+      LoadSmolgen(s, emb_, heads_, &e, &sg_hc_, &sg_hs_, &sg_gen_, &any_smolgen_);
       if (fp8_ && q_smolgen_) {
-        if ((64 * hc) % 128 || hs % 128 || (gen / heads_) % 128) {
+        if ((64 * sg_hc_) % 128 || sg_hs_ % 128 || (sg_gen_ / heads_) % 128) {
           throw Error("fp8_gemms=smolgen needs smolgen widths (64 x compression, hidden, generator per head) that are "
                       "multiples of 128.");
         }
-        e.sg_compress8 = MakeLinearF8(s.compress, hc, emb_);
-        e.sg_dense18 = MakeLinearF8(s.dense1_w, hs, 64 * hc);
-        e.sg_dense28 = MakeLinearF8(s.dense2_w, gen, hs);
+        e.sg_compress8 = MakeLinearF8(s.compress, sg_hc_, emb_);
+        e.sg_dense18 = MakeLinearF8(s.dense1_w, sg_hs_, 64 * sg_hc_);
+        e.sg_dense28 = MakeLinearF8(s.dense2_w, sg_gen_, sg_hs_);
       }
     }
-    if (fold_layer_norm_ && !fp8_ && emb_ % 8 == 0) {
+    if (fold_layer_norm_ && !fp8_ && dtype_ == Dtype::kHalf && emb_ % 8 == 0) {
       // Folded layer norms (fp16 path): the layers after a norm get its gamma and beta multiplied in, the layers
       // before one get alpha multiplied into their bias (the GEMM scales the sum by alpha).
       const size_t li = encoders_.size();
@@ -1331,20 +1510,8 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   }
   if (any_smolgen_) {
     const int g = sg_gen_ / heads_;
-    if (w.smolgen_w.size() != static_cast<size_t>(4096) * g) throw Error("Global smolgen weights have a wrong size.");
-    // Rows permuted so that the generated logits come out in the layout the
-    // attention kernel reads with one 16-byte load per lane.
-    Vec perm(w.smolgen_w.size());
-    for (int q = 0; q < 64; q++)
-      for (int k = 0; k < 64; k++)
-        std::memcpy(&perm[static_cast<size_t>(SmolgenBiasIndex(q, k)) * g], &w.smolgen_w[static_cast<size_t>(q * 64 + k) * g],
-                    sizeof(float) * g);
-    smolgen_w_ = MakeLinear(perm, Vec(), 4096, g);
+    EnsureSmolgenGlobal(w, g);
     if (fp8_ && q_smolgen_) {
-      // One set of codes for all layers; every layer brings the scale of its own operand.
-      LinearF8 shared = MakeLinearF8(perm, 4096, g);
-      smolgen_w8_ = shared.w;
-      smolgen_w8_scale_ = shared.wscale;
       for (EncoderDev& e : encoders_) {
         if (!e.has_smolgen) continue;
         e.sg_global8.w = smolgen_w8_;
@@ -1352,7 +1519,7 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
         e.sg_global8.col_scale = AllocF(4096);
       }
     }
-    if (fused_smolgen_attention_ && SmolgenAttentionSupported(heads_, depth_, g)) {
+    if (fused_smolgen_attention_ && dtype_ == Dtype::kHalf && SmolgenAttentionSupported(heads_, depth_, g)) {
       // The same weights in the fragment order of the kernel that generates the logits inside the attention.
       std::vector<half_t> frag(w.smolgen_w.size());
       for (int row = 0; row < 4096; row++)
@@ -1365,7 +1532,7 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
   // Heads.
   pol_emb_act_ = default_act_;
   pe_ffn_act_ = ffn_act_;
-  BuildAttentionPolicy(ph, emb_);
+  BuildAttentionPolicy(w, ph, emb_);
 
   val_ch_ = static_cast<int>(vh.ip_val_b.size());
   val_fc_ = static_cast<int>(vh.ip1_val_b.size());
@@ -1434,9 +1601,6 @@ template <typename T>
 void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
   const NetWeights& w = file.weights;
   const NetworkFormat& nf = file.format;
-  if (attn_policy_ && sizeof(T) != 2) {
-    throw Error("The attention policy head on a residual tower needs precision=fp16.");
-  }
   if (w.residual.empty() && w.input.weights.empty()) throw Error("Network has no input convolution.");
   const PolicyHead& ph = w.policy_heads.at(policy_head_);
   const ValueHead& vh = w.value_heads.at(value_head_);
@@ -1512,7 +1676,7 @@ void Mi355xNetwork::BuildResnet(const WeightsFile& file) {
     // encoders' FFN (hard-coded in the reference, network_blas.cc:822-842).
     pol_emb_act_ = kActSelu;
     pe_ffn_act_ = kActSelu;
-    BuildAttentionPolicy(ph, filters_);
+    BuildAttentionPolicy(w, ph, filters_);
   } else if (conv_policy_) {
     res_policy1_ = make_conv(ph.policy1, filters_, filters_);
     const int pol_out = static_cast<int>(ph.policy.biases.size());
@@ -1616,7 +1780,7 @@ void Mi355xNetwork::ForwardResnet(int B) {
   }
   // Policy head.
   if (attn_policy_) {
-    if constexpr (sizeof(T) == 2) ForwardAttentionPolicy(static_cast<const half_t*>(r_x_), filters_, B);
+    ForwardAttentionPolicy(static_cast<const half_t*>(r_x_), filters_, B);
   } else if (conv_policy_) {
     // (the heads above do not touch r_v_, so the tower's last fused transform is still there)
     const bool v2 = WinogradConv<T>("gemm_winograd_policy", res_policy1_, r_x_, nullptr, nullptr, default_act_, r_y_, B,
@@ -1635,31 +1799,54 @@ void Mi355xNetwork::ForwardResnet(int B) {
 // ------------------------------------------------------------------ forward --
 void Mi355xNetwork::ForwardAttentionBody(int B) {
   const int T = B * 64;
+  // Element-typed views of the plane kernels (the activations are half_t* storage whatever the type).
+  auto by_type = [&](auto&& f) {
+    if (dtype_ == Dtype::kFloat) f(static_cast<float*>(nullptr));
+    else if (dtype_ == Dtype::kBf16) f(static_cast<bf16_t*>(nullptr));
+    else f(static_cast<half_t*>(nullptr));
+  };
   if (pe_dense_) {
-    Timed("piece_planes", 0.0, B * (12.0 * 12 + 768.0 * 2), [&] { LaunchPiecePlanes(d_masks_, d_values_, pre_in_, B, stream_); });
+    Timed("piece_planes", 0.0, B * (12.0 * 12 + 768.0 * es_), [&] {
+      by_type([&](auto* tag) {
+        using E = std::remove_pointer_t<decltype(tag)>;
+        LaunchPiecePlanes(d_masks_, d_values_, reinterpret_cast<E*>(pre_in_), B, stream_);
+      });
+    });
     Gemm("gemm_pos_encoding", pre_in_, 768, preproc_lin_, pre_out_, 64 * enc_ch_, B, kActNone);
-    Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * 2 + 64.0 * enc_ch_ * 2), [&] {
-      LaunchExpandPlanesDense(d_masks_, d_values_, pre_out_, enc_ch_, in0_, in_ld_, B, stream_);
+    Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * es_ + 64.0 * enc_ch_ * es_), [&] {
+      by_type([&](auto* tag) {
+        using E = std::remove_pointer_t<decltype(tag)>;
+        LaunchExpandPlanesDense(d_masks_, d_values_, reinterpret_cast<const E*>(pre_out_), enc_ch_,
+                                reinterpret_cast<E*>(in0_), in_ld_, B, stream_);
+      });
     });
   } else {
-    Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * 2),
-          [&] { LaunchExpandPlanesAttn<half_t>(d_masks_, d_values_, pos_enc_, in0_, in_ld_, B, stream_); });
+    Timed("expand_planes", 0.0, B * (112.0 * 12 + 64.0 * in_ld_ * es_), [&] {
+      by_type([&](auto* tag) {
+        using E = std::remove_pointer_t<decltype(tag)>;
+        LaunchExpandPlanesAttn<E>(d_masks_, d_values_, reinterpret_cast<const E*>(pos_enc_), reinterpret_cast<E*>(in0_),
+                                  in_ld_, B, stream_);
+      });
+    });
   }
   Gemm("gemm_embedding", in0_, in_ld_, emb_lin_, x_, emb_, T, default_act_);
   if (pe_dense_) {
-    Timed("layer_norm_skip", 0.0, 4.0 * T * emb_, [&] {
-      LaunchLayerNorm(x_, nullptr, x_, emb_ln_g_, emb_ln_b_, T, emb_, 1.0f, 1e-3f, stream_);
-    });
+    Timed("layer_norm_skip", 0.0, 2.0 * es_ * T * emb_,
+          [&] { LayerNorm(x_, nullptr, x_, emb_ln_g_, emb_ln_b_, T, emb_, 1.0f, 1e-3f); });
   }
   if (gating_) {
-    Timed("input_gating", 0.0, 4.0 * T * emb_, [&] { LaunchInputGating(x_, gate_mult_, gate_add_, B, 64 * emb_, stream_); });
+    Timed("input_gating", 0.0, 2.0 * es_ * T * emb_, [&] {
+      by_type([&](auto* tag) {
+        using E = std::remove_pointer_t<decltype(tag)>;
+        LaunchInputGating(reinterpret_cast<E*>(x_), gate_mult_, gate_add_, B, 64 * emb_, stream_);
+      });
+    });
   }
   if (pe_dense_) {
     Gemm("gemm_emb_ffn1", x_, emb_, emb_ffn1_, ffn_, emb_dff_, T, ffn_act_);
     Gemm("gemm_emb_ffn2", ffn_, emb_dff_, emb_ffn2_, t_, emb_, T, kActNone);
-    Timed("layer_norm_skip", 0.0, 6.0 * T * emb_, [&] {
-      LaunchLayerNorm(t_, x_, x_, emb_ffn_ln_g_, emb_ffn_ln_b_, T, emb_, alpha_, 1e-3f, stream_);
-    });
+    Timed("layer_norm_skip", 0.0, 3.0 * es_ * T * emb_,
+          [&] { LayerNorm(t_, x_, x_, emb_ffn_ln_g_, emb_ffn_ln_b_, T, emb_, alpha_, 1e-3f); });
   }
   // fp8: the large GEMMs read e4m3 operands written by the kernel that produces each tensor. The last
   // fp8_fp16_layers_ layers (closest to the heads) can be kept in fp16.
@@ -1746,6 +1933,8 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
           LaunchQuantizeF8(sg3_, sg3q_, static_cast<long long>(B) * sg_gen_, 1.0f / e.s_sg3, ss);
         }, ss);
         GemmF8("gemm_smolgen_global", sg3q_, smolgen_w_, e.sg_global8, sbias_, B * heads_, kActNone, false, 1.0f, ss);
+      } else if (dtype_ != Dtype::kHalf) {
+        SmolgenChain(e, x_, emb_, heads_, sg_hc_, sg_hs_, sg_gen_, sg1_, sg2_, sg3_, sbias_, B, ss, chain_first);
       } else {
       Gemm("gemm_smolgen_compress", x_, emb_, norm_in ? e.sg_compress_n : e.sg_compress, sg1_, sg_hc_, T, kActNone,
            false, ss, 1, chain_first, norm_in ? &cons_in : nullptr);
@@ -1809,8 +1998,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
           LaunchSmolgenAttention(qkv_, sg3_, smolgen_wfrag_, att_, B, heads_, depth_, gen_sz, att_scale, stream_);
         });
       } else {
-        Timed("attention", att_flops, att_bytes,
-              [&] { LaunchAttention(qkv_, bias, att_, B, heads_, att_scale, stream_, depth_); });
+        Timed("attention", att_flops, att_bytes, [&] { Attention(qkv_, bias, att_, B, heads_, depth_, stream_); });
       }
       if (calibrating_) RecordAbsMax(att_, static_cast<size_t>(T) * d_model_, static_cast<int>(4 * li + 1));
       if (fold) {
@@ -1834,9 +2022,8 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       Gemm("gemm_mha_dense", att_, d_model_, e.dense, t_, emb_, T, kActNone);
     }
     const bool ln1_f8 = f8 && q_ffn1_;
-    Timed("layer_norm_skip", 0.0, (ln1_f8 ? 7.0 : 6.0) * T * emb_, [&] {
-      LaunchLayerNorm(t_, x_, x_, e.ln1_g, e.ln1_b, T, emb_, alpha_, eps_, stream_, ln1_f8 ? xq_ : nullptr,
-                      1.0f / e.s_x1);
+    Timed("layer_norm_skip", 0.0, (ln1_f8 ? 7.0 : 3.0 * es_) * T * emb_, [&] {
+      LayerNorm(t_, x_, x_, e.ln1_g, e.ln1_b, T, emb_, alpha_, eps_, stream_, ln1_f8 ? xq_ : nullptr, 1.0f / e.s_x1);
     });
     if (calibrating_) RecordAbsMax(x_, nx, static_cast<int>(4 * li + 2));
     const bool ffn_f8 = f8 && q_ffn2_;   // FFN2 reads an e4m3 operand
@@ -1858,9 +2045,9 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, t_, emb_, T, kActNone);
     }
     const bool ln2_f8 = f8_any && li + 1 < n_f8_layers && (q_qkv_ || q_smolgen_);   // the next layer reads an e4m3 copy
-    Timed("layer_norm_skip", 0.0, (ln2_f8 ? 7.0 : 6.0) * T * emb_, [&] {
-      LaunchLayerNorm(t_, x_, x_, e.ln2_g, e.ln2_b, T, emb_, alpha_, eps_, stream_, ln2_f8 ? xq_ : nullptr,
-                      last ? 1.0f : 1.0f / encoders_[li + 1].s_x);
+    Timed("layer_norm_skip", 0.0, (ln2_f8 ? 7.0 : 3.0 * es_) * T * emb_, [&] {
+      LayerNorm(t_, x_, x_, e.ln2_g, e.ln2_b, T, emb_, alpha_, eps_, stream_, ln2_f8 ? xq_ : nullptr,
+                last ? 1.0f : 1.0f / encoders_[li + 1].s_x);
     });
     if (calibrating_) RecordAbsMax(x_, nx, static_cast<int>(4 * li + 4));
   }

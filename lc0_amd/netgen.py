@@ -137,7 +137,9 @@ def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_s
     embedding FFN (src/neural/backends/blas/network_blas.cc:612-712) instead of PE_MAP.
     gating: ip_mult_gate / ip_add_gate. multihead: network format 7 with policy heads
     vanilla / optimistic_st / soft (shared embedding) and value heads winner / q / st.
-    pol_encoder = (layers, heads, dff): encoder layers inside the policy head (legacy format only).
+    pol_encoder = (layers, heads, dff[, smolgen]): encoder layers inside the policy head (legacy format only);
+    their optional smolgen = (hidden_channels, hidden_sz, gen_sz) shares the net's smolgen_w, so gen_sz must be
+    the body's.
     """
     g = _Gen(seed)
     d_model = d_model or emb          # heads * head depth
@@ -195,9 +197,10 @@ def attention_body(emb, layers, heads, dff, seed, smolgen=None, std=0.02, bias_s
     else:
         w["ip_pol_w"], w["ip_pol_b"] = fc(policy_d, emb)
         if pol_encoder:
-            n_enc, enc_heads, enc_dff = pol_encoder
-            w["pol_encoder"] = [_encoder_layer(g, policy_d, policy_d, enc_dff, std, bias_std, perturb_ln=perturb_ln)
-                                for _ in range(n_enc)]
+            n_enc, enc_heads, enc_dff = pol_encoder[:3]
+            enc_smolgen = pol_encoder[3] if len(pol_encoder) > 3 else None
+            w["pol_encoder"] = [_encoder_layer(g, policy_d, policy_d, enc_dff, std, bias_std, smolgen=enc_smolgen,
+                                               heads=enc_heads, perturb_ln=perturb_ln) for _ in range(n_enc)]
             w["pol_headcount"] = enc_heads
         w.update(policy_head())
         w.update(value_head())
@@ -311,6 +314,11 @@ CONFIGS = {
     # fp8-capable widths with the dense position encoding, gating and the multi-head format
     "tiny_attn_dense_f8": lambda: attention_body(128, 2, 4, 256, seed=2010, smolgen=(8, 32, 32), perturb_ln=True, std=0.07,
                                                  pe_dense=(16, 128), gating=True, multihead=True),
+    # head depth 48: none of the depths the matrix-core attention kernel takes
+    "tiny_attn_d48": lambda: attention_body(96, 2, 2, 128, seed=2022, smolgen=(8, 32, 32), perturb_ln=True, std=0.08),
+    # smolgen inside the policy head's encoder layer as well (it shares the body's generator layer)
+    "tiny_attn_polenc_sg": lambda: attention_body(64, 2, 2, 96, seed=2023, smolgen=(8, 32, 32), perturb_ln=True, std=0.1,
+                                                  pol_encoder=(1, 2, 96, (8, 32, 32))),
     "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True, std=0.1),
     # ---- what real files contain beyond FLOAT32 layers of the current format ----
     # batch-norm statistics on every convolution block, incl. the bias-less and gamma-less old forms

@@ -666,10 +666,84 @@ def test_head_depth_64_policy_encoders_and_attention_policy_on_a_tower(name, bat
     _compare(res, want, positions["legal"][:batch], logit_frac=0.08 if name == "tiny_resnet_attnpolicy" else None)
 
 
-def test_attention_policy_on_a_tower_needs_fp16():
+@pytest.mark.parametrize("name,batch", [("tiny_attn", 37), ("tiny_attn_dense", 24), ("tiny_attn_d64", 20),
+                                        ("tiny_attn_nosmolgen", 33), ("tiny_resnet_attnpolicy", 19),
+                                        ("c1_attn_10x256", 64)])
+def test_attention_nets_in_fp32_match_oracle_within_1e_3(name, batch, positions):
+    """precision=fp32 on attention bodies (and on the attention policy head of a tower): float weights and
+    activations, fp32 matrix instructions, float layer norm and attention. The reference computes in fp32 throughout
+    (network_blas.cc:271-471); the bar is 1e-3 on softmaxed policy and W/D/L, and the logits within 1e-3 plus 1 % of
+    their spread."""
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    net_w = nr.load(path)
+    kw = dict(policy_head="vanilla", value_head="winner")
+    want = onn.BlasNetwork(net_w, **kw).forward(masks, values)
+    net, res = _run_gpu(path, masks, values, "precision=fp32")
+    _compare(res, want, positions["legal"][:batch], tol=1e-3)
+    net.SetProfiling(True)
+    comp = net.NewComputation()
+    comp.AddInputs(masks, values)
+    comp.ComputeBlocking()
+    names = [k.name for k in net.TakeProfile()]
+    net.SetProfiling(False)
+    assert any("gemm_f32_mfma" in n for n in names) and not any("gemm_dma" in n or "gemm_64x64" in n for n in names), names
+
+
+@pytest.mark.parametrize("name,batch", [("tiny_attn", 37), ("tiny_attn_dense", 24), ("tiny_attn_d64", 20),
+                                        ("c1_attn_10x256", 64), ("c2_bt4_15x1024", 40)])
+def test_attention_nets_in_bf16_match_oracle(name, batch, positions):
+    """precision=bf16: bfloat16 weights and activations on the bf16 matrix instructions (fp32 accumulation, fp32
+    layer-norm statistics and softmax). A bfloat16 carries 8 significant bits against the half's 11, so the fp16
+    bars do not apply; the bounds are about twice what these nets measure: softmaxed policy 2e-3 (measured up to
+    1.6e-4), q and d 3e-2 (1.5e-2), logits 5e-3 plus 20 % of their spread at worst (16 %) and 3 % of it rms (1.4 %),
+    moves-left 5 % (1.6 %). Top-1 agreement with the fp32 oracle is printed (0.95 to 1.0 on 20 to 64 positions)."""
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    _, res = _run_gpu(path, masks, values, "precision=bf16")
+    sm_g, sm_o = onn.softmax_rows(res["policy"]), onn.softmax_rows(want["policy"])
+    legal = positions["legal"][:batch]
+    spread = float(np.concatenate([want["policy"][i, lg] for i, lg in enumerate(legal)]).std())
+    stats = dict(policy_softmax=float(np.abs(sm_g - sm_o).max()), logits=float(np.abs(res["policy"] - want["policy"]).max()),
+                 logit_rms=_legal_logit_rms(res["policy"], want["policy"], legal), spread=spread,
+                 q=float(np.abs(res["q"] - (want["wdl"][:, 0] - want["wdl"][:, 2])).max()),
+                 d=float(np.abs(res["d"] - want["wdl"][:, 1]).max()),
+                 mlh_rel=float((np.abs(res["m"] - want["m"]) / np.maximum(np.abs(want["m"]), 1.0)).max()),
+                 top1=float(np.mean([lg[res["policy"][i, lg].argmax()] == lg[want["policy"][i, lg].argmax()]
+                                     for i, lg in enumerate(legal)])))
+    print("bf16 parity (%s):" % name, stats)
+    assert stats["policy_softmax"] <= 2e-3 and stats["q"] <= 3e-2 and stats["d"] <= 3e-2 and stats["mlh_rel"] <= 0.05
+    assert stats["logits"] <= 5e-3 + 0.2 * spread
+    assert stats["logit_rms"] <= 0.03 * spread
+
+
+@pytest.mark.parametrize("name,options", [("tiny_attn_d48", ""), ("tiny_attn_d48", "precision=bf16"),
+                                          ("tiny_attn_d48", "precision=fp32"), ("tiny_attn_polenc_sg", ""),
+                                          ("tiny_attn_polenc_sg", "precision=fp32")])
+def test_head_depths_and_policy_encoder_smolgen_the_tuned_kernels_do_not_take(name, options, positions):
+    """The reference runs any head depth and runs smolgen in the policy head's encoder layers through the same
+    ForwardEncoderLayer as the body's (network_blas.cc:271-471, 836-842). tiny_attn_d48 has heads of depth 48
+    (general attention kernel instead of the matrix-core one), tiny_attn_polenc_sg a policy encoder layer with
+    smolgen."""
+    batch = 29
+    path = netgen.cached_config(name)
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    _, res = _run_gpu(path, masks, values, options)
+    if "bf16" in options:
+        assert np.abs(onn.softmax_rows(res["policy"]) - onn.softmax_rows(want["policy"])).max() <= 2e-3
+        assert _legal_logit_rms(res["policy"], want["policy"], positions["legal"][:batch]) <= 0.03 * want["policy"].std()
+    else:
+        _compare(res, want, positions["legal"][:batch], tol=1e-3 if "fp32" in options else TOL)
+
+
+def test_precision_options_that_do_not_apply_are_errors():
     from lc0_amd import BackendError, Network
-    with pytest.raises(BackendError, match="precision=fp16"):
-        Network(netgen.cached_config("tiny_resnet_attnpolicy"), "precision=fp32")
+    with pytest.raises(BackendError, match="attention-body networks only"):
+        Network(netgen.cached_config("tiny_resnet"), "precision=bf16")
+    with pytest.raises(BackendError, match="not supported"):
+        Network(netgen.cached_config("tiny_attn"), "precision=int8")
 
 
 @pytest.mark.parametrize("name", ["tiny_attn", "tiny_attn_d64", "tiny_resnet", "tiny_resnet_convpolicy",
