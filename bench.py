@@ -29,6 +29,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 # a run is a small JSON file {"workload", "batch", "source", "kernels": {kernel: bytes per launch}}; when one
 # for this workload and batch is given (or sits under profiles/), roofline.traffic is taken from it, else null.
 def measured_traffic(path, workload, batch, kernel):
+    """(bytes per launch, where they come from). None when there is no record for this workload, batch and kernel,
+    or when the record was measured on other kernel sources than the ones in the tree now (its sources_sha16)."""
     path = path or os.path.join(ROOT, "profiles", "hbm_traffic_%s_batch%d.txt" % (workload, batch))
     try:
         rec = json.load(open(path))
@@ -36,7 +38,12 @@ def measured_traffic(path, workload, batch, kernel):
         return None, None
     if rec.get("workload") != workload or rec.get("batch") != batch:
         return None, None
-    return rec.get("kernels", {}).get(kernel), rec.get("source")
+    from lc0_amd.profile_summary import sources_sha16
+    now = sources_sha16()
+    if rec.get("sources_sha16") != now:
+        return None, "stale: %s was measured on kernel sources %s, the tree holds %s" % (
+            os.path.relpath(path, ROOT), rec.get("sources_sha16"), now)
+    return rec.get("kernels", {}).get(kernel), "%s (sources %s); %s" % (os.path.relpath(path, ROOT), now, rec.get("source"))
 
 
 WORKLOADS = {

@@ -191,7 +191,7 @@ __host__ __device__ int SmolgenBiasIndex(int q, int k);
 bool SmolgenAttentionSupported(int heads, int depth, int gen_sz);
 long long SmolgenFragmentIndex(int row, int col, int gen_sz);
 void LaunchSmolgenAttention(const half_t* qkv, const half_t* gen, const half_t* wfrag, half_t* out, int batch,
-                            int heads, int depth, int gen_sz, float scale, hipStream_t stream);
+                            int heads, int depth, int gen_sz, float scale, hipStream_t stream, bool bf16 = false);
 void LaunchSmolgenAttentionF8Out(const half_t* qkv, const half_t* gen, const half_t* wfrag, uint8_t* out,
                                  float out_mul, int batch, int heads, int depth, int gen_sz, float scale,
                                  hipStream_t stream);

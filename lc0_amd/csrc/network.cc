@@ -1519,13 +1519,13 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
         e.sg_global8.col_scale = AllocF(4096);
       }
     }
-    if (fused_smolgen_attention_ && dtype_ == Dtype::kHalf && SmolgenAttentionSupported(heads_, depth_, g)) {
+    if (fused_smolgen_attention_ && dtype_ != Dtype::kFloat && SmolgenAttentionSupported(heads_, depth_, g)) {
       // The same weights in the fragment order of the kernel that generates the logits inside the attention.
-      std::vector<half_t> frag(w.smolgen_w.size());
+      std::vector<float> frag(w.smolgen_w.size());
       for (int row = 0; row < 4096; row++)
         for (int col = 0; col < g; col++)
-          frag[SmolgenFragmentIndex(row, col, g)] = (half_t)w.smolgen_w[static_cast<size_t>(row) * g + col];
-      smolgen_wfrag_ = arena_.Upload(frag);
+          frag[SmolgenFragmentIndex(row, col, g)] = w.smolgen_w[static_cast<size_t>(row) * g + col];
+      smolgen_wfrag_ = UploadElems(frag);
     }
   }
 
@@ -1882,6 +1882,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       prod_mid.bias = e.dense_ab; prod_mid.scale = alpha_; prod_mid.norm_n = emb_; prod_mid.eps = eps_;
     }
     const bool norm_in = fold && pend_stats != nullptr;   // this layer reads an un-normalised x_
+    const bool bf16 = dtype_ == Dtype::kBf16;
     // The smolgen chain depends only on x: it runs on the side stream next to the
     // QKV projection (on the main stream when profiling, for clean per-kernel times).
     hipStream_t ss = (profiling_ || single_stream_ || B < overlap_min_batch_) ? stream_ : side_stream_;
@@ -1933,7 +1934,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
           LaunchQuantizeF8(sg3_, sg3q_, static_cast<long long>(B) * sg_gen_, 1.0f / e.s_sg3, ss);
         }, ss);
         GemmF8("gemm_smolgen_global", sg3q_, smolgen_w_, e.sg_global8, sbias_, B * heads_, kActNone, false, 1.0f, ss);
-      } else if (dtype_ != Dtype::kHalf) {
+      } else if (dtype_ == Dtype::kFloat) {
         SmolgenChain(e, x_, emb_, heads_, sg_hc_, sg_hs_, sg_gen_, sg1_, sg2_, sg3_, sbias_, B, ss, chain_first);
       } else {
       Gemm("gemm_smolgen_compress", x_, emb_, norm_in ? e.sg_compress_n : e.sg_compress, sg1_, sg_hc_, T, kActNone,
@@ -1946,14 +1947,14 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
              chain_first);
         Timed("layer_norm_rows", 0.0, 4.0 * B * sg_hs_, [&] {
           LaunchLayerNormRows(nullptr, 0, 0, sg2_, kActNone, nullptr, sg2_, e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f,
-                              1e-3f, ss);
+                              1e-3f, ss, bf16);
         }, ss);
       } else {
         const int split = std::max(1, std::min(16, (64 * sg_hc_) / 256));
         Gemm("gemm_smolgen_dense1", sg1_, 64 * sg_hc_, e.sg_dense1, sg2f_, sg_hs_, B, kActNone, true, ss, split);
         Timed("layer_norm_rows", 0.0, (4.0 * split + 2.0) * B * sg_hs_, [&] {
           LaunchLayerNormRows(sg2f_, split, static_cast<long long>(B) * sg_hs_, nullptr, smolgen_act_, nullptr, sg2_,
-                              e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f, 1e-3f, ss);
+                              e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f, 1e-3f, ss, bf16);
         }, ss);
       }
       if (calibrating_ && q_smolgen_) {
@@ -1963,7 +1964,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       Gemm("gemm_smolgen_dense2", sg2_, sg_hs_, e.sg_dense2, sg3_, sg_gen_, B, smolgen_act_, false, ss, 1, chain_first);
       Timed("layer_norm_rows", 0.0, 4.0 * B * sg_gen_, [&] {
         LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f, 1e-3f,
-                            ss);
+                            ss, bf16);
       }, ss);
       if (calibrating_ && q_smolgen_) RecordAbsMax(sg3_, static_cast<size_t>(B) * sg_gen_, SmolgenSlot(li, 2), ss);
       if (!fused_gen) {
@@ -1995,7 +1996,7 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     } else {
       if (fused_gen) {
         Timed("smolgen_attention", att_flops, att_bytes, [&] {
-          LaunchSmolgenAttention(qkv_, sg3_, smolgen_wfrag_, att_, B, heads_, depth_, gen_sz, att_scale, stream_);
+          LaunchSmolgenAttention(qkv_, sg3_, smolgen_wfrag_, att_, B, heads_, depth_, gen_sz, att_scale, stream_, bf16);
         });
       } else {
         Timed("attention", att_flops, att_bytes, [&] { Attention(qkv_, bias, att_, B, heads_, depth_, stream_); });

@@ -23,15 +23,10 @@
 #include <stdexcept>
 #include <type_traits>
 
-#include "device_math.h"
-#include "kernels.h"
+#include "kernel_common.h"
 
 namespace lc0mi {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -66,12 +61,16 @@ __device__ __forceinline__ float Reduce4Rows(float x, F&& op) {
 
 // FULL: 32 heads and an even number of samples, so that every (sample, head) column of every workgroup exists and
 // the loop over head pairs carries no branches (the compiler then overlaps neighbouring pairs).
-template <int NKS, typename OutT, bool FULL>
+// ET: half_t or bf16_t, the type of qkv, gen, wfrag, of the logits kept in LDS and of a 16-bit output (all typed
+// half_t here: the same storage).
+template <int NKS, typename OutT, bool FULL, typename ET>
 __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t* __restrict__ qkv,
                                                                     const half_t* __restrict__ gen,
                                                                     const half_t* __restrict__ wfrag,
                                                                     OutT* __restrict__ out, int batch, int heads,
                                                                     float scale, float out_mul) {
+  using ev8 = typename Vec16<ET>::v8;
+  using ev4 = typename Vec16<ET>::v4;
   constexpr int DEPTH = 32;
   __shared__ __attribute__((aligned(1024))) unsigned char smem[kLogitBytes + 8 * kVBytesPerWave];
   const int lane = threadIdx.x & 63;
@@ -94,8 +93,8 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
     // This wave's four row tiles (two queries x two key halves) are 4 * NKS consecutive fragments of 1 KiB.
     constexpr int NF = 4 * NKS;
     constexpr int PF = NF < 12 ? NF : 12;   // loads in flight per wave
-    const half8* wp = reinterpret_cast<const half8*>(wfrag) + ((long long)(32 * qt + wave * 4) * NKS) * 64 + lane;
-    half8 ring[PF];
+    const ev8* wp = reinterpret_cast<const ev8*>(wfrag) + ((long long)(32 * qt + wave * 4) * NKS) * 64 + lane;
+    ev8 ring[PF];
 #pragma unroll
     for (int f = 0; f < PF; f++) ring[f] = wp[f * 64];
     // The generator vectors of the 64 columns: once per workgroup through LDS (the region phase 2 stages K and V in), 16-byte
@@ -112,13 +111,13 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
       *reinterpret_cast<uint4*>(gl + (c * kSlotsPerCol + (sl ^ (c & (kSlotsPerCol - 1)))) * 16) = v;
     }
     __syncthreads();
-    half8 bf[2][NKS];
+    ev8 bf[2][NKS];
 #pragma unroll
     for (int ct = 0; ct < 2; ct++)
 #pragma unroll
       for (int ks = 0; ks < NKS; ks++) {
         const int c = ct * 32 + r;
-        bf[ct][ks] = *reinterpret_cast<const half8*>(gl + (c * kSlotsPerCol + ((ks * 2 + g) ^ (c & (kSlotsPerCol - 1)))) * 16);
+        bf[ct][ks] = *reinterpret_cast<const ev8*>(gl + (c * kSlotsPerCol + ((ks * 2 + g) ^ (c & (kSlotsPerCol - 1)))) * 16);
       }
     floatx16 acc[2];
 #pragma unroll
@@ -128,10 +127,10 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
 #pragma unroll
         for (int e = 0; e < 16; e++) { acc[0][e] = 0.0f; acc[1][e] = 0.0f; }
       }
-      const half8 a = ring[f % PF];
+      const ev8 a = ring[f % PF];
       if (f + PF < NF) ring[f % PF] = wp[(f + PF) * 64];
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bf[0][ks], acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bf[1][ks], acc[1], 0, 0, 0);
+      acc[0] = Mfma32(a, bf[0][ks], acc[0]);
+      acc[1] = Mfma32(a, bf[1][ks], acc[1]);
       if (ks == NKS - 1) {
         const int rt = wave * 4 + f / NKS;   // row tile within the query group
         const int qq = rt >> 1, mt = rt & 1;
@@ -140,11 +139,11 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
         for (int ct = 0; ct < 2; ct++)
 #pragma unroll
           for (int q4 = 0; q4 < 4; q4++) {
-            half4 hv;
+            ev4 hv;
 #pragma unroll
-            for (int e = 0; e < 4; e++) hv[e] = (half_t)acc[ct][q4 * 4 + e];
+            for (int e = 0; e < 4; e++) hv[e] = (ET)acc[ct][q4 * 4 + e];
             const int u = 8 * mt + 2 * q4 + g;
-            *reinterpret_cast<half4*>(smem + LogitSlot(ct * 32 + r, qq, u & 3, u >> 2)) = hv;
+            *reinterpret_cast<ev4*>(smem + LogitSlot(ct * 32 + r, qq, u & 3, u >> 2)) = hv;
           }
       }
     }
@@ -168,8 +167,8 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
   const int lr = lane >> 3, ch = lane & 7;
   unsigned char* stg = smem + kLogitBytes + wave * kVBytesPerWave;
   struct PairData {
-    half8 k[2][4], v[2][4];   // [32-row tile][8-row group]
-    half8 q[2];               // [head]: query j, depth 8 g4 .. 8 g4 + 7
+    ev8 k[2][4], v[2][4];   // [32-row tile][8-row group]
+    ev8 q[2];               // [head]: query j, depth 8 g4 .. 8 g4 + 7
   };
   auto load_pair = [&](int pi, PairData& d) {
     const int ca = wave * 8 + 2 * pi;
@@ -186,34 +185,34 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const unsigned off = (unsigned)(32 * t + 8 * i) * (unsigned)ld;
-        d.k[t][i] = *reinterpret_cast<const half8*>(Kp + off);
-        d.v[t][i] = *reinterpret_cast<const half8*>(Vp + off);
+        d.k[t][i] = *reinterpret_cast<const ev8*>(Kp + off);
+        d.v[t][i] = *reinterpret_cast<const ev8*>(Vp + off);
       }
     const half_t* Q = base + ha_c * DEPTH + (unsigned)(kQueriesPerGroup * qt + j) * (unsigned)ld + 8u * g4;
-    d.q[0] = *reinterpret_cast<const half8*>(Q);
-    d.q[1] = *reinterpret_cast<const half8*>(Q + (has_b ? DEPTH : 0));
+    d.q[0] = *reinterpret_cast<const ev8*>(Q);
+    d.q[1] = *reinterpret_cast<const ev8*>(Q + (has_b ? DEPTH : 0));
   };
   // fr[head][16-row half]: rows of the staged tile in operand layout (lane j = row of the half, g4 = 8-half group)
-  auto stage_tile = [&](const half8 (&raw)[4], half8 (&fr)[2][2]) {
+  auto stage_tile = [&](const ev8 (&raw)[4], ev8 (&fr)[2][2]) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int row = 8 * i + lr;
-      *reinterpret_cast<half8*>(stg + row * 128 + ((ch ^ ((row >> 1) & 7)) * 16)) = raw[i];
+      *reinterpret_cast<ev8*>(stg + row * 128 + ((ch ^ ((row >> 1) & 7)) * 16)) = raw[i];
     }
 #pragma unroll
     for (int hb = 0; hb < 2; hb++)
 #pragma unroll
       for (int th = 0; th < 2; th++) {
         const int row = 16 * th + j, c = hb * 4 + g4;
-        fr[hb][th] = *reinterpret_cast<const half8*>(stg + row * 128 + ((c ^ ((row >> 1) & 7)) * 16));
+        fr[hb][th] = *reinterpret_cast<const ev8*>(stg + row * 128 + ((c ^ ((row >> 1) & 7)) * 16));
       }
   };
   // Identity fragments: B operand of the transposing product, element (k, column) = [k == 16 dt + column].
-  half8 ident[2];
+  ev8 ident[2];
 #pragma unroll
   for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-    for (int e = 0; e < 8; e++) ident[dt][e] = (8 * g4 + e == 16 * dt + j) ? (half_t)1.0f : (half_t)0.0f;
+    for (int e = 0; e < 8; e++) ident[dt][e] = (8 * g4 + e == 16 * dt + j) ? (ET)1.0f : (ET)0.0f;
   const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
   PairData cur, nxt;
@@ -231,20 +230,20 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
       floatx4 st[2][4];
 #pragma unroll
       for (int tt = 0; tt < 2; tt++) {
-        half8 kf[2][2];
+        ev8 kf[2][2];
         stage_tile(cur.k[tt], kf);
 #pragma unroll
         for (int hb = 0; hb < 2; hb++)
 #pragma unroll
           for (int th = 0; th < 2; th++)
-            st[hb][2 * tt + th] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[hb][th], cur.q[hb], zero4, 0, 0, 0);
+            st[hb][2 * tt + th] = Mfma16(kf[hb][th], cur.q[hb], zero4);
       }
       // V^T of both heads as halves in operand layout: vt[head][depth half][32-key step], lane (depth index, g4),
       // elements = keys 32 s + 4 g4 + (0..3) and 32 s + 16 + 4 g4 + (0..3), the order of the P operand below
-      half8 vt[2][2][2];
+      ev8 vt[2][2][2];
 #pragma unroll
       for (int tt = 0; tt < 2; tt++) {
-        half8 vr[2][2];
+        ev8 vr[2][2];
         stage_tile(cur.v[tt], vr);
 #pragma unroll
         for (int hb = 0; hb < 2; hb++)
@@ -252,9 +251,9 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
           for (int dt = 0; dt < 2; dt++)
 #pragma unroll
             for (int th = 0; th < 2; th++) {
-              const floatx4 tr = __builtin_amdgcn_mfma_f32_16x16x32_f16(vr[hb][th], ident[dt], zero4, 0, 0, 0);
+              const floatx4 tr = Mfma16(vr[hb][th], ident[dt], zero4);
 #pragma unroll
-              for (int e = 0; e < 4; e++) vt[hb][dt][tt][4 * th + e] = (half_t)tr[e];
+              for (int e = 0; e < 4; e++) vt[hb][dt][tt][4 * th + e] = (ET)tr[e];
             }
       }
 #pragma unroll
@@ -262,8 +261,8 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
         if (hb == 1 && !live_b) break;
         const int c = ca + hb;
         // scale, add the logits, softmax over the 64 keys of this lane's query: 16 here, 48 in the lanes 16, 32, 48 away
-        const half8 lg0 = *reinterpret_cast<const half8*>(smem + LogitSlot(c, j, g4, 0));
-        const half8 lg1 = *reinterpret_cast<const half8*>(smem + LogitSlot(c, j, g4, 2));
+        const ev8 lg0 = *reinterpret_cast<const ev8*>(smem + LogitSlot(c, j, g4, 0));
+        const ev8 lg1 = *reinterpret_cast<const ev8*>(smem + LogitSlot(c, j, g4, 2));
         float sv[16];
         float mx = -3.0e38f;
 #pragma unroll
@@ -284,26 +283,26 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
         }
         sum = Reduce4Rows(sum, [](float a, float b) { return a + b; });
         const float inv = __builtin_amdgcn_rcpf(sum);   // 1 ulp
-        half8 pf[2];
+        ev8 pf[2];
 #pragma unroll
         for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
-          for (int e = 0; e < 8; e++) pf[s2][e] = (half_t)sv[8 * s2 + e];
+          for (int e = 0; e < 8; e++) pf[s2][e] = (ET)sv[8 * s2 + e];
         // O^T = V^T . P^T: lane (query j, g4), register e = depth index 16 dt + 4 g4 + e
         OutT* O = out + (long long)(b * 64 + kQueriesPerGroup * qt + j) * d_model + (ha + hb) * DEPTH + 4 * g4;
 #pragma unroll
         for (int dt = 0; dt < 2; dt++) {
           floatx4 o = zero4;
 #pragma unroll
-          for (int s2 = 0; s2 < 2; s2++) o = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt[hb][dt][s2], pf[s2], o, 0, 0, 0);
+          for (int s2 = 0; s2 < 2; s2++) o = Mfma16(vt[hb][dt][s2], pf[s2], o);
           if constexpr (sizeof(OutT) == 1) {
             const float m = inv * out_mul;
             *reinterpret_cast<unsigned*>(O + 16 * dt) = PackFp8x4(o[0] * m, o[1] * m, o[2] * m, o[3] * m);
           } else {
-            half4 h4;
+            ev4 h4;
 #pragma unroll
-            for (int e = 0; e < 4; e++) h4[e] = (half_t)(o[e] * inv);
-            *reinterpret_cast<half4*>(O + 16 * dt) = h4;
+            for (int e = 0; e < 4; e++) h4[e] = (ET)(o[e] * inv);
+            *reinterpret_cast<ev4*>(O + 16 * dt) = h4;
           }
         }
       }
@@ -314,7 +313,7 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
 
 template <typename OutT>
 void LaunchT(const half_t* qkv, const half_t* gen, const half_t* wfrag, OutT* out, float out_mul, int batch, int heads,
-             int depth, int gen_sz, float scale, hipStream_t stream) {
+             int depth, int gen_sz, float scale, hipStream_t stream, bool bf16 = false) {
   if (!SmolgenAttentionSupported(heads, depth, gen_sz)) {
     throw std::runtime_error("LaunchSmolgenAttention: unsupported shape");
   }
@@ -323,8 +322,15 @@ void LaunchT(const half_t* qkv, const half_t* gen, const half_t* wfrag, OutT* ou
   const dim3 grid(((pairs + 7) / 8) * 32), block(512);
   const bool full = heads == 32 && batch % 2 == 0;
   auto launch = [&](auto nks_tag, auto full_tag) {
-    hipLaunchKernelGGL((smolgen_attention_kernel<decltype(nks_tag)::value, OutT, decltype(full_tag)::value>), grid, block, 0,
-                       stream, qkv, gen, wfrag, out, batch, heads, scale, out_mul);
+    if constexpr (sizeof(OutT) == 2) {
+      if (bf16) {
+        hipLaunchKernelGGL((smolgen_attention_kernel<decltype(nks_tag)::value, OutT, decltype(full_tag)::value, bf16_t>), grid,
+                           block, 0, stream, qkv, gen, wfrag, out, batch, heads, scale, out_mul);
+        return;
+      }
+    }
+    hipLaunchKernelGGL((smolgen_attention_kernel<decltype(nks_tag)::value, OutT, decltype(full_tag)::value, half_t>), grid,
+                       block, 0, stream, qkv, gen, wfrag, out, batch, heads, scale, out_mul);
   };
   auto by_width = [&](auto full_tag) {
     switch (gen_sz) {
@@ -350,8 +356,8 @@ long long SmolgenFragmentIndex(int row, int col, int gen_sz) {
 }
 
 void LaunchSmolgenAttention(const half_t* qkv, const half_t* gen, const half_t* wfrag, half_t* out, int batch,
-                            int heads, int depth, int gen_sz, float scale, hipStream_t stream) {
-  LaunchT<half_t>(qkv, gen, wfrag, out, 1.0f, batch, heads, depth, gen_sz, scale, stream);
+                            int heads, int depth, int gen_sz, float scale, hipStream_t stream, bool bf16) {
+  LaunchT<half_t>(qkv, gen, wfrag, out, 1.0f, batch, heads, depth, gen_sz, scale, stream, bf16);
 }
 
 void LaunchSmolgenAttentionF8Out(const half_t* qkv, const half_t* gen, const half_t* wfrag, uint8_t* out,
