@@ -1,6 +1,6 @@
 """Benchmark of the NN-evaluation hot path on one MI355X.
 
-Metric (BASELINE.json): NN evals/sec at batch 256 on the BT4-shape fp16 net,
+Metric: NN evals/sec at batch 256 on the BT4-shape fp16 net,
 with the dominant kernel's fraction of the MFMA roofline and the CPU oracle's
 evals/sec on the same host next to it. A "step" is one device pass over one
 batch of 256 seeded random-playout positions already resident in HBM: `value` is
@@ -56,6 +56,9 @@ WORKLOADS = {
     "c4_bt4_fp8": dict(batch=1024, net="c2_bt4_15x1024", options="precision=fp8", dtype="fp8_e4m3",
                        desc="BT4-shape attention body with e4m3 operands (fp32 accumulation) in the QKV, attention-output "
                             "and FFN GEMMs; weights scaled per output row, activations per tensor; the rest fp16"),
+    "c2_bt4_bf16": dict(batch=256, net="c2_bt4_15x1024", options="precision=bf16", dtype="bf16",
+                        desc="BT4-shape attention body as c2_bt4_15x1024 with bfloat16 weights and activations "
+                             "(bf16 matrix instructions, fp32 accumulation)"),
     "bt4_dense_15x1024": dict(batch=256, desc="BT4 as published: PE_DENSE embedding (64 channels, embedding FFN 1536), "
                                               "15 layers, d=1024, 32 heads, dff 1536, smolgen, multi-head format, fp16"),
     "tiny_attn": dict(batch=64, desc="tiny smolgen attention body (test net)"),

@@ -103,8 +103,9 @@ int lc0mi_net_take_profile(lc0mi_net* net, char* buf, int cap);
 int lc0mi_net_time_resident_forward(lc0mi_net* net, int batch, int iters, double* ms_per_pass);
 
 /* ---- fp8 configuration (backend option precision=fp8, attention-body nets) ----
- * The four large GEMMs of every encoder layer run on e4m3 operands: weights with one scale per
- * output row (absmax / 448), activations with one scale per tensor taken from a calibration pass
+ * The four large GEMMs of every encoder layer (and by default the smolgen chain, option fp8_gemms) run on e4m3
+ * operands: weights with one scale per output row (absmax / 448), activations with one scale per tensor taken from a
+ * calibration pass
  * (the reference reaches fp8 only by handing the whole graph to MIGraphX,
  * src/neural/backends/onnx/network_onnx.cc:757, and converts with src/utils/fp8_utils.h:111-155). At creation the network calibrates
  * itself on built-in pseudo-positions; this call replaces those scales with ones derived from n

@@ -47,6 +47,18 @@ int lc0mi_k_gemm_norm_consumer(const uint16_t* U, int ldu, const uint16_t* W, in
  * 6 row panels of 16x16 to 64x32 outputs, 7 direct-to-LDS 128x64x64, 8 unused (automatic choice), 9 direct-to-LDS
  * 128x32x64, 10 direct-to-LDS 64x64x64). */
 int lc0mi_k_set_gemm_variant(int variant);
+/* Test hook, process-wide: from now on the 16-bit buffers of lc0mi_k_gemm, lc0mi_k_layer_norm, lc0mi_k_layer_norm_rows,
+ * lc0mi_k_attention and lc0mi_k_smolgen_attention (half output) hold bfloat16 values and the kernels run their bf16
+ * instances (precision=bf16 of the network; the reference's type: src/utils/bf16_utils.h). 0 switches back to half. */
+int lc0mi_k_set_bf16(int on);
+/* The general attention and layer norm kernels (any element type, head depth up to 128, any row length): dtype 0 half,
+ * 1 bfloat16, 2 float for qkv / bias / out and x / skip / y. Same contracts as lc0mi_k_attention (bias [b][h][q][k])
+ * and lc0mi_k_layer_norm, with an activation (lc0's numbering) applied to x first. Counterparts in the reference:
+ * src/neural/backends/blas/network_blas.cc:352-439, src/neural/backends/blas/encoder.h:29-66. */
+int lc0mi_k_attention_generic(int dtype, const void* qkv, const void* bias, int batch, int heads, int depth, float scale,
+                              void* out);
+int lc0mi_k_layer_norm_generic(int dtype, const void* x, const void* skip, const float* gamma, const float* beta, int rows,
+                               int C, float alpha, float eps, int pre_act, void* y);
 /* float variant (fp32 configuration). */
 int lc0mi_k_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, int M, int N, int K,
                      float scale, int act, float* C, int ldc);

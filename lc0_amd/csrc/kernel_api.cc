@@ -80,7 +80,17 @@ int Guard(F&& f) {
 }
 }  // namespace
 
+namespace {
+// Test hook (lc0mi_k_set_bf16): the 16-bit buffers of the entry points that say so hold bfloat16 instead of half.
+bool g_bf16 = false;
+}  // namespace
+
 extern "C" {
+
+int lc0mi_k_set_bf16(int on) {
+  g_bf16 = on != 0;
+  return 0;
+}
 
 int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* W, int ldw, long long strideW,
                  const float* bias, int M, int N, int K, int batch, float scale, int act, int out_f32, void* C,
@@ -101,6 +111,7 @@ int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* 
     K_CHECK(hipMemcpy(g.C, C, c_elems * c_size, hipMemcpyHostToDevice));
     g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
     g.M = M; g.N = N; g.K = K; g.batch = batch; g.scale = scale; g.act = act; g.out_f32 = out_f32 != 0;
+    g.bf16 = g_bf16;
     lc0mi::LaunchGemm(g, nullptr);
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());
@@ -225,7 +236,7 @@ int lc0mi_k_layer_norm_rows(const float* x_f32, const uint16_t* x_f16, int pre_a
     auto* dy = reinterpret_cast<half_t*>(dev.Alloc(n * 2));
     float* dg = dev.Put(gamma, (size_t)C);
     float* db = dev.Put(beta, (size_t)C);
-    lc0mi::LaunchLayerNormRows(dxf, dxf ? 1 : 0, 0, dxh, pre_act, ds, dy, dg, db, rows, C, alpha, eps, nullptr);
+    lc0mi::LaunchLayerNormRows(dxf, dxf ? 1 : 0, 0, dxh, pre_act, ds, dy, dg, db, rows, C, alpha, eps, nullptr, g_bf16);
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());
     K_CHECK(hipMemcpy(y, dy, n * 2, hipMemcpyDeviceToHost));
@@ -270,7 +281,7 @@ int lc0mi_k_layer_norm(const uint16_t* x, const uint16_t* skip, const float* gam
     auto* dy = reinterpret_cast<half_t*>(dev.Alloc(n * 2));
     float* dg = dev.Put(gamma, (size_t)C);
     float* db = dev.Put(beta, (size_t)C);
-    lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr);
+    lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr, nullptr, 1.0f, g_bf16);
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());
     K_CHECK(hipMemcpy(y, dy, n * 2, hipMemcpyDeviceToHost));
@@ -297,13 +308,86 @@ int lc0mi_k_attention(const uint16_t* qkv, const uint16_t* bias, int batch, int 
       db = reinterpret_cast<half_t*>(dev.Put(perm.data(), perm.size()));
     }
     auto* dout = reinterpret_cast<half_t*>(dev.Alloc((size_t)batch * 64 * d * 2));
-    lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr, depth);
+    lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr, depth, g_bf16);
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());
     K_CHECK(hipMemcpy(out, dout, (size_t)batch * 64 * d * 2, hipMemcpyDeviceToHost));
     if (time_iters > 0 && ms) {
       *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchAttention(dq, db, dout, batch, heads, scale, nullptr, depth); });
     }
+  });
+}
+
+int lc0mi_k_attention_generic(int dtype, const void* qkv, const void* bias, int batch, int heads, int depth, float scale,
+                              void* out) {
+  return Guard([&] {
+    RequireDevice();
+    if (batch < 1 || heads < 1 || !lc0mi::AttentionGenericDepthSupported(depth) || dtype < 0 || dtype > 2) {
+      throw Error("bad attention shape");
+    }
+    Dev dev;
+    const size_t es = dtype == 2 ? 4 : 2;
+    const size_t d = (size_t)heads * depth;
+    void* dq = dev.Alloc((size_t)batch * 64 * 3 * d * es);
+    K_CHECK(hipMemcpy(dq, qkv, (size_t)batch * 64 * 3 * d * es, hipMemcpyHostToDevice));
+    void* db = nullptr;
+    if (bias) {   // natural [b][h][q][k] order in, the kernels' order on the device
+      std::vector<char> perm((size_t)batch * heads * 4096 * es);
+      const char* src = static_cast<const char*>(bias);
+      for (size_t bh = 0; bh < (size_t)batch * heads; bh++)
+        for (int q = 0; q < 64; q++)
+          for (int k = 0; k < 64; k++)
+            std::memcpy(&perm[(bh * 4096 + lc0mi::SmolgenBiasIndex(q, k)) * es], src + (bh * 4096 + q * 64 + k) * es, es);
+      db = dev.Alloc(perm.size());
+      K_CHECK(hipMemcpy(db, perm.data(), perm.size(), hipMemcpyHostToDevice));
+    }
+    void* dout = dev.Alloc((size_t)batch * 64 * d * es);
+    if (dtype == 2) {
+      lc0mi::LaunchAttentionGeneric(static_cast<const float*>(dq), static_cast<const float*>(db), static_cast<float*>(dout),
+                                    batch, heads, depth, scale, nullptr);
+    } else if (dtype == 1) {
+      lc0mi::LaunchAttentionGeneric(static_cast<const lc0mi::bf16_t*>(dq), static_cast<const lc0mi::bf16_t*>(db),
+                                    static_cast<lc0mi::bf16_t*>(dout), batch, heads, depth, scale, nullptr);
+    } else {
+      lc0mi::LaunchAttentionGeneric(static_cast<const half_t*>(dq), static_cast<const half_t*>(db),
+                                    static_cast<half_t*>(dout), batch, heads, depth, scale, nullptr);
+    }
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(out, dout, (size_t)batch * 64 * d * es, hipMemcpyDeviceToHost));
+  });
+}
+
+int lc0mi_k_layer_norm_generic(int dtype, const void* x, const void* skip, const float* gamma, const float* beta, int rows,
+                               int C, float alpha, float eps, int pre_act, void* y) {
+  return Guard([&] {
+    RequireDevice();
+    if (rows < 1 || C < 1 || dtype < 0 || dtype > 2) throw Error("bad layer norm shape");
+    Dev dev;
+    const size_t bytes = (size_t)rows * C * (dtype == 2 ? 4 : 2);
+    void* dx = dev.Alloc(bytes);
+    K_CHECK(hipMemcpy(dx, x, bytes, hipMemcpyHostToDevice));
+    void* ds = nullptr;
+    if (skip) {
+      ds = dev.Alloc(bytes);
+      K_CHECK(hipMemcpy(ds, skip, bytes, hipMemcpyHostToDevice));
+    }
+    const float* dg = dev.Put(gamma, (size_t)C);
+    const float* db = dev.Put(beta, (size_t)C);
+    void* dy = dev.Alloc(bytes);
+    if (dtype == 2) {
+      lc0mi::LaunchLayerNormGeneric(static_cast<const float*>(dx), static_cast<const float*>(ds), static_cast<float*>(dy), dg,
+                                    db, rows, C, alpha, eps, pre_act, nullptr);
+    } else if (dtype == 1) {
+      lc0mi::LaunchLayerNormGeneric(static_cast<const lc0mi::bf16_t*>(dx), static_cast<const lc0mi::bf16_t*>(ds),
+                                    static_cast<lc0mi::bf16_t*>(dy), dg, db, rows, C, alpha, eps, pre_act, nullptr);
+    } else {
+      lc0mi::LaunchLayerNormGeneric(static_cast<const half_t*>(dx), static_cast<const half_t*>(ds),
+                                    static_cast<half_t*>(dy), dg, db, rows, C, alpha, eps, pre_act, nullptr);
+    }
+    K_CHECK(hipDeviceSynchronize());
+    K_CHECK(hipGetLastError());
+    K_CHECK(hipMemcpy(y, dy, bytes, hipMemcpyDeviceToHost));
   });
 }
 
@@ -597,7 +681,8 @@ int lc0mi_k_smolgen_attention(const uint16_t* qkv, const uint16_t* gen, const ui
         lc0mi::LaunchSmolgenAttentionF8Out(dq, dg, dw, static_cast<uint8_t*>(dout), out_mul, batch, heads, 32, gen_sz,
                                            scale, nullptr);
       } else {
-        lc0mi::LaunchSmolgenAttention(dq, dg, dw, static_cast<half_t*>(dout), batch, heads, 32, gen_sz, scale, nullptr);
+        lc0mi::LaunchSmolgenAttention(dq, dg, dw, static_cast<half_t*>(dout), batch, heads, 32, gen_sz, scale, nullptr,
+                                      g_bf16);
       }
     };
     launch();

@@ -321,6 +321,7 @@ struct ModelState {
   bool fp8_ = false;
   bool q_qkv_ = true, q_dense_ = true, q_ffn1_ = true, q_ffn2_ = true;   // option fp8_gemms
   bool q_smolgen_ = false;   // ... +smolgen: the four layers of the smolgen chain as well
+  bool q_smolgen_auto_ = false;   // fp8_gemms=auto: the chain too, if its widths are multiples of 128
   uint8_t* smolgen_w8_ = nullptr;        // e4m3 codes of the shared generator layer (rows in SmolgenBiasIndex order)
   std::vector<float> smolgen_w8_scale_;  // their per-row scales
   int fp8_fp16_layers_ = 0;   // option fp8_fp16_layers: the last that many encoder layers keep fp16 operands
@@ -1011,9 +1012,14 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   dtype_ = fp32_ ? Dtype::kFloat : precision == "bf16" ? Dtype::kBf16 : Dtype::kHalf;
   es_ = fp32_ ? 4 : 2;
   {
-    // Which of the four encoder GEMMs use e4m3 operands: names joined by '+'.
-    const std::string which = options.GetString("fp8_gemms", "qkv+dense+ffn1+ffn2");
+    // Which layers of an encoder use e4m3 operands: names joined by '+'. The default, "auto", takes the four large
+    // GEMMs and the smolgen chain where the chain's widths allow it (multiples of 128: the e4m3 k-tile).
+    std::string which = options.GetString("fp8_gemms", "auto");
     q_qkv_ = q_dense_ = q_ffn1_ = q_ffn2_ = q_smolgen_ = false;
+    if (which == "auto") {
+      which = "qkv+dense+ffn1+ffn2";
+      q_smolgen_auto_ = true;
+    }
     size_t pos = 0;
     while (pos <= which.size()) {
       const size_t end = std::min(which.find('+', pos), which.size());
@@ -1446,6 +1452,15 @@ void Mi355xNetwork::BuildAttentionBody(const WeightsFile& file) {
     pos_enc_ = UploadElems(PosEncoding());
   }
 
+  if (fp8_ && q_smolgen_auto_) {
+    for (const EncoderLayer& l : w.encoder) {
+      if (!l.mha.has_smolgen) continue;
+      const Smolgen& sg = l.mha.smolgen;
+      const size_t hc64 = 64 * (sg.compress.size() / emb_), hs = sg.dense1_b.size(), g = sg.dense2_b.size() / heads_;
+      q_smolgen_ = hc64 % 128 == 0 && hs % 128 == 0 && g % 128 == 0 && sg.dense2_b.size() % heads_ == 0;
+      break;
+    }
+  }
   for (const EncoderLayer& l : w.encoder) {
     EncoderDev e;
     if (static_cast<int>(l.mha.q_b.size()) != d_model_ || static_cast<int>(l.ffn.dense1_b.size()) != dff_) {

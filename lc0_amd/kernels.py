@@ -36,6 +36,8 @@ def _lib():
         lib.lc0mi_k_attention_f8.argtypes = [vp, vp, ci, ci, cf, cf, vp]
         lib.lc0mi_k_smolgen_attention.argtypes = [vp, vp, vp, ci, ci, ci, cf, ci, cf, vp, ci, cd]
         lib.lc0mi_k_legal_softmax.argtypes = [vp, vp, vp, cf, ci, vp]
+        lib.lc0mi_k_attention_generic.argtypes = [ci, vp, vp, ci, ci, ci, cf, vp]
+        lib.lc0mi_k_layer_norm_generic.argtypes = [ci, vp, vp, vp, vp, ci, ci, cf, cf, ci, vp]
         lib._k_ready = True
     return lib
 
@@ -45,8 +47,46 @@ def _check(rc):
         raise BackendError(load_library().lc0mi_last_error().decode(errors="replace"))
 
 
+_BF16 = False
+
+
+def to_bf16(a):
+    """float array -> uint16 bfloat16 bits, round to nearest even."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def from_bf16(bits):
+    return (np.ascontiguousarray(bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+class bf16:
+    """with kernels.bf16(): the 16-bit operands of gemm, layer_norm, layer_norm_rows, attention and
+    smolgen_attention are bfloat16 (inputs rounded to it, results returned as float32) and the kernels run their
+    bf16 instances."""
+
+    def __enter__(self):
+        global _BF16
+        _BF16 = True
+        _lib().lc0mi_k_set_bf16(1)
+
+    def __exit__(self, *exc):
+        global _BF16
+        _BF16 = False
+        _lib().lc0mi_k_set_bf16(0)
+
+
 def _h(a):
-    return np.ascontiguousarray(a, dtype=np.float16)
+    """16-bit operand: halves, or bfloat16 bits inside `with bf16()`."""
+    return to_bf16(a) if _BF16 else np.ascontiguousarray(a, dtype=np.float16)
+
+
+def _out16(shape):
+    return np.zeros(shape, np.uint16 if _BF16 else np.float16)
+
+
+def _ret16(out):
+    return from_bf16(out) if _BF16 and out.dtype == np.uint16 else out
 
 
 def _ptr(a):
@@ -62,12 +102,12 @@ def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
         a, w = a[None], w[None]
     batch, m, k = a.shape
     n = w.shape[1]
-    out = np.zeros((batch, m, n), np.float32 if out_f32 else np.float16)
+    out = np.zeros((batch, m, n), np.float32) if out_f32 else _out16((batch, m, n))
     b = np.ascontiguousarray(bias, np.float32) if bias is not None else None
     ms = C.c_double(0)
     _check(_lib().lc0mi_k_gemm(_ptr(a), k, m * k, _ptr(w), k, n * k, _ptr(b), m, n, k, batch, scale, act,
                                int(out_f32), _ptr(out), n, m * n, time_iters, C.byref(ms)))
-    out = out if batched else out[0]
+    out = _ret16(out if batched else out[0])
     return (out, ms.value) if time_iters else out
 
 
@@ -139,10 +179,10 @@ def layer_norm_rows(x, skip, gamma, beta, alpha, eps, pre_act=ACT_NONE, x_is_f32
     g = np.ascontiguousarray(gamma, np.float32)
     b = np.ascontiguousarray(beta, np.float32)
     rows, c = np.shape(x)
-    y = np.zeros((rows, c), np.float16)
+    y = _out16((rows, c))
     _check(_lib().lc0mi_k_layer_norm_rows(_ptr(xf), _ptr(xh), pre_act, _ptr(s), _ptr(g), _ptr(b), rows, c, alpha, eps,
                                           _ptr(y)))
-    return y
+    return _ret16(y)
 
 
 def gemm_f32(a, w, bias=None, scale=1.0, act=ACT_NONE):
@@ -165,6 +205,7 @@ def layer_norm(x, skip, gamma, beta, alpha, eps, time_iters=0):
     ms = C.c_double(0)
     _check(_lib().lc0mi_k_layer_norm(_ptr(x), _ptr(s), _ptr(g), _ptr(b), x.shape[0], x.shape[1], alpha, eps,
                                      _ptr(y), time_iters, C.byref(ms)))
+    y = _ret16(y)
     return (y, ms.value) if time_iters else y
 
 
@@ -172,11 +213,40 @@ def attention(qkv, bias, batch, heads, scale, time_iters=0, depth=32):
     """qkv [B*64, 3*heads*depth], bias [B, heads, 64, 64] or None -> [B*64, heads*depth]."""
     qkv = _h(qkv)
     b = _h(bias) if bias is not None else None
-    out = np.zeros((batch * 64, heads * depth), np.float16)
+    out = _out16((batch * 64, heads * depth))
     ms = C.c_double(0)
     _check(_lib().lc0mi_k_attention(_ptr(qkv), _ptr(b), batch, heads, depth, scale, _ptr(out), time_iters,
                                     C.byref(ms)))
+    out = _ret16(out)
     return (out, ms.value) if time_iters else out
+
+
+_DTYPES = {"half": (0, np.float16), "bf16": (1, np.uint16), "float": (2, np.float32)}
+
+
+def _typed(a, dtype):
+    return to_bf16(a) if dtype == "bf16" else np.ascontiguousarray(a, _DTYPES[dtype][1])
+
+
+def attention_generic(qkv, bias, batch, heads, depth, scale, dtype="float"):
+    """The general attention kernel: any head depth up to 128, dtype half / bf16 / float. Returns float32."""
+    q = _typed(qkv, dtype)
+    b = _typed(bias, dtype) if bias is not None else None
+    out = np.zeros((batch * 64, heads * depth), _DTYPES[dtype][1])
+    _check(_lib().lc0mi_k_attention_generic(_DTYPES[dtype][0], _ptr(q), _ptr(b), batch, heads, depth, scale, _ptr(out)))
+    return from_bf16(out) if dtype == "bf16" else out.astype(np.float32)
+
+
+def layer_norm_generic(x, skip, gamma, beta, alpha, eps, pre_act=ACT_NONE, dtype="float"):
+    """The general layer norm: LN(act(x) * alpha + skip) for any row length, dtype half / bf16 / float."""
+    xt = _typed(x, dtype)
+    st = _typed(skip, dtype) if skip is not None else None
+    g = np.ascontiguousarray(gamma, np.float32)
+    b = np.ascontiguousarray(beta, np.float32)
+    y = np.zeros(xt.shape, _DTYPES[dtype][1])
+    _check(_lib().lc0mi_k_layer_norm_generic(_DTYPES[dtype][0], _ptr(xt), _ptr(st), _ptr(g), _ptr(b), xt.shape[0],
+                                             xt.shape[1], alpha, eps, pre_act, _ptr(y)))
+    return from_bf16(y) if dtype == "bf16" else y.astype(np.float32)
 
 
 def gemm_f8(a, w, col_scale, bias=None, act=ACT_NONE, out_f8=False, out_mul=1.0, time_iters=0):
@@ -225,10 +295,11 @@ def attention_f8(qkv, bias, batch, heads, scale, out_mul):
 def smolgen_attention(qkv, gen, w, batch, heads, scale, f8_out=False, out_mul=1.0, time_iters=0):
     """qkv [B*64, 3*heads*32], gen [B, heads, gen_sz], w [4096, gen_sz] -> [B*64, heads*32] (halves, or e4m3 bytes)."""
     qkv, gen, w = _h(qkv), _h(gen), _h(w)
-    out = np.zeros((batch * 64, heads * 32), np.uint8 if f8_out else np.float16)
+    out = np.zeros((batch * 64, heads * 32), np.uint8) if f8_out else _out16((batch * 64, heads * 32))
     ms = C.c_double(0)
     _check(_lib().lc0mi_k_smolgen_attention(_ptr(qkv), _ptr(gen), _ptr(w), batch, heads, w.shape[1], scale,
                                             int(f8_out), out_mul, _ptr(out), time_iters, C.byref(ms)))
+    out = _ret16(out)
     return (out, ms.value) if time_iters else out
 
 

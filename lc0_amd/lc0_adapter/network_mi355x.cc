@@ -92,7 +92,7 @@ class Mi355xNetwork : public Network {
     const std::string precision = options.GetOrDefault<std::string>("precision", "fp16");
     add("precision", precision);
     if (precision == "fp8") {
-      add("fp8_gemms", options.GetOrDefault<std::string>("fp8_gemms", "qkv+dense+ffn1+ffn2"));
+      add("fp8_gemms", options.GetOrDefault<std::string>("fp8_gemms", "auto"));
       add("fp8_fp16_layers", std::to_string(options.GetOrDefault<int>("fp8_fp16_layers", 0)));
     }
     add("qkv_first", options.GetOrDefault<bool>("qkv_first", true) ? "true" : "false");

@@ -574,3 +574,117 @@ def test_layer_norm_folding_in_every_gemm_variant_that_has_it(producer_variant, 
     np.testing.assert_allclose(u32, alpha * onn.fc(a, w1.reshape(-1), b1, nr.ACT_NONE) + s, rtol=3e-3, atol=3e-3)
     want = onn.fc(onn.layer_norm_skip(u32, 1.0, None, g1, be1, eps), w2.reshape(-1), b2, nr.ACT_MISH)
     np.testing.assert_allclose(got, want, rtol=4e-3, atol=4e-3)
+
+
+# ---- bfloat16 instances of the 16-bit kernels, and the general (any type, any shape) kernels ----------------------
+def _bf(a):
+    """Values rounded to bfloat16, as float32."""
+    from lc0_amd import kernels as K
+    return K.from_bf16(K.to_bf16(a))
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 7, 9, 10])
+@pytest.mark.parametrize("m,n,k", [(2048, 1024, 256), (777, 200, 128), (300, 1858, 64), (1000, 32, 256)])
+def test_every_gemm_variant_in_bf16_vs_oracle_fc(variant, m, n, k):
+    """Every tile shape of the dense-layer kernels with bfloat16 operands (v_mfma_f32_32x32x16_bf16, fp32
+    accumulation, bfloat16 output) against the oracle's Forward1D on the same bfloat16-rounded inputs. The only
+    difference allowed is the rounding of the output to 8 significant bits and the summation order."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(variant * 7 + m + n + k)
+    a = _bf(rng.standard_normal((m, k)) * 0.5)
+    w = _bf(rng.standard_normal((n, k)) * 0.1)
+    b = rng.standard_normal(n).astype(f32)
+    want = onn.fc(a, w.reshape(-1), b, nr.ACT_MISH)
+    try:
+        K.set_gemm_variant(variant)
+        with K.bf16():
+            got = K.gemm(a, w, b, act=nr.ACT_MISH)
+            got_f32 = K.gemm(a, w, b, act=nr.ACT_NONE, out_f32=True)
+    finally:
+        K.set_gemm_variant(-1)
+    np.testing.assert_allclose(got, want, rtol=2.0 ** -7, atol=2e-3)          # one rounding to bfloat16 (2^-9) and slack
+    np.testing.assert_allclose(got_f32, onn.fc(a, w.reshape(-1), b, nr.ACT_NONE), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("rows,c", [(300, 256), (128, 1024), (9, 8192)])
+def test_layer_norms_in_bf16_vs_oracle(rows, c):
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(rows + c)
+    x, s = _bf(rng.standard_normal((rows, c))), _bf(rng.standard_normal((rows, c)) * 0.5)
+    g, b = (1 + 0.1 * rng.standard_normal(c)).astype(f32), (0.1 * rng.standard_normal(c)).astype(f32)
+    want = onn.layer_norm_skip(x, 0.7, s, g, b, 1e-6)
+    with K.bf16():
+        got = K.layer_norm(x, s, g, b, 0.7, 1e-6)
+        got_rows = K.layer_norm_rows(x, s, g, b, 0.7, 1e-6)
+    np.testing.assert_allclose(got, want, rtol=2.0 ** -7, atol=2.0 ** -8)
+    np.testing.assert_allclose(got_rows, want, rtol=2.0 ** -7, atol=2.0 ** -8)
+
+
+@pytest.mark.parametrize("batch,heads,depth", [(3, 2, 32), (2, 4, 64), (2, 2, 128)])
+def test_attention_in_bf16_vs_oracle(batch, heads, depth):
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(batch * 100 + heads + depth)
+    d = heads * depth
+    qkv = _bf(rng.standard_normal((batch * 64, 3 * d)))
+    bias = _bf(rng.standard_normal((batch, heads, 64, 64)) * 2)
+    scale = 1.0 / np.sqrt(float(depth))
+    q, k, v = (qkv[:, i * d:(i + 1) * d].reshape(batch, 64, heads, depth).transpose(0, 2, 1, 3) for i in range(3))
+    p = onn.softmax_rows(np.matmul(q, k.transpose(0, 1, 3, 2)) * f32(scale) + bias)
+    want = np.matmul(p, v).transpose(0, 2, 1, 3).reshape(batch * 64, d)
+    with K.bf16():
+        got = K.attention(qkv, bias, batch, heads, scale, depth=depth)
+    # probabilities and the output are rounded to bfloat16 (2^-9 each)
+    np.testing.assert_allclose(got, want, rtol=2.0 ** -6, atol=2.0 ** -6)
+
+
+def test_smolgen_attention_in_bf16_vs_reference():
+    from lc0_amd import kernels as K
+    batch, heads, gen_sz = 6, 32, 256
+    rng = np.random.default_rng(77)
+    d = heads * 32
+    qkv = _bf(rng.standard_normal((batch * 64, 3 * d)))
+    gen = _bf(rng.standard_normal((batch, heads, gen_sz)))
+    w = _bf(rng.standard_normal((4096, gen_sz)) * (2.0 / np.sqrt(gen_sz)))
+    scale = 1.0 / np.sqrt(32.0)
+    logits = _bf(gen.reshape(batch * heads, -1) @ w.T).reshape(batch, heads, 64, 64)   # kept as bfloat16 in LDS
+    q, k, v = (qkv[:, i * d:(i + 1) * d].reshape(batch, 64, heads, 32).transpose(0, 2, 1, 3) for i in range(3))
+    p = onn.softmax_rows(np.matmul(q, k.transpose(0, 1, 3, 2)) * f32(scale) + logits)
+    want = np.matmul(p, v).transpose(0, 2, 1, 3).reshape(batch * 64, d)
+    with K.bf16():
+        got = K.smolgen_attention(qkv, gen, w, batch, heads, scale)
+    np.testing.assert_allclose(got, want, rtol=2.0 ** -5, atol=2.0 ** -5)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float", 2e-6), ("half", 2e-3), ("bf16", 2.0 ** -7)])
+@pytest.mark.parametrize("batch,heads,depth,with_bias", [(2, 3, 48, True), (1, 2, 20, False), (2, 2, 128, True),
+                                                         (3, 4, 32, True)])
+def test_general_attention_kernel_vs_oracle(dtype, tol, batch, heads, depth, with_bias):
+    """attention_generic_kernel: head depths the matrix-core kernel does not take, every element type (float:
+    the reference's arithmetic, agreement to rounding)."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(batch + 10 * heads + depth)
+    rnd = {"float": lambda a: a.astype(f32), "half": lambda a: _h(a).astype(f32), "bf16": _bf}[dtype]
+    d = heads * depth
+    qkv = rnd(rng.standard_normal((batch * 64, 3 * d)))
+    bias = rnd(rng.standard_normal((batch, heads, 64, 64)) * 2) if with_bias else None
+    scale = 1.0 / np.sqrt(float(depth))
+    q, k, v = (qkv[:, i * d:(i + 1) * d].reshape(batch, 64, heads, depth).transpose(0, 2, 1, 3) for i in range(3))
+    s = np.matmul(q, k.transpose(0, 1, 3, 2)) * f32(scale)
+    p = onn.softmax_rows(s + bias if with_bias else s)
+    want = np.matmul(p, v).transpose(0, 2, 1, 3).reshape(batch * 64, d)
+    got = K.attention_generic(qkv, bias, batch, heads, depth, scale, dtype=dtype)
+    np.testing.assert_allclose(got, want, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float", 2e-6), ("half", 2e-3), ("bf16", 2.0 ** -7)])
+@pytest.mark.parametrize("rows,c,act", [(37, 100, nr.ACT_NONE), (5, 8200, nr.ACT_SWISH), (64, 36, nr.ACT_MISH)])
+def test_general_layer_norm_kernel_vs_oracle(dtype, tol, rows, c, act):
+    """layer_norm_generic_kernel: row lengths that are no multiple of 8 or exceed 8192, an activation applied first."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(rows + c)
+    rnd = {"float": lambda a: a.astype(f32), "half": lambda a: _h(a).astype(f32), "bf16": _bf}[dtype]
+    x, s = rnd(rng.standard_normal((rows, c))), rnd(rng.standard_normal((rows, c)) * 0.5)
+    g, b = (1 + 0.1 * rng.standard_normal(c)).astype(f32), (0.1 * rng.standard_normal(c)).astype(f32)
+    want = onn.layer_norm_skip(onn.activate(x, act), 0.6, s, g, b, 1e-3)
+    got = K.layer_norm_generic(x, s, g, b, 0.6, 1e-3, pre_act=act, dtype=dtype)
+    np.testing.assert_allclose(got, want, rtol=tol, atol=2 * tol)

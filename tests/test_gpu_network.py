@@ -393,10 +393,13 @@ def _legal_logit_rms(a, b, legal):
     return float(np.sqrt((err * err).mean()))
 
 
-def _emulation_of(path, net, gemms=ALL_FP8_GEMMS, **kw):
-    """oracle/fp8_net.py with the activation scales the backend is using."""
+def _emulation_of(path, net, gemms=None, **kw):
+    """oracle/fp8_net.py with the activation scales the backend is using (and, unless told, with the smolgen chain in
+    e4m3 exactly when the backend reports scales for it)."""
     from oracle import fp8_net
     sc = net.Fp8Scales()
+    if gemms is None:
+        gemms = ALL_FP8_GEMMS + (("smolgen",) if (sc[:, 4:] != 1.0).any() else ())
     return fp8_net.Fp8BlasNetwork(nr.load(path), scales=sc[:, :4], smolgen_scales=sc[:, 4:], gemms=gemms, **kw)
 
 
@@ -426,6 +429,7 @@ def test_bt4_shape_fp8_batch_sweep(positions):
     masks, values, legal = positions["masks"][:64], positions["values"][:64], positions["legal"][:64]
     want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
     net, res = _run_gpu(path, masks, values, "precision=fp8")
+    assert (net.Fp8Scales()[:, 4:] != 1.0).all()   # the default takes the smolgen chain in e4m3 too, as configs[4] lists it
     s = _fp8_report(res, want, legal)
     assert s["kl_max"] <= 1e-4 and s["softmax_maxabs"] <= 1e-3
     assert s["q"] <= 1e-2 and s["d"] <= 1e-2 and s["mlh_rel"] <= 2e-2
@@ -485,8 +489,8 @@ def test_bt4_shape_fp8_batch_sweep(positions):
 
 @pytest.mark.parametrize("name,batch", [("tiny_attn_f8_sg", 40), ("c2_bt4_15x1024", 33)])
 def test_fp8_smolgen_chain_in_e4m3(name, batch, positions):
-    """fp8_gemms=...+smolgen (configs[4] lists the smolgen GEMMs among the e4m3 ones): compression, both dense layers
-    and the shared generator run on e4m3 operands. Against the emulation of the same arithmetic and, by noise
+    """fp8_gemms=...+smolgen (configs[4] lists the smolgen GEMMs among the e4m3 ones; the default where the chain's
+    widths allow it): compression, both dense layers and the shared generator run on e4m3 operands. Against the emulation of the same arithmetic and, by noise
     level, against the fp32 oracle; the profile must show the chain's fp8 kernels."""
     path = netgen.cached_config(name)
     masks, values, legal = positions["masks"][:batch], positions["values"][:batch], positions["legal"][:batch]
