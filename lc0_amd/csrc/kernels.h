@@ -149,9 +149,11 @@ void SetGemmVariantOverride(int variant);
 // where x is half (x_f16) or the sum of n_partials float arrays x_f32 + i * partial_stride
 // (split-K partial sums); exactly one of x_f32 / x_f16 is non-null. pre_act is an
 // Activation enum value applied before the norm. C % 8 == 0, C <= 8192.
+// y_f8 (optional): also receives e4m3(y * f8_mul), saturating, taken from the float values.
 void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_stride, const half_t* x_f16,
                          int pre_act, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows,
-                         int C, float alpha, float eps, hipStream_t stream, bool bf16 = false);
+                         int C, float alpha, float eps, hipStream_t stream, bool bf16 = false,
+                         uint8_t* y_f8 = nullptr, float f8_mul = 1.0f);
 
 // rows x C layer norm: y = beta + gamma * (t - mean) / sqrt(var + eps) with
 // t = x * alpha + skip (skip may be null). x, skip, y may alias. C % 8 == 0, C <= 8192.

@@ -259,7 +259,7 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __res
                                                               int pre_act, const half_t* skip, half_t* y,
                                                               const float* __restrict__ gamma,
                                                               const float* __restrict__ beta, int C, float alpha,
-                                                              float eps) {
+                                                              float eps, uint8_t* yq, float q_mul) {
   using ev8 = typename Vec16<ET>::v8;
   __shared__ float red[4];
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -337,9 +337,19 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __res
         bt[i][1] = *reinterpret_cast<const floatx4*>(beta + v * 8 + 4);
       }
       ev8 o;
+      float f[8];
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = (ET)(bt[i][e / 4][e % 4] + gm[i][e / 4][e % 4] * (t[i][e] - mean) * den);
+      for (int e = 0; e < 8; e++) {
+        f[e] = bt[i][e / 4][e % 4] + gm[i][e / 4][e % 4] * (t[i][e] - mean) * den;
+        o[e] = (ET)f[e];
+      }
       *reinterpret_cast<ev8*>(y + (long long)row * C + v * 8) = o;
+      if (yq != nullptr) {   // e4m3 copy of the same row (from the float values) for a following fp8 GEMM
+        uint2 q;
+        q.x = PackFp8x4(f[0] * q_mul, f[1] * q_mul, f[2] * q_mul, f[3] * q_mul);
+        q.y = PackFp8x4(f[4] * q_mul, f[5] * q_mul, f[6] * q_mul, f[7] * q_mul);
+        *reinterpret_cast<uint2*>(yq + (long long)row * C + v * 8) = q;
+      }
     }
   }
 }
@@ -365,12 +375,12 @@ void LaunchZero(float* p, long long n, hipStream_t stream) {
 
 void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_stride, const half_t* x_f16,
                          int pre_act, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows,
-                         int C, float alpha, float eps, hipStream_t stream, bool bf16) {
+                         int C, float alpha, float eps, hipStream_t stream, bool bf16, uint8_t* y_f8, float f8_mul) {
   if (rows <= 0) return;
   auto launch = [&](auto early_tag, auto elem_tag) {
     using ET = decltype(elem_tag);
     hipLaunchKernelGGL((layer_norm_rows_kernel<decltype(early_tag)::value, ET>), dim3(rows), dim3(256), 0, stream, x_f32,
-                       n_partials, partial_stride, x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps);
+                       n_partials, partial_stride, x_f16, pre_act, skip, y, gamma, beta, C, alpha, eps, y_f8, f8_mul);
   };
   if (bf16) {
     if (rows <= 64) launch(std::true_type{}, bf16_t{});

@@ -1930,23 +1930,17 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       const bool chain_first = f8 || B <= chain_latency_max_batch_;
       if (chain_f8) {
         // The whole chain on e4m3 operands: the compression reads the e4m3 copy of x that the QKV projection reads
-        // and writes e4m3 itself; the two row norms write halves, which a small kernel quantises.
+        // and writes e4m3 itself; the two row norms write halves and their e4m3 copies.
         GemmF8("gemm_smolgen_compress", xq_, e.sg_compress, e.sg_compress8, sg1q_, T, kActNone, true, 1.0f / e.s_sg1, ss);
         GemmF8("gemm_smolgen_dense1", sg1q_, e.sg_dense1, e.sg_dense18, sg2_, B, smolgen_act_, false, 1.0f, ss);
-        Timed("layer_norm_rows", 0.0, 4.0 * B * sg_hs_, [&] {
+        Timed("layer_norm_rows", 0.0, 5.0 * B * sg_hs_, [&] {
           LaunchLayerNormRows(nullptr, 0, 0, sg2_, kActNone, nullptr, sg2_, e.sg_ln1_g, e.sg_ln1_b, B, sg_hs_, 1.0f,
-                              1e-3f, ss);
-        }, ss);
-        Timed("quantize_f8", 0.0, 3.0 * B * sg_hs_, [&] {
-          LaunchQuantizeF8(sg2_, sg2q_, static_cast<long long>(B) * sg_hs_, 1.0f / e.s_sg2, ss);
+                              1e-3f, ss, false, sg2q_, 1.0f / e.s_sg2);
         }, ss);
         GemmF8("gemm_smolgen_dense2", sg2q_, e.sg_dense2, e.sg_dense28, sg3_, B, smolgen_act_, false, 1.0f, ss);
-        Timed("layer_norm_rows", 0.0, 4.0 * B * sg_gen_, [&] {
+        Timed("layer_norm_rows", 0.0, 5.0 * B * sg_gen_, [&] {
           LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f,
-                              1e-3f, ss);
-        }, ss);
-        Timed("quantize_f8", 0.0, 3.0 * B * sg_gen_, [&] {
-          LaunchQuantizeF8(sg3_, sg3q_, static_cast<long long>(B) * sg_gen_, 1.0f / e.s_sg3, ss);
+                              1e-3f, ss, false, sg3q_, 1.0f / e.s_sg3);
         }, ss);
         GemmF8("gemm_smolgen_global", sg3q_, smolgen_w_, e.sg_global8, sbias_, B * heads_, kActNone, false, 1.0f, ss);
       } else if (dtype_ == Dtype::kFloat) {

@@ -179,11 +179,11 @@ class Fp8BlasNetwork(BlasNetwork):
                 t = qw["sg_compress"](xq, s_x, None, nr.ACT_NONE)
                 tq = quantize_activation(t, ss[0]).reshape(bsz, 64 * hc)
                 t = self._h(qw["sg_dense1"](tq, ss[0], sg.dense1_b, smolgen_act))
-                # (the two row norms store halves; their e4m3 copies are made from those)
-                t = self._h(layer_norm_skip(t, 1.0, None, sg.ln1_gammas, sg.ln1_betas, 1e-3))
+                # (the two row norms write their e4m3 copies from the float values, like the body's norms)
+                t = layer_norm_skip(t, 1.0, None, sg.ln1_gammas, sg.ln1_betas, 1e-3)
                 tq = quantize_activation(t, ss[1])
                 t = self._h(qw["sg_dense2"](tq, ss[1], sg.dense2_b, smolgen_act))
-                t = self._h(layer_norm_skip(t, 1.0, None, sg.ln2_gammas, sg.ln2_betas, 1e-3))
+                t = layer_norm_skip(t, 1.0, None, sg.ln2_gammas, sg.ln2_betas, 1e-3)
                 tq = quantize_activation(t, ss[2]).reshape(bsz * heads, gen // heads)
                 qk_bias = self._h(qw["sg_global"](tq, ss[2], None, nr.ACT_NONE))
             else:
