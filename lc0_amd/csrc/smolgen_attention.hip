@@ -59,8 +59,22 @@ __device__ __forceinline__ float Reduce4Rows(float x, F&& op) {
   return op(y, c);
 }
 
-// FULL: 32 heads and an even number of samples, so that every (sample, head) column of every workgroup exists and
-// the loop over head pairs carries no branches (the compiler then overlaps neighbouring pairs).
+// The same for two independent values at once (the two heads of a pair): the swaps of both share the wait states.
+template <typename F>
+__device__ __forceinline__ void Reduce4Rows2(float& x0, float& x1, F&& op) {
+  float a0 = x0, b0 = x0, a1 = x1, b1 = x1;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\ts_nop 1"
+               : "+v"(a0), "+v"(b0), "+v"(a1), "+v"(b1));
+  float y0 = op(a0, b0), y1 = op(a1, b1);
+  float c0 = y0, c1 = y1;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\ts_nop 1"
+               : "+v"(y0), "+v"(c0), "+v"(y1), "+v"(c1));
+  x0 = op(y0, c0);
+  x1 = op(y1, c1);
+}
+
+// FULL: 32 heads, so that every (sample, head) column of every workgroup exists (or repeats an existing one), the
+// loop over head pairs carries no branches and its interleaved order fits the registers.
 // ET: half_t or bf16_t, the type of qkv, gen, wfrag, of the logits kept in LDS and of a 16-bit output (all typed
 // half_t here: the same storage).
 template <int NKS, typename OutT, bool FULL, typename ET>
@@ -72,7 +86,10 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
   using ev8 = typename Vec16<ET>::v8;
   using ev4 = typename Vec16<ET>::v4;
   constexpr int DEPTH = 32;
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[kLogitBytes + 8 * kVBytesPerWave];
+  // Two arrays, not one with offsets: the compiler can then tell that staging a K or V tile never touches the logits
+  // and moves the staging of the next pair of heads in among the softmax arithmetic of this one.
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kLogitBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char stage_lds[8 * kVBytesPerWave];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 31, g = lane >> 5;
@@ -99,7 +116,7 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
     for (int f = 0; f < PF; f++) ring[f] = wp[f * 64];
     // The generator vectors of the 64 columns: once per workgroup through LDS (the region phase 2 stages K and V in), 16-byte
     // slot s of column c at slot s ^ (c & 31) of its row, then into the registers of every wave as MFMA "B" operands.
-    unsigned char* gl = smem + kLogitBytes;
+    unsigned char* gl = stage_lds;
     constexpr int kSlotsPerCol = G / 8;
     for (int i = threadIdx.x; i < 64 * kSlotsPerCol; i += 512) {
       const int c = i / kSlotsPerCol, sl = i - c * kSlotsPerCol;
@@ -165,30 +182,43 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
   // are in flight while this one is computed.
   const int j = lane & 15, g4 = lane >> 4;
   const int lr = lane >> 3, ch = lane & 7;
-  unsigned char* stg = smem + kLogitBytes + wave * kVBytesPerWave;
+  unsigned char* stg = stage_lds + wave * kVBytesPerWave;
   struct PairData {
     ev8 k[2][4], v[2][4];   // [32-row tile][8-row group]
     ev8 q[2];               // [head]: query j, depth 8 g4 .. 8 g4 + 7
   };
-  auto load_pair = [&](int pi, PairData& d) {
+  // The pieces of a pair's rows are loaded separately, each into the registers that the same piece of the pair
+  // before has just left for LDS: one set of registers serves all four pairs.
+  auto pair_base = [&](int pi, const half_t*& Kp, const half_t*& Q, bool& has_b) {
     const int ca = wave * 8 + 2 * pi;
     const int b = ca >= 32 ? b1 : b0;
     const int ha = ca & 31;
     const int ha_c = (FULL || ha < heads) ? ha : 0;
-    const bool has_b = FULL || ha_c + 1 < heads;
+    has_b = FULL || ha_c + 1 < heads;
     const half_t* base = qkv + (long long)b * 64 * ld;
     // (without a head B the upper half of the row repeats head A instead of running past the row)
-    const half_t* Kp = base + d_model + ha_c * DEPTH + (has_b ? ch : (ch & 3)) * 8 + (unsigned)lr * (unsigned)ld;
-    const half_t* Vp = Kp + d_model;
+    Kp = base + d_model + ha_c * DEPTH + (has_b ? ch : (ch & 3)) * 8 + (unsigned)lr * (unsigned)ld;
+    Q = base + ha_c * DEPTH + (unsigned)(kQueriesPerGroup * qt + j) * (unsigned)ld + 8u * g4;
+  };
+  auto load_k = [&](int pi, int t, PairData& d) {
+    const half_t *Kp, *Q;
+    bool has_b;
+    pair_base(pi, Kp, Q, has_b);
 #pragma unroll
-    for (int t = 0; t < 2; t++)
+    for (int i = 0; i < 4; i++) d.k[t][i] = *reinterpret_cast<const ev8*>(Kp + (unsigned)(32 * t + 8 * i) * (unsigned)ld);
+  };
+  auto load_v = [&](int pi, int t, PairData& d) {
+    const half_t *Kp, *Q;
+    bool has_b;
+    pair_base(pi, Kp, Q, has_b);
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const unsigned off = (unsigned)(32 * t + 8 * i) * (unsigned)ld;
-        d.k[t][i] = *reinterpret_cast<const ev8*>(Kp + off);
-        d.v[t][i] = *reinterpret_cast<const ev8*>(Vp + off);
-      }
-    const half_t* Q = base + ha_c * DEPTH + (unsigned)(kQueriesPerGroup * qt + j) * (unsigned)ld + 8u * g4;
+    for (int i = 0; i < 4; i++)
+      d.v[t][i] = *reinterpret_cast<const ev8*>(Kp + d_model + (unsigned)(32 * t + 8 * i) * (unsigned)ld);
+  };
+  auto load_q = [&](int pi, PairData& d) {
+    const half_t *Kp, *Q;
+    bool has_b;
+    pair_base(pi, Kp, Q, has_b);
     d.q[0] = *reinterpret_cast<const ev8*>(Q);
     d.q[1] = *reinterpret_cast<const ev8*>(Q + (has_b ? DEPTH : 0));
   };
@@ -215,99 +245,146 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
     for (int e = 0; e < 8; e++) ident[dt][e] = (8 * g4 + e == 16 * dt + j) ? (ET)1.0f : (ET)0.0f;
   const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
-  PairData cur, nxt;
-  load_pair(0, cur);
+  // Software pipeline over the wave's four pairs of heads: while the softmax and P.V of pair p run (vector ALU work
+  // with long dependency chains: exponentials, lane swaps), the scores and V^T of pair p + 1 are prepared (LDS round
+  // trips and matrix instructions), and the rows of pair p + 2 are on their way from memory. The two kinds of work
+  // are written alternately below, step by step and for both heads of a pair at once, because the compiler keeps
+  // the order of the source here and would otherwise run every chain to its end before starting the next.
+  struct Prep {
+    floatx4 st[2][4];   // S^T[key][query] of both heads: [head][16-key tile], register e = key 16 t + 4 g4 + e
+    ev8 vt[2][2][2];    // V^T of both heads as operands: [head][depth half][32-key step], lane (depth index, g4),
+  };                    //   elements = keys 32 s + 4 g4 + (0..3) and 32 s + 16 + 4 g4 + (0..3), the order of P below
+  auto prep_k = [&](const PairData& d, int tt, Prep& o) {
+    ev8 kf[2][2];
+    stage_tile(d.k[tt], kf);
+#pragma unroll
+    for (int hb = 0; hb < 2; hb++)
+#pragma unroll
+      for (int th = 0; th < 2; th++) o.st[hb][2 * tt + th] = Mfma16(kf[hb][th], d.q[hb], zero4);
+  };
+  auto prep_v = [&](const PairData& d, int tt, Prep& o) {
+    ev8 vr[2][2];
+    stage_tile(d.v[tt], vr);
+#pragma unroll
+    for (int hb = 0; hb < 2; hb++)
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int th = 0; th < 2; th++) {
+          const floatx4 tr = Mfma16(vr[hb][th], ident[dt], zero4);
+#pragma unroll
+          for (int e = 0; e < 4; e++) o.vt[hb][dt][tt][4 * th + e] = (ET)tr[e];
+        }
+  };
+
+  // Step 0..3 of preparing the pair whose rows are in `raw`; every step refills the registers it has emptied with the
+  // same piece of pair `next` (if there is one).
+  PairData raw;
+  auto prep_step = [&](int step, int next, Prep& o) {
+    if (step < 2) {
+      prep_k(raw, step, o);
+      if (next < 4) {
+        load_k(next, step, raw);
+        if (step == 1) load_q(next, raw);
+      }
+    } else {
+      prep_v(raw, step - 2, o);
+      if (next < 4) load_v(next, step - 2, raw);
+    }
+  };
+  Prep prep[2];
+  load_k(0, 0, raw);
+  load_q(0, raw);
+  load_k(0, 1, raw);
+  load_v(0, 0, raw);
+  load_v(0, 1, raw);
+#pragma unroll
+  for (int step = 0; step < 4; step++) prep_step(step, 1, prep[0]);
 #pragma unroll
   for (int pi = 0; pi < 4; pi++) {
     const int ca = wave * 8 + 2 * pi;
     const int ha = ca & 31;
+    const int b = ca >= 32 ? b1 : b0;
+    // (columns that do not exist - heads past the last, the second sample of an odd batch - are computed on the rows
+    // of a head that does and not stored)
     const bool live_a = FULL || (ha < heads && (ca < 32 || valid1));   // uniform over the wave
     const bool live_b = FULL || (live_a && ha + 1 < heads);
-    if (pi + 1 < 4) load_pair(pi + 1, nxt);
-    if (live_a) {
-      const int b = ca >= 32 ? b1 : b0;
-      // S^T[key][query] of both heads: st[head][16-key tile], register e = key 16 t + 4 g4 + e
-      floatx4 st[2][4];
+    const bool more = pi + 1 < 4;
+    const Prep& cp = prep[pi & 1];
+    Prep& np = prep[(pi + 1) & 1];
+
+    if (more && FULL) prep_step(0, pi + 2, np);
+    // scale, add the logits, maximum over the 64 keys of this lane's query: 16 here, 48 in the lanes 16, 32, 48 away
+    float sv[2][16], mx[2], sum[2];
 #pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
-        ev8 kf[2][2];
-        stage_tile(cur.k[tt], kf);
+    for (int hb = 0; hb < 2; hb++) {
+      const int c = ca + hb;
+      const ev8 lg0 = *reinterpret_cast<const ev8*>(smem + LogitSlot(c, j, g4, 0));
+      const ev8 lg1 = *reinterpret_cast<const ev8*>(smem + LogitSlot(c, j, g4, 2));
+      mx[hb] = -3.0e38f;
 #pragma unroll
-        for (int hb = 0; hb < 2; hb++)
+      for (int t = 0; t < 4; t++)
 #pragma unroll
-          for (int th = 0; th < 2; th++)
-            st[hb][2 * tt + th] = Mfma16(kf[hb][th], cur.q[hb], zero4);
-      }
-      // V^T of both heads as halves in operand layout: vt[head][depth half][32-key step], lane (depth index, g4),
-      // elements = keys 32 s + 4 g4 + (0..3) and 32 s + 16 + 4 g4 + (0..3), the order of the P operand below
-      ev8 vt[2][2][2];
-#pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
-        ev8 vr[2][2];
-        stage_tile(cur.v[tt], vr);
-#pragma unroll
-        for (int hb = 0; hb < 2; hb++)
-#pragma unroll
-          for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-            for (int th = 0; th < 2; th++) {
-              const floatx4 tr = Mfma16(vr[hb][th], ident[dt], zero4);
-#pragma unroll
-              for (int e = 0; e < 4; e++) vt[hb][dt][tt][4 * th + e] = (ET)tr[e];
-            }
-      }
-#pragma unroll
-      for (int hb = 0; hb < 2; hb++) {
-        if (hb == 1 && !live_b) break;
-        const int c = ca + hb;
-        // scale, add the logits, softmax over the 64 keys of this lane's query: 16 here, 48 in the lanes 16, 32, 48 away
-        const ev8 lg0 = *reinterpret_cast<const ev8*>(smem + LogitSlot(c, j, g4, 0));
-        const ev8 lg1 = *reinterpret_cast<const ev8*>(smem + LogitSlot(c, j, g4, 2));
-        float sv[16];
-        float mx = -3.0e38f;
-#pragma unroll
-        for (int t = 0; t < 4; t++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const float lgv = (float)(t < 2 ? lg0[4 * t + e] : lg1[4 * (t - 2) + e]);
-            sv[4 * t + e] = st[hb][t][e] * scale + lgv;
-            mx = fmaxf(mx, sv[4 * t + e]);
-          }
-        mx = Reduce4Rows(mx, [](float a, float b) { return fmaxf(a, b); });
-        float sum = 0.0f;
-        const float kLog2e = 1.44269504f, neg_mx = -mx * kLog2e;
-#pragma unroll
-        for (int e = 0; e < 16; e++) {
-          sv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[e], kLog2e, neg_mx));   // e^(s - mx) <= 1
-          sum += sv[e];
+        for (int e = 0; e < 4; e++) {
+          const float lgv = (float)(t < 2 ? lg0[4 * t + e] : lg1[4 * (t - 2) + e]);
+          sv[hb][4 * t + e] = cp.st[hb][t][e] * scale + lgv;
+          mx[hb] = fmaxf(mx[hb], sv[hb][4 * t + e]);
         }
-        sum = Reduce4Rows(sum, [](float a, float b) { return a + b; });
-        const float inv = __builtin_amdgcn_rcpf(sum);   // 1 ulp
-        ev8 pf[2];
+    }
+    if (more && FULL) prep_step(1, pi + 2, np);
+    Reduce4Rows2(mx[0], mx[1], [](float a, float b) { return fmaxf(a, b); });
+    const float kLog2e = 1.44269504f;
 #pragma unroll
-        for (int s2 = 0; s2 < 2; s2++)
+    for (int hb = 0; hb < 2; hb++) {
+      const float neg_mx = -mx[hb] * kLog2e;
+      sum[hb] = 0.0f;
 #pragma unroll
-          for (int e = 0; e < 8; e++) pf[s2][e] = (ET)sv[8 * s2 + e];
-        // O^T = V^T . P^T: lane (query j, g4), register e = depth index 16 dt + 4 g4 + e
-        OutT* O = out + (long long)(b * 64 + kQueriesPerGroup * qt + j) * d_model + (ha + hb) * DEPTH + 4 * g4;
+      for (int e = 0; e < 16; e++) {
+        sv[hb][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[hb][e], kLog2e, neg_mx));   // e^(s - mx) <= 1
+        sum[hb] += sv[hb][e];
+      }
+    }
+    if (more && FULL) prep_step(2, pi + 2, np);
+    Reduce4Rows2(sum[0], sum[1], [](float a, float b) { return a + b; });
+    ev8 pf[2][2];
 #pragma unroll
-        for (int dt = 0; dt < 2; dt++) {
-          floatx4 o = zero4;
+    for (int hb = 0; hb < 2; hb++)
 #pragma unroll
-          for (int s2 = 0; s2 < 2; s2++) o = Mfma16(vt[hb][dt][s2], pf[s2], o);
-          if constexpr (sizeof(OutT) == 1) {
-            const float m = inv * out_mul;
-            *reinterpret_cast<unsigned*>(O + 16 * dt) = PackFp8x4(o[0] * m, o[1] * m, o[2] * m, o[3] * m);
-          } else {
-            ev4 h4;
+      for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) h4[e] = (ET)(o[e] * inv);
-            *reinterpret_cast<ev4*>(O + 16 * dt) = h4;
-          }
+        for (int e = 0; e < 8; e++) pf[hb][s2][e] = (ET)sv[hb][8 * s2 + e];
+    if (more && FULL) prep_step(3, pi + 2, np);
+    // O^T = V^T . P^T: lane (query j, g4), register e = depth index 16 dt + 4 g4 + e
+#pragma unroll
+    for (int hb = 0; hb < 2; hb++) {
+      const float inv = __builtin_amdgcn_rcpf(sum[hb]);   // 1 ulp
+      OutT* O = out + (long long)(b * 64 + kQueriesPerGroup * qt + j) * d_model + (ha + hb) * DEPTH + 4 * g4;
+      const bool live = hb == 0 ? live_a : live_b;
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++) {
+        floatx4 o = zero4;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++) o = Mfma16(cp.vt[hb][dt][s2], pf[hb][s2], o);
+        if (!live) continue;
+        if constexpr (sizeof(OutT) == 1) {
+          const float m = inv * out_mul;
+          *reinterpret_cast<unsigned*>(O + 16 * dt) = PackFp8x4(o[0] * m, o[1] * m, o[2] * m, o[3] * m);
+        } else {
+          ev4 h4;
+#pragma unroll
+          for (int e = 0; e < 4; e++) h4[e] = (ET)(o[e] * inv);
+          *reinterpret_cast<ev4*>(O + 16 * dt) = h4;
         }
       }
     }
-    if (pi + 1 < 4) cur = nxt;
+    // (with liveness branches in the way the interleaved order needs more registers than there are: one pair after
+    // the other then)
+    if constexpr (!FULL) {
+      if (more) {
+#pragma unroll
+        for (int step = 0; step < 4; step++) prep_step(step, pi + 2, np);
+      }
+    }
   }
 }
 
@@ -320,7 +397,9 @@ void LaunchT(const half_t* qkv, const half_t* gen, const half_t* wfrag, OutT* ou
   if (batch <= 0) return;
   const int pairs = (batch + 1) / 2;
   const dim3 grid(((pairs + 7) / 8) * 32), block(512);
-  const bool full = heads == 32 && batch % 2 == 0;
+  // (an odd batch runs the full instance too: the last workgroup then takes its one sample twice and both halves store
+  // the same values to the same places)
+  const bool full = heads == 32;
   auto launch = [&](auto nks_tag, auto full_tag) {
     if constexpr (sizeof(OutT) == 2) {
       if (bf16) {
