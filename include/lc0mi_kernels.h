@@ -51,6 +51,11 @@ int lc0mi_k_set_gemm_variant(int variant);
  * lc0mi_k_attention and lc0mi_k_smolgen_attention (half output) hold bfloat16 values and the kernels run their bf16
  * instances (precision=bf16 of the network; the reference's type: src/utils/bf16_utils.h). 0 switches back to half. */
 int lc0mi_k_set_bf16(int on);
+/* Profiling hook, process-wide: with mib > 0 every timed launch (time_iters of the entry points here) is preceded by
+ * an untimed copy of mib MiB, so that the kernel finds its operands in memory rather than in L2 or the memory-side
+ * cache, as it does between other kernels inside a forward pass; the timed launches are then timed one by one.
+ * 0 switches back to back-to-back launches. No counterpart in the reference. */
+int lc0mi_k_set_cold_cache(int mib);
 /* The general attention and layer norm kernels (any element type, head depth up to 128, any row length): dtype 0 half,
  * 1 bfloat16, 2 float for qkv / bias / out and x / skip / y. Same contracts as lc0mi_k_attention (bias [b][h][q][k])
  * and lc0mi_k_layer_norm, with an activation (lc0's numbering) applied to x first. Counterparts in the reference:

@@ -13,10 +13,10 @@
 //     halves in the layout phase 2 reads (128 KiB for the workgroup: 32 contiguous bytes per reading lane, the
 //     positions XOR-ed with the column so that the writers of one instruction spread over eight bank groups).
 //   Phase 2 (memory and vector ALU): every wave takes 8 of the 64 (sample, head) columns. With 16-wide MFMA tiles the 16
-//     queries are one tile: S^T = K.Q^T, plus the logits from LDS, softmax in registers with two lane exchanges,
-//     O^T = V^T.P^T with V transposed on the matrix cores (no LDS gather) and 8-byte output stores straight from the
-//     accumulators. K and V come in by full 128-byte rows of two neighbouring heads; the next pair's are in flight
-//     while this one is computed.
+//     queries are one tile: S^T = K.Q^T, plus the logits from LDS, softmax in registers with one lane exchange (the
+//     maximum; the row sums come from the matrix cores as 1.P^T), O^T = V^T.P^T with V^T read from the staged V tile
+//     by transposing LDS loads, and 8-byte output stores straight from the accumulators. K and V come in by full
+//     128-byte rows of two neighbouring heads; the next pair's are in flight while this one is computed.
 // Per workgroup 0.5 MiB of weights, 0.5 MiB of K and V and 64 KiB of Q come from L2; nothing but the output is written.
 #include <hip/hip_runtime.h>
 
@@ -26,7 +26,6 @@
 #include "kernel_common.h"
 
 namespace lc0mi {
-
 
 namespace {
 
@@ -42,24 +41,14 @@ __device__ __forceinline__ int LogitSlot(int c, int qq, int g4, int t) {
   return (((c * 16 + (qq ^ ((c >> 2) & 1))) * 4 + (g4 ^ (c & 3))) * 32) + t * 8;
 }
 
-// x combined with the values of the lanes 16, 32 and 48 away, with the lane-swap instructions of gfx950 (two vector
-// ALU operations per step instead of a round trip through the LDS crossbar). v_permlane16_swap exchanges the odd
-// 16-lane rows of its first register with the even rows of its second, v_permlane32_swap the upper half of the
-// first with the lower half of the second: fed the same value twice, the two registers afterwards hold the value
-// of this lane's row (half) and of its neighbour's. Written as assembly: the compiler's builtin for these
-// instructions loses track of the second result register. The no-ops cover the wait states between a vector ALU
-// write and a lane swap that reads it, and between the swap and its readers.
-template <typename F>
-__device__ __forceinline__ float Reduce4Rows(float x, F&& op) {
-  float a = x, b = x;
-  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-  float y = op(a, b);
-  float c = y;
-  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(y), "+v"(c));
-  return op(y, c);
-}
-
-// The same for two independent values at once (the two heads of a pair): the swaps of both share the wait states.
+// x0 and x1 (two independent values: the two heads of a pair), each combined with its values in the lanes 16, 32 and
+// 48 away, with the lane-swap instructions of gfx950 (two vector ALU operations per step instead of a round trip
+// through the LDS crossbar). v_permlane16_swap exchanges the odd 16-lane rows of its first register with the even
+// rows of its second, v_permlane32_swap the upper half of the first with the lower half of the second: fed the same
+// value twice, the two registers afterwards hold the value of this lane's row (half) and of its neighbour's. Written
+// as assembly: the compiler's builtin for these instructions loses track of the second result register. The no-ops
+// cover the wait states between a vector ALU write and a lane swap that reads it, and between the swap and its
+// readers; the swaps of the two values share them.
 template <typename F>
 __device__ __forceinline__ void Reduce4Rows2(float& x0, float& x1, F&& op) {
   float a0 = x0, b0 = x0, a1 = x1, b1 = x1;
@@ -173,13 +162,16 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
   // softmax elements:
   //   S^T tiles (16 keys x 16 queries, the whole head depth in one MFMA), plus the logits of phase 1 from LDS;
   //   softmax over the 16 values of a lane and the lanes 16, 32 and 48 away;
-  //   V transposed on the matrix cores (V_tile . I leaves a lane per depth index holding keys in the order of P);
-  //   O^T = V^T . P^T, so that a lane ends up with depth values of its own query, scales them by 1 / sum and stores.
+  //   V^T read from the staged V tile with the transposing LDS load of gfx950 (ds_read_b64_tr_b16), which hands a
+  //   lane per depth index four keys at a time, in the order of P;
+  //   O^T = V^T . P^T, so that a lane ends up with depth values of its own query, and 1 . P^T in the same way (the
+  //   row sums of the rounded P that the product itself uses) to scale them by before storing.
   // K and V are fetched for two neighbouring heads at once by 128-byte rows (both heads' 32 halves side by side), eight
   // lanes per row, so that every load instruction touches eight full cache lines instead of 32 partial ones; a tile
-  // of 32 rows then passes through this wave's 4 KiB of LDS (16-byte chunk c of row w at chunk c ^ ((w >> 1) & 7):
-  // both directions free of bank conflicts) to reach the lanes in operand layout. The loads of the next pair of heads
-  // are in flight while this one is computed.
+  // of 32 rows then passes through this wave's 4 KiB of LDS to reach the lanes in operand layout, 16-byte chunk c of
+  // row w at chunk c ^ swizzle(w): (w >> 1) & 7 for a K tile, read back as 16 bytes per lane from 16 rows, and
+  // ((w & 3) << 1) | ((w >> 2) & 1) for a V tile, read back as 8 bytes per lane from 4 rows x 32 bytes per 16 lanes
+  // (either way the lanes that are served together spread evenly over the banks).
   const int j = lane & 15, g4 = lane >> 4;
   const int lr = lane >> 3, ch = lane & 7;
   unsigned char* stg = stage_lds + wave * kVBytesPerWave;
@@ -237,12 +229,39 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
         fr[hb][th] = *reinterpret_cast<const ev8*>(stg + row * 128 + ((c ^ ((row >> 1) & 7)) * 16));
       }
   };
-  // Identity fragments: B operand of the transposing product, element (k, column) = [k == 16 dt + column].
-  ev8 ident[2];
+  // V^T fragments of a staged V tile: the transposing load treats the 16 lanes of a group as a 16 x 4 matrix of
+  // 16-bit elements D[s][c] (lane s supplies the address of its four contiguous elements) and returns to lane i the
+  // elements D[4 e + (i >> 2)][i & 3], e = 0..3. With lane s of group g4 pointing at key 16 h + 4 g4 + (s >> 2),
+  // depth 16 dt + 4 (s & 3), lane i = depth index receives the keys 16 h + 4 g4 + e of depth 16 dt + i.
+  typedef short short4v __attribute__((ext_vector_type(4)));
+  typedef short short8v __attribute__((ext_vector_type(8)));
+  auto stage_v_tile = [&](const ev8 (&raw)[4], ev8 (&vt)[2][2]) {   // vt[head][depth half]
 #pragma unroll
-  for (int dt = 0; dt < 2; dt++)
+    for (int i = 0; i < 4; i++) {
+      const int row = 8 * i + lr;
+      const int swz = ((row & 3) << 1) | ((row >> 2) & 1);
+      *reinterpret_cast<ev8*>(stg + row * 128 + ((ch ^ swz) * 16)) = raw[i];
+    }
 #pragma unroll
-    for (int e = 0; e < 8; e++) ident[dt][e] = (8 * g4 + e == 16 * dt + j) ? (ET)1.0f : (ET)0.0f;
+    for (int hb = 0; hb < 2; hb++)
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++) {
+        short4v part[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int row = 16 * h + 4 * g4 + (j >> 2), q = j & 3;
+          const int swz = ((row & 3) << 1) | ((row >> 2) & 1);
+          const int c = hb * 4 + 2 * dt + (q >> 1);
+          part[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) short4v*)(stg + row * 128 + ((c ^ swz) * 16) + (q & 1) * 8));
+        }
+        const short8v both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        vt[hb][dt] = __builtin_bit_cast(ev8, both);
+      }
+  };
+  ev8 ones;
+#pragma unroll
+  for (int e = 0; e < 8; e++) ones[e] = (ET)1.0f;
   const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
   // Software pipeline over the wave's four pairs of heads: while the softmax and P.V of pair p run (vector ALU work
@@ -263,18 +282,12 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
       for (int th = 0; th < 2; th++) o.st[hb][2 * tt + th] = Mfma16(kf[hb][th], d.q[hb], zero4);
   };
   auto prep_v = [&](const PairData& d, int tt, Prep& o) {
-    ev8 vr[2][2];
-    stage_tile(d.v[tt], vr);
+    ev8 vt[2][2];
+    stage_v_tile(d.v[tt], vt);
 #pragma unroll
     for (int hb = 0; hb < 2; hb++)
 #pragma unroll
-      for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-        for (int th = 0; th < 2; th++) {
-          const floatx4 tr = Mfma16(vr[hb][th], ident[dt], zero4);
-#pragma unroll
-          for (int e = 0; e < 4; e++) o.vt[hb][dt][tt][4 * th + e] = (ET)tr[e];
-        }
+      for (int dt = 0; dt < 2; dt++) o.vt[hb][dt][tt] = vt[hb][dt];
   };
 
   // Step 0..3 of preparing the pair whose rows are in `raw`; every step refills the registers it has emptied with the
@@ -315,7 +328,7 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
 
     if (more && FULL) prep_step(0, pi + 2, np);
     // scale, add the logits, maximum over the 64 keys of this lane's query: 16 here, 48 in the lanes 16, 32, 48 away
-    float sv[2][16], mx[2], sum[2];
+    float sv[2][16], mx[2];
 #pragma unroll
     for (int hb = 0; hb < 2; hb++) {
       const int c = ca + hb;
@@ -337,15 +350,12 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
 #pragma unroll
     for (int hb = 0; hb < 2; hb++) {
       const float neg_mx = -mx[hb] * kLog2e;
-      sum[hb] = 0.0f;
 #pragma unroll
       for (int e = 0; e < 16; e++) {
         sv[hb][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[hb][e], kLog2e, neg_mx));   // e^(s - mx) <= 1
-        sum[hb] += sv[hb][e];
       }
     }
     if (more && FULL) prep_step(2, pi + 2, np);
-    Reduce4Rows2(sum[0], sum[1], [](float a, float b) { return a + b; });
     ev8 pf[2][2];
 #pragma unroll
     for (int hb = 0; hb < 2; hb++)
@@ -357,7 +367,12 @@ __global__ __launch_bounds__(512, 1) void smolgen_attention_kernel(const half_t*
     // O^T = V^T . P^T: lane (query j, g4), register e = depth index 16 dt + 4 g4 + e
 #pragma unroll
     for (int hb = 0; hb < 2; hb++) {
-      const float inv = __builtin_amdgcn_rcpf(sum[hb]);   // 1 ulp
+      // Sum over all 64 keys of this lane's query, the same in all four registers: one more row block of the product,
+      // with ones for V^T (no additions and no lane exchanges on the vector ALU).
+      floatx4 den = zero4;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; s2++) den = Mfma16(ones, pf[hb][s2], den);
+      const float inv = __builtin_amdgcn_rcpf(den[0]);   // 1 ulp
       OutT* O = out + (long long)(b * 64 + kQueriesPerGroup * qt + j) * d_model + (ha + hb) * DEPTH + 4 * g4;
       const bool live = hb == 0 ? live_a : live_b;
 #pragma unroll

@@ -111,6 +111,12 @@ def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
     return (out, ms.value) if time_iters else out
 
 
+def set_cold_cache(mib):
+    """Profiling: with mib > 0 every timed launch (time_iters) is preceded by an untimed copy of mib MiB, so that the
+    kernel reads its operands from memory as inside a forward pass; 0 restores back-to-back launches."""
+    _lib().lc0mi_k_set_cold_cache(int(mib))
+
+
 def set_gemm_variant(variant):
     """-1 automatic, 0..2 direct-to-LDS 256x{256,192,128} tiles, 3 128x128, 4 64x64, 5 direct-to-LDS 128x128,
     6 row panels (16x16 to 64x32 outputs per workgroup, K split over its waves), 7 direct-to-LDS 128x64,

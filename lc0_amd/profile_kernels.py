@@ -33,7 +33,12 @@ def main():
                     help="operand values for gemm / gemm_f8: the same instruction stream runs faster on "
                          "constant operands (less switching power, higher sustained clock)")
     ap.add_argument("--variant", type=int, default=-1, help="force a GEMM tile variant (see kernels.set_gemm_variant)")
+    ap.add_argument("--cold-mib", type=int, default=0,
+                    help="copy this many MiB before every timed launch, so that the kernel reads its operands from "
+                         "memory as inside a forward pass (0: back-to-back launches on cached operands)")
     args = ap.parse_args()
+    if args.cold_mib > 0:
+        K.set_cold_cache(args.cold_mib)
     if args.variant >= 0:
         K.set_gemm_variant(args.variant)
     rng = np.random.default_rng(0)

@@ -340,6 +340,22 @@ def test_gemm_f8_vs_exact_product(variant, m, n, k):
         K.set_gemm_variant(-1)
 
 
+def test_cold_cache_timing_hook_leaves_results_alone():
+    """The profiling hook times launches one by one behind a cache-flushing copy: same output, a positive time."""
+    from lc0_amd import kernels as K
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((512, 256), dtype=np.float32).astype(np.float16)
+    g, b = np.ones(256, np.float32), np.zeros(256, np.float32)
+    warm, ms_warm = K.layer_norm(x, x, g, b, 0.5, 1e-6, time_iters=3)
+    K.set_cold_cache(64)
+    try:
+        cold, ms_cold = K.layer_norm(x, x, g, b, 0.5, 1e-6, time_iters=3)
+    finally:
+        K.set_cold_cache(0)
+    assert np.array_equal(warm, cold)
+    assert ms_warm > 0 and ms_cold > 0
+
+
 def test_layer_norm_f8_output():
     from lc0_amd import kernels as K
     rng = np.random.default_rng(77)
