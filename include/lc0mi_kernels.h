@@ -51,6 +51,13 @@ int lc0mi_k_set_gemm_variant(int variant);
  * lc0mi_k_attention and lc0mi_k_smolgen_attention (half output) hold bfloat16 values and the kernels run their bf16
  * instances (precision=bf16 of the network; the reference's type: src/utils/bf16_utils.h). 0 switches back to half. */
 int lc0mi_k_set_bf16(int on);
+/* Test hook, process-wide: the kind of output stores of lc0mi_k_gemm and lc0mi_k_gemm_f8 (256-row tiles of the
+ * direct-to-LDS kernel; others always store ordinarily) and of lc0mi_k_layer_norm: 0 by output size (ordinary or
+ * streaming), 1 by output size (ordinary or written through), 2 ordinary, 3 streaming (non-temporal), 4 written
+ * through at system scope (the layer norm then also reads x with non-temporal loads). The network picks 1 and the
+ * written-through layer norm for the big tensors of an encoder layer while a layer's activations fit the memory-side
+ * cache. No counterpart in the reference. */
+int lc0mi_k_set_out_stores(int kind);
 /* Profiling hook, process-wide: with mib > 0 every timed launch (time_iters of the entry points here) is preceded by
  * an untimed copy of mib MiB, so that the kernel finds its operands in memory rather than in L2 or the memory-side
  * cache, as it does between other kernels inside a forward pass; the timed launches are then timed one by one.

@@ -415,11 +415,27 @@ __device__ __forceinline__ void DmaToLds16(const void* gptr, void* lds_base) {
   }
 }
 
+template <int STORES>
+__device__ __forceinline__ void StoreOut16(void* dst, intx4 val) {
+  if constexpr (STORES == 1) {
+    __builtin_nontemporal_store(val, reinterpret_cast<intx4*>(dst));
+  } else if constexpr (STORES == 2) {
+    // (the no-op covers the wait states that the hardware needs between a store of more than eight bytes and a vector
+    // ALU write to its data registers - two on this part; the compiler adds them after its own stores and does not
+    // look into this one: without them the 256x128 tiles, which reuse the registers at once, stored wrong values)
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" ::"v"(dst), "v"(val) : "memory");
+  } else {
+    *reinterpret_cast<intx4*>(dst) = val;
+  }
+}
+
 // The same kernel serves fp16 operands (Args = GemmArgs: BKB = 128 bytes = 64
 // halves per tile row, v_mfma_f32_32x32x16_f16) and e4m3 operands (Args =
 // GemmF8Args: 128 bytes = 128 values per row, v_mfma_f32_32x32x64_f8f6f4);
 // BKB is the k-tile in bytes. OutT is half_t or uint8_t (e4m3, fp8 operands only).
-// STREAM: the output is written with streaming (non-temporal) stores.
+// STORES: how the 16-byte output vectors are stored: 0 ordinary stores (the output stays in L2 and the memory-side
+// cache), 1 streaming (non-temporal) stores, 2 stores written through at system scope (they leave L2 alone like the
+// streaming ones, but what they wrote is found faster by the next kernel; plain epilogue only).
 // EPI (fp16 operands only): 0 the plain epilogue, 1 the consumer and 2 the producer side of a folded layer norm
 // (GemmArgs::row_stats / GemmArgs::skip).
 // NSTAGES k-tiles of LDS: NSTAGES - 1 of them are in flight while one is consumed. Two stages suffice when the
@@ -427,7 +443,7 @@ __device__ __forceinline__ void DmaToLds16(const void* gptr, void* lds_base) {
 // every workgroup streams weights nobody has touched since the previous pass) a k-tile takes longer to arrive than
 // to consume, and more stages hide that.
 // ET (fp16-type operands only): half_t or bf16_t; the output type is then ET as well.
-template <int BM, int BN, int BKB, int WAVES_M, int WAVES_N, typename Args, typename OutT, bool STREAM = false,
+template <int BM, int BN, int BKB, int WAVES_M, int WAVES_N, typename Args, typename OutT, int STORES = 0,
           int EPI = 0, int NSTAGES = 2, typename ET = half_t>
 // Second launch bound = waves per SIMD: with small wave tiles two workgroups share a CU
 // (4 waves per SIMD, at most 128 VGPRs) and overlap each other's prologue and epilogue.
@@ -782,11 +798,7 @@ void gemm_dma_kernel(Args p) {
           if (!ok) s1 = s2 = 0.0f;
           if (ok) {
             half_t* dst = reinterpret_cast<half_t*>(C) + (long long)m * p.ldc + n;
-            if constexpr (STREAM) {
-              __builtin_nontemporal_store(__builtin_bit_cast(intx4, o), reinterpret_cast<intx4*>(dst));
-            } else {
-              *reinterpret_cast<half8*>(dst) = o;
-            }
+            StoreOut16<STORES>(dst, __builtin_bit_cast(intx4, o));
           }
           // Sum over the CHUNKS_PER_ROW (4 or 8) neighbouring lanes of a row, with data-parallel-primitive moves.
           static_assert(CHUNKS_PER_ROW == 4 || CHUNKS_PER_ROW == 8, "row reduction written for 4 or 8 lanes per row");
@@ -809,11 +821,7 @@ void gemm_dma_kernel(Args p) {
           OutT* dst = C + (long long)m * p.ldc + n;
           if (vec_ok && n + OV - 1 < N) {
             const intx4 val = *reinterpret_cast<const intx4*>(&strip[row * EPI_STRIDE + ch * OV]);
-            if constexpr (STREAM) {
-              __builtin_nontemporal_store(val, reinterpret_cast<intx4*>(dst));
-            } else {
-              *reinterpret_cast<intx4*>(dst) = val;
-            }
+            StoreOut16<STORES>(dst, val);
           } else {
             for (int e = 0; e < OV && n + e < N; e++) dst[e] = strip[row * EPI_STRIDE + ch * OV + e];
           }
@@ -850,21 +858,31 @@ inline bool StreamOutput(long long m, long long n, long long batch, int elem_byt
   return bytes >= (64LL << 20) || (m >= 16384 && bytes >= (32LL << 20));
 }
 
+// The STORES instance for a launch: what the caller asked for (GemmArgs::out_stores), or by the size rule above.
+inline int OutputStores(int requested, long long m, long long n, long long batch, int elem_bytes) {
+  if (requested == kStoresCached) return 0;
+  if (requested == kStoresStream) return 1;
+  if (requested == kStoresWriteThrough) return 2;
+  if (!StreamOutput(m, n, batch, elem_bytes)) return 0;
+  return requested == kStoresAutoKeep ? 2 : 1;
+}
+
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int NSTAGES = 2>
 void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
   dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, a.batch);
   const dim3 block(WAVES_M * WAVES_N * 64);
-  auto launch = [&](auto stream_tag) {
-    constexpr bool S = decltype(stream_tag)::value;
+  auto launch = [&](auto stores_tag) {
+    constexpr int S = decltype(stores_tag)::value;
+    constexpr int SF = S == 2 ? 1 : S;   // (the folded-layer-norm epilogues know cached and streaming stores only)
     // The folded-layer-norm epilogues exist with two stages only (LaunchGemmDmaStaged sends them there).
     if (a.skip != nullptr) {
       if constexpr (((BN / WAVES_N) % 64 == 0 || BN / WAVES_N == 32) && NSTAGES == 2) {
-        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 2, 2>), grid, block, 0,
+        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, SF, 2, 2>), grid, block, 0,
                            stream, a);
       }
     } else if (a.row_stats != nullptr) {
       if constexpr (NSTAGES == 2) {
-        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, S, 1, 2>), grid, block, 0,
+        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BK * 2, WAVES_M, WAVES_N, GemmArgs, half_t, SF, 1, 2>), grid, block, 0,
                            stream, a);
       }
     } else if (a.bf16) {
@@ -876,12 +894,11 @@ void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
     }
   };
   if constexpr (BM == 256) {
-    if (StreamOutput(a.M, a.N, a.batch, 2)) {
-      launch(std::true_type{});
-      return;
-    }
+    const int stores = OutputStores(a.out_stores, a.M, a.N, a.batch, 2);
+    if (stores == 1) return launch(std::integral_constant<int, 1>{});
+    if (stores == 2) return launch(std::integral_constant<int, 2>{});
   }
-  launch(std::false_type{});
+  launch(std::integral_constant<int, 0>{});
 }
 
 // As many LDS stages (2 to 4) as leave room on the CUs for all of the launch's workgroups at once: with one
@@ -907,22 +924,25 @@ void LaunchGemmDmaF8(const GemmF8Args& a, hipStream_t stream) {
   dim3 grid((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, 1);
   const dim3 block(WAVES_M * WAVES_N * 64);
   if constexpr (BM == 256) {
-    if (StreamOutput(a.M, a.N, 1, a.out_f8 ? 1 : 2)) {
+    const int stores = OutputStores(a.out_stores, a.M, a.N, 1, a.out_f8 ? 1 : 2);
+    auto launch = [&](auto stores_tag) {
+      constexpr int S = decltype(stores_tag)::value;
       if (a.out_f8) {
-        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, uint8_t, true>), grid, block, 0,
+        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, uint8_t, S>), grid, block, 0,
                            stream, a);
       } else {
-        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, half_t, true>), grid, block, 0,
+        hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, half_t, S>), grid, block, 0,
                            stream, a);
       }
-      return;
-    }
+    };
+    if (stores == 1) return launch(std::integral_constant<int, 1>{});
+    if (stores == 2) return launch(std::integral_constant<int, 2>{});
   }
   if (a.out_f8) {
-    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, uint8_t, false, 0, NSTAGES>), grid,
+    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, uint8_t, 0, 0, NSTAGES>), grid,
                        block, 0, stream, a);
   } else {
-    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, half_t, false, 0, NSTAGES>), grid,
+    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, BKB, WAVES_M, WAVES_N, GemmF8Args, half_t, 0, 0, NSTAGES>), grid,
                        block, 0, stream, a);
   }
 }

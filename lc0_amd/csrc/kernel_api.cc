@@ -110,6 +110,8 @@ int Guard(F&& f) {
 namespace {
 // Test hook (lc0mi_k_set_bf16): the 16-bit buffers of the entry points that say so hold bfloat16 instead of half.
 bool g_bf16 = false;
+// Test hook (lc0mi_k_set_out_stores): the kind of output stores of lc0mi_k_gemm, lc0mi_k_gemm_f8 and lc0mi_k_layer_norm.
+int g_out_stores = lc0mi::kStoresAuto;
 }  // namespace
 
 extern "C" {
@@ -117,6 +119,13 @@ extern "C" {
 int lc0mi_k_set_cold_cache(int mib) {
   g_cold_mib = mib > 0 ? mib : 0;
   return 0;
+}
+
+int lc0mi_k_set_out_stores(int kind) {
+  return Guard([&] {
+    if (kind < lc0mi::kStoresAuto || kind > lc0mi::kStoresWriteThrough) throw Error("bad kind of output stores");
+    g_out_stores = kind;
+  });
 }
 
 int lc0mi_k_set_bf16(int on) {
@@ -144,6 +153,7 @@ int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* 
     g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
     g.M = M; g.N = N; g.K = K; g.batch = batch; g.scale = scale; g.act = act; g.out_f32 = out_f32 != 0;
     g.bf16 = g_bf16;
+    g.out_stores = g_out_stores;
     lc0mi::LaunchGemm(g, nullptr);
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());
@@ -313,12 +323,15 @@ int lc0mi_k_layer_norm(const uint16_t* x, const uint16_t* skip, const float* gam
     auto* dy = reinterpret_cast<half_t*>(dev.Alloc(n * 2));
     float* dg = dev.Put(gamma, (size_t)C);
     float* db = dev.Put(beta, (size_t)C);
-    lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr, nullptr, 1.0f, g_bf16);
+    const bool through = g_out_stores == lc0mi::kStoresWriteThrough;
+    lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr, nullptr, 1.0f, g_bf16, through);
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());
     K_CHECK(hipMemcpy(y, dy, n * 2, hipMemcpyDeviceToHost));
     if (time_iters > 0 && ms) {
-      *ms = TimeLaunches(time_iters, [&] { lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr); });
+      *ms = TimeLaunches(time_iters, [&] {
+        lc0mi::LaunchLayerNorm(dx, ds, dy, dg, db, rows, C, alpha, eps, nullptr, nullptr, 1.0f, g_bf16, through);
+      });
     }
   });
 }
@@ -624,6 +637,7 @@ int lc0mi_k_gemm_f8(const uint8_t* A, int lda, const uint8_t* W, int ldw, const 
     g.col_scale = dev.Put(col_scale, (size_t)N);
     g.bias = bias ? dev.Put(bias, (size_t)N) : nullptr;
     g.M = M; g.N = N; g.K = K; g.act = act; g.out_f8 = out_f8 != 0; g.out_mul = out_mul;
+    g.out_stores = g_out_stores;
     lc0mi::LaunchGemmF8(g, nullptr);
     K_CHECK(hipDeviceSynchronize());
     K_CHECK(hipGetLastError());

@@ -20,6 +20,15 @@ enum class Dtype { kHalf, kBf16, kFloat };
 // Requirements: K % 8 == 0, lda % 8 == 0, ldw % 8 == 0, 16-byte aligned bases
 // and batch strides; M, N arbitrary. bias may be null (then no bias; the
 // activation is still applied). out_f32 selects float output.
+// How a large GEMM writes its output (GemmArgs::out_stores, GemmF8Args::out_stores; only the 256-row tiles of the
+// direct-to-LDS kernel know more than ordinary stores). kStoresAuto: ordinary stores, or streaming (non-temporal)
+// ones for an output so large that it would push the operands out of L2. kStoresAutoKeep: the same size rule, but
+// with stores written through at system scope in place of the streaming ones: they leave L2 alone as well, and the
+// kernel that reads the output next finds it in the memory-side cache, which streamed data is not. For outputs
+// whose reader is bound by memory (attention, layer norm) as long as a layer's activations fit that cache.
+// The last three name a kind of store outright.
+enum OutStores { kStoresAuto = 0, kStoresAutoKeep = 1, kStoresCached = 2, kStoresStream = 3, kStoresWriteThrough = 4 };
+
 struct GemmArgs {
   const half_t* A = nullptr; int lda = 0; long long strideA = 0;
   const half_t* W = nullptr; int ldw = 0; long long strideW = 0;
@@ -31,6 +40,7 @@ struct GemmArgs {
   bool out_f32 = false;
   // A, W and (unless out_f32) C hold bfloat16 instead of half values. Not with the folded layer-norm fields.
   bool bf16 = false;
+  int out_stores = kStoresAuto;
   // split_k > 1: the K range is cut into split_k slices computed by different
   // workgroups; slice s stores its partial sums (float, out_f32 required, no
   // activation, bias only in slice 0) at C + s * split_stride. The consumer adds
@@ -92,6 +102,7 @@ struct GemmF8Args {
   int act = 3;
   bool out_f8 = false;
   float out_mul = 1.0f;
+  int out_stores = kStoresAuto;
 };
 void LaunchGemmF8(const GemmF8Args& args, hipStream_t stream);
 const char* GemmF8VariantName(const GemmF8Args& args);
@@ -158,9 +169,12 @@ void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_s
 // rows x C layer norm: y = beta + gamma * (t - mean) / sqrt(var + eps) with
 // t = x * alpha + skip (skip may be null). x, skip, y may alias. C % 8 == 0, C <= 8192.
 // y_f8 (optional): also receives e4m3(y * f8_mul), saturating, the operand of a following fp8 GEMM.
+// through: for tensors far larger than L2 inside a pass whose activations fit the memory-side cache: x (not read
+// again) comes in with non-temporal loads, y goes out with stores written through at system scope, where the
+// kernels that read it next find it (GemmArgs::out_stores has the measurements).
 void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
                      int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8 = nullptr,
-                     float f8_mul = 1.0f, bool bf16 = false);
+                     float f8_mul = 1.0f, bool bf16 = false, bool through = false);
 // The same for any element type (half_t, bf16_t, float) and any row length, with an activation applied to x first:
 // y = norm(act(x) * alpha + skip). One workgroup per row, scalar accesses.
 template <typename T>

@@ -167,7 +167,7 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restric
                                                          half_t* y, uint8_t* yq, float q_mul,
                                                          const float* __restrict__ gamma,
                                                          const float* __restrict__ beta, int rows, int C,
-                                                         float alpha, float eps) {
+                                                         float alpha, float eps, bool through) {
   using ev8 = typename Vec16<ET>::v8;
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -181,7 +181,9 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restric
   for (int i = 0; i < NV; i++) {
     int v = lane + i * 64;
     if (v < nvec) {
-      ev8 hx = *reinterpret_cast<const ev8*>(xr + v * 8);
+      // (through: x is not read again and is kept out of the caches on its way in)
+      ev8 hx = through ? __builtin_nontemporal_load(reinterpret_cast<const ev8*>(xr + v * 8))
+                       : *reinterpret_cast<const ev8*>(xr + v * 8);
       if (sr) {
         ev8 hs = *reinterpret_cast<const ev8*>(sr + v * 8);
 #pragma unroll
@@ -220,7 +222,12 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const half_t* __restric
         f[e] = beta[v * 8 + e] + gamma[v * 8 + e] * (t[i][e] - mean) * den;
         o[e] = (ET)f[e];
       }
-      *reinterpret_cast<ev8*>(yr + v * 8) = o;
+      if (through) {   // written through at system scope: past L2, into the memory-side cache (the no-op: the wait
+                       // states between a 16-byte store and a vector ALU write to its data registers)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" ::"v"(yr + v * 8), "v"(o) : "memory");
+      } else {
+        *reinterpret_cast<ev8*>(yr + v * 8) = o;
+      }
       if (yq) {  // e4m3 copy of the same row for the next fp8 GEMM
         uint2 q;
         q.x = PackFp8x4(f[0] * q_mul, f[1] * q_mul, f[2] * q_mul, f[3] * q_mul);
@@ -392,12 +399,13 @@ void LaunchLayerNormRows(const float* x_f32, int n_partials, long long partial_s
 }
 
 void LaunchLayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
-                     int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8, float f8_mul, bool bf16) {
+                     int rows, int C, float alpha, float eps, hipStream_t stream, uint8_t* y_f8, float f8_mul, bool bf16,
+                     bool through) {
   if (rows <= 0) return;
   dim3 grid((rows + 3) / 4), block(256);
   auto launch = [&](auto nv_tag, auto elem_tag) {
     hipLaunchKernelGGL((layer_norm_kernel<decltype(nv_tag)::value, decltype(elem_tag)>), grid, block, 0, stream, x, skip,
-                       y, y_f8, f8_mul, gamma, beta, rows, C, alpha, eps);
+                       y, y_f8, f8_mul, gamma, beta, rows, C, alpha, eps, through);
   };
   auto by_width = [&](auto elem_tag) {
     if (C <= 512) launch(std::integral_constant<int, 1>{}, elem_tag);

@@ -292,6 +292,7 @@ struct ModelState {
   int fused_smolgen_min_batch_ = 72;
   int dense1_split_min_batch_ = 112;   // smallest batch whose smolgen dense1 splits K between workgroups
   bool qkv_first_ = true;
+  bool write_through_ = true;   // big activations go to the memory-side cache while a layer's worth fits it
   int chain_latency_max_batch_ = 128;   // largest fp16 batch whose smolgen chain takes the shortest-latency GEMM variants
   half_t* smolgen_wfrag_ = nullptr;   // smolgen_w in the fragment order of smolgen_attention_kernel (null: not fused)
   bool any_smolgen_ = false;
@@ -400,7 +401,7 @@ class Mi355xNetwork : public Network, protected ModelState {
   Linear MakeLinearNormFolded(const Vec& w, const Vec& b, const Vec& gamma, const Vec& beta, int out, int in);
   LinearF8 MakeLinearF8(const Vec& w, int out, int in);
   void GemmF8(const char* name, const uint8_t* A, const Linear& lin, const LinearF8& q, void* C, int M, int act,
-              bool out_f8, float out_mul, hipStream_t st = nullptr);
+              bool out_f8, float out_mul, hipStream_t st = nullptr, int out_stores = kStoresAuto);
   void RecordAbsMax(const half_t* x, size_t n, int slot, hipStream_t st = nullptr);
   // Slot of the calibration maxima: 4 per layer plus the last layer's output, then 3 per layer for the smolgen chain.
   int SmolgenSlot(size_t li, int which) const { return static_cast<int>(4 * encoders_.size() + 1 + 3 * li + which); }
@@ -431,13 +432,14 @@ class Mi355xNetwork : public Network, protected ModelState {
   void Timed(const char* name, double flops, double bytes, F&& launch, hipStream_t st = nullptr);
   void Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act,
             bool out_f32 = false, hipStream_t st = nullptr, int split_k = 1, bool latency_first = false,
-            const NormFold* fold = nullptr);
+            const NormFold* fold = nullptr, int out_stores = kStoresAuto);
   GemmArgs MakeGemmArgs(const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M, int act, bool out_f32,
                         int split_k, bool latency_first, const NormFold* fold) const;
   // Kernels other than the dense layers, by the network's element type (and, for 16-bit types, by whether the tuned
   // kernel takes the shape).
   void LayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta, int rows, int C,
-                 float alpha, float eps, hipStream_t st = nullptr, uint8_t* y_f8 = nullptr, float f8_mul = 1.0f);
+                 float alpha, float eps, hipStream_t st = nullptr, uint8_t* y_f8 = nullptr, float f8_mul = 1.0f,
+                 bool through = false);
   void LayerNormRows(const half_t* x, half_t* y, const float* gamma, const float* beta, int rows, int C,
                      hipStream_t st);
   void Attention(const half_t* qkv, const half_t* bias, half_t* out, int B, int heads, int depth, hipStream_t st);
@@ -664,7 +666,7 @@ GemmArgs Mi355xNetwork::MakeGemmArgs(const half_t* A, int lda, const Linear& lin
 
 void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linear& lin, void* C, int ldc, int M,
                          int act, bool out_f32, hipStream_t st, int split_k, bool latency_first,
-                         const NormFold* fold) {
+                         const NormFold* fold, int out_stores) {
   if (st == nullptr) st = stream_;
   if (dtype_ == Dtype::kFloat) {
     if (split_k != 1 || fold != nullptr) throw Error("internal: split or folded GEMM requested in the float configuration");
@@ -683,6 +685,7 @@ void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linea
   }
   GemmArgs g = MakeGemmArgs(A, lda, lin, C, ldc, M, act, out_f32, split_k, latency_first, fold);
   g.bf16 = dtype_ == Dtype::kBf16;
+  g.out_stores = out_stores;
   if (fold != nullptr && fold->parts_out != nullptr) *fold->parts_out = GemmStatsParts(g);
   const double flops = 2.0 * M * lin.out * lin.in;
   const double bytes = 2.0 * (static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in) +
@@ -694,13 +697,14 @@ void Mi355xNetwork::Gemm(const char* name, const half_t* A, int lda, const Linea
 }
 
 void Mi355xNetwork::LayerNorm(const half_t* x, const half_t* skip, half_t* y, const float* gamma, const float* beta,
-                              int rows, int C, float alpha, float eps, hipStream_t st, uint8_t* y_f8, float f8_mul) {
+                              int rows, int C, float alpha, float eps, hipStream_t st, uint8_t* y_f8, float f8_mul,
+                              bool through) {
   if (st == nullptr) st = stream_;
   if (dtype_ == Dtype::kFloat) {
     LaunchLayerNormGeneric<float>(reinterpret_cast<const float*>(x), reinterpret_cast<const float*>(skip),
                                   reinterpret_cast<float*>(y), gamma, beta, rows, C, alpha, eps, kActNone, st);
   } else {
-    LaunchLayerNorm(x, skip, y, gamma, beta, rows, C, alpha, eps, st, y_f8, f8_mul, dtype_ == Dtype::kBf16);
+    LaunchLayerNorm(x, skip, y, gamma, beta, rows, C, alpha, eps, st, y_f8, f8_mul, dtype_ == Dtype::kBf16, through);
   }
 }
 
@@ -816,7 +820,7 @@ LinearF8 Mi355xNetwork::MakeLinearF8(const Vec& w, int out, int in) {
 }
 
 void Mi355xNetwork::GemmF8(const char* name, const uint8_t* A, const Linear& lin, const LinearF8& q, void* C, int M,
-                           int act, bool out_f8, float out_mul, hipStream_t st) {
+                           int act, bool out_f8, float out_mul, hipStream_t st, int out_stores) {
   if (st == nullptr) st = stream_;
   GemmF8Args g;
   g.A = A; g.lda = lin.in;
@@ -828,6 +832,7 @@ void Mi355xNetwork::GemmF8(const char* name, const uint8_t* A, const Linear& lin
   g.act = act;
   g.out_f8 = out_f8;
   g.out_mul = out_mul;
+  g.out_stores = out_stores;
   const double flops = 2.0 * M * lin.out * lin.in;
   const double bytes = static_cast<double>(M) * lin.in + static_cast<double>(lin.out) * lin.in +
                        static_cast<double>(M) * lin.out * (out_f8 ? 1 : 2);
@@ -1041,6 +1046,7 @@ Mi355xNetwork::Mi355xNetwork(const WeightsFile& file, Options& options) {
   fused_smolgen_min_batch_ = options.GetInt("fused_smolgen_min_batch", 72);
   dense1_split_min_batch_ = options.GetInt("dense1_split_min_batch", 112);
   qkv_first_ = options.GetBool("qkv_first", true);
+  write_through_ = options.GetBool("write_through", true);
   chain_latency_max_batch_ = options.GetInt("chain_latency_max_batch", 128);
   fp8_fp16_layers_ = options.GetInt("fp8_fp16_layers", 0);
   if (fp8_fp16_layers_ < 0) throw Error("fp8_fp16_layers must not be negative.");
@@ -1878,6 +1884,17 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
   // norms of a layer run inside the GEMM before them (residual + row sums) and the GEMMs after them (row
   // normalisation of the product), and x_ carries the un-normalised sums from layer to layer.
   const bool fold = !fp8_ && !calibrating_ && CanFoldLayerNorms(B);
+  // Where the outputs of a layer's kernels go. A layer writes about eight [T x d_model] tensors of two bytes (the
+  // projection's counts for three); while two layers' worth fit the 256 MiB memory-side cache (up to 512 positions
+  // at d_model 1024), the large GEMMs whose output is read next by a kernel that is bound by memory (QKV before the
+  // attention, attention output and FFN2 before the layer norms) write it through to that cache instead of streaming
+  // it past it, and the layer norms do the same. FFN1 keeps streaming: FFN2 does not mind where its operand comes
+  // from, and 1.5 tensors' worth of cache stay free for the others. Same-machine runs of the 15x1024 net, fp16
+  // 384 positions +1.5 %, 256 +1.8 % (the attention kernel inside a pass 59 -> 46-52 us, both layer norms together
+  // 43 -> 37), 512 +0 %, 1024 -4.5 % if forced there; e4m3 256 +1.9 %, 512 +0.5 %, 1024 -1.2 % if forced.
+  const bool cache_fits = write_through_ && static_cast<size_t>(T) * d_model_ * 16 <= (static_cast<size_t>(512) << 20);
+  const int keep = cache_fits ? kStoresAutoKeep : kStoresAuto;
+  const bool ln_through = cache_fits && dtype_ != Dtype::kFloat && static_cast<size_t>(T) * emb_ * 2 >= (32u << 20);
   const float* pend_stats = nullptr;   // row sums of x_ when it holds an un-normalised sum
   const float *pend_gamma = nullptr, *pend_beta = nullptr;
   int pend_parts = 0, mid_parts = 0;
@@ -1904,13 +1921,18 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
     // The generator layer (smolgen_w) runs inside the attention kernel where that kernel serves the shape.
     // (not with e4m3 operands in the chain: the generator is then an fp8 GEMM of its own)
     const bool chain_f8 = f8 && q_smolgen_ && e.has_smolgen;
-    const bool fused_gen = e.has_smolgen && smolgen_wfrag_ != nullptr && B >= fused_smolgen_min_batch_ && !chain_f8;
+    // The generator layer inside the attention kernel (fp16 operands there). With the chain in e4m3 by the default
+    // fp8_gemms=auto that still holds - the three layers before it run on e4m3 operands, the generator on the halves
+    // the last row norm writes: 4 to 8 % of a pass at 96 to 512 positions against an e4m3 generator GEMM of its own
+    // plus the plain attention kernel. An explicit fp8_gemms=...+smolgen keeps all four layers in e4m3.
+    const bool fused_gen = e.has_smolgen && smolgen_wfrag_ != nullptr && B >= fused_smolgen_min_batch_ &&
+                           (!chain_f8 || q_smolgen_auto_);
     auto launch_qkv = [&] {
       if (f8 && q_qkv_) {
-        GemmF8("gemm_qkv", xq_, e.qkv, e.qkv8, qkv_, T, kActNone, false, 1.0f);
+        GemmF8("gemm_qkv", xq_, e.qkv, e.qkv8, qkv_, T, kActNone, false, 1.0f, nullptr, keep);
       } else {
         Gemm("gemm_qkv", x_, emb_, norm_in ? e.qkv_n : e.qkv, qkv_, 3 * d_model_, T, kActNone, false, nullptr, 1, false,
-             norm_in ? &cons_in : nullptr);
+             norm_in ? &cons_in : nullptr, keep);
       }
     };
     // With two streams the projection is recorded before the chain: a replayed graph then keeps it on the hardware
@@ -1938,11 +1960,13 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
                               1e-3f, ss, false, sg2q_, 1.0f / e.s_sg2);
         }, ss);
         GemmF8("gemm_smolgen_dense2", sg2q_, e.sg_dense2, e.sg_dense28, sg3_, B, smolgen_act_, false, 1.0f, ss);
-        Timed("layer_norm_rows", 0.0, 5.0 * B * sg_gen_, [&] {
+        Timed("layer_norm_rows", 0.0, (fused_gen ? 4.0 : 5.0) * B * sg_gen_, [&] {
           LaunchLayerNormRows(nullptr, 0, 0, sg3_, kActNone, nullptr, sg3_, e.sg_ln2_g, e.sg_ln2_b, B, sg_gen_, 1.0f,
-                              1e-3f, ss, false, sg3q_, 1.0f / e.s_sg3);
+                              1e-3f, ss, false, fused_gen ? nullptr : sg3q_, 1.0f / e.s_sg3);
         }, ss);
-        GemmF8("gemm_smolgen_global", sg3q_, smolgen_w_, e.sg_global8, sbias_, B * heads_, kActNone, false, 1.0f, ss);
+        if (!fused_gen) {
+          GemmF8("gemm_smolgen_global", sg3q_, smolgen_w_, e.sg_global8, sbias_, B * heads_, kActNone, false, 1.0f, ss);
+        }
       } else if (dtype_ == Dtype::kFloat) {
         SmolgenChain(e, x_, emb_, heads_, sg_hc_, sg_hs_, sg_gen_, sg1_, sg2_, sg3_, sbias_, B, ss, chain_first);
       } else {
@@ -1997,11 +2021,11 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
         LaunchSmolgenAttentionF8Out(qkv_, sg3_, smolgen_wfrag_, attq_, 1.0f / e.s_att, B, heads_, depth_, gen_sz,
                                     att_scale, stream_);
       });
-      GemmF8("gemm_mha_dense", attq_, e.dense, e.dense8, t_, T, kActNone, false, 1.0f);
+      GemmF8("gemm_mha_dense", attq_, e.dense, e.dense8, t_, T, kActNone, false, 1.0f, nullptr, keep);
     } else if (att_f8) {
       Timed("attention", att_flops, att_bytes,
             [&] { LaunchAttentionF8Out(qkv_, bias, attq_, 1.0f / e.s_att, B, heads_, att_scale, stream_, depth_); });
-      GemmF8("gemm_mha_dense", attq_, e.dense, e.dense8, t_, T, kActNone, false, 1.0f);
+      GemmF8("gemm_mha_dense", attq_, e.dense, e.dense8, t_, T, kActNone, false, 1.0f, nullptr, keep);
     } else {
       if (fused_gen) {
         Timed("smolgen_attention", att_flops, att_bytes, [&] {
@@ -2029,11 +2053,12 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
         }
         continue;
       }
-      Gemm("gemm_mha_dense", att_, d_model_, e.dense, t_, emb_, T, kActNone);
+      Gemm("gemm_mha_dense", att_, d_model_, e.dense, t_, emb_, T, kActNone, false, nullptr, 1, false, nullptr, keep);
     }
     const bool ln1_f8 = f8 && q_ffn1_;
     Timed("layer_norm_skip", 0.0, (ln1_f8 ? 7.0 : 3.0 * es_) * T * emb_, [&] {
-      LayerNorm(t_, x_, x_, e.ln1_g, e.ln1_b, T, emb_, alpha_, eps_, stream_, ln1_f8 ? xq_ : nullptr, 1.0f / e.s_x1);
+      LayerNorm(t_, x_, x_, e.ln1_g, e.ln1_b, T, emb_, alpha_, eps_, stream_, ln1_f8 ? xq_ : nullptr, 1.0f / e.s_x1,
+                ln_through);
     });
     if (calibrating_) RecordAbsMax(x_, nx, static_cast<int>(4 * li + 2));
     const bool ffn_f8 = f8 && q_ffn2_;   // FFN2 reads an e4m3 operand
@@ -2050,14 +2075,14 @@ void Mi355xNetwork::ForwardAttentionBody(int B) {
       }
     }
     if (ffn_f8) {
-      GemmF8("gemm_ffn2", ffnq_, e.ffn2, e.ffn28, t_, T, kActNone, false, 1.0f);
+      GemmF8("gemm_ffn2", ffnq_, e.ffn2, e.ffn28, t_, T, kActNone, false, 1.0f, nullptr, keep);
     } else {
-      Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, t_, emb_, T, kActNone);
+      Gemm("gemm_ffn2", ffn_, dff_, e.ffn2, t_, emb_, T, kActNone, false, nullptr, 1, false, nullptr, keep);
     }
     const bool ln2_f8 = f8_any && li + 1 < n_f8_layers && (q_qkv_ || q_smolgen_);   // the next layer reads an e4m3 copy
     Timed("layer_norm_skip", 0.0, (ln2_f8 ? 7.0 : 3.0 * es_) * T * emb_, [&] {
       LayerNorm(t_, x_, x_, e.ln2_g, e.ln2_b, T, emb_, alpha_, eps_, stream_, ln2_f8 ? xq_ : nullptr,
-                last ? 1.0f : 1.0f / encoders_[li + 1].s_x);
+                last ? 1.0f : 1.0f / encoders_[li + 1].s_x, ln_through);
     });
     if (calibrating_) RecordAbsMax(x_, nx, static_cast<int>(4 * li + 4));
   }

@@ -111,6 +111,15 @@ def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
     return (out, ms.value) if time_iters else out
 
 
+STORES_AUTO, STORES_AUTO_KEEP, STORES_CACHED, STORES_STREAM, STORES_WRITE_THROUGH = range(5)
+
+
+def set_out_stores(kind):
+    """Kind of output stores of gemm, gemm_f8 (256-row direct-to-LDS tiles) and layer_norm: STORES_AUTO (by size),
+    STORES_AUTO_KEEP, STORES_CACHED, STORES_STREAM, STORES_WRITE_THROUGH."""
+    _check(_lib().lc0mi_k_set_out_stores(int(kind)))
+
+
 def set_cold_cache(mib):
     """Profiling: with mib > 0 every timed launch (time_iters) is preceded by an untimed copy of mib MiB, so that the
     kernel reads its operands from memory as inside a forward pass; 0 restores back-to-back launches."""

@@ -96,6 +96,7 @@ class Mi355xNetwork : public Network {
       add("fp8_fp16_layers", std::to_string(options.GetOrDefault<int>("fp8_fp16_layers", 0)));
     }
     add("qkv_first", options.GetOrDefault<bool>("qkv_first", true) ? "true" : "false");
+    add("write_through", options.GetOrDefault<bool>("write_through", true) ? "true" : "false");
     add("policy_head", options.GetOrDefault<std::string>("policy_head", "vanilla"));
     add("value_head", options.GetOrDefault<std::string>("value_head", "winner"));
     add("mlh", options.GetOrDefault<bool>("mlh", true) ? "true" : "false");

@@ -43,6 +43,11 @@ def short_name(n):
     if m:
         nums = re.findall(r"L[ib](\d+)E", n.split("NS_")[0].split("DF16")[0])
         tail = " e4m3" if "GemmF8" in n else " bf16" if "DF16b" in n else ""
+        if m.group(1) == "gemm_dma_kernel" and "ArgsE" in n:
+            # template arguments behind the argument struct: output type, kind of output stores, epilogue, stages
+            rest = re.findall(r"L[ib](\d+)E", n.split("ArgsE", 1)[1])
+            if rest:
+                tail += ", " + {"0": "ordinary", "1": "streaming", "2": "written-through"}.get(rest[0], rest[0]) + " stores"
         return "%s<%s>%s" % (m.group(1), ",".join(nums), tail)
     return re.sub(r"E[PKv].*$", "", n)[:70]
 
@@ -103,16 +108,16 @@ def cmd_traffic(args):
         f = sum(fv) / len(fv) * scale["FETCH_SIZE"][1]
         w = sum(wv) / len(wv) * scale["WRITE_SIZE"][1]
         rows.append((len(fv) * (f + w), short_name(k), len(fv), f, w))
-    by = {}
     for _, n, cnt, f, w in sorted(rows, reverse=True)[:args.top]:
         print("| `%s` | %d | %.0f | %.0f |" % (n, cnt, f, w))
-        by[n] = (f + w) * 1024
     if args.json:
         def find(prefix):
-            for n, v in by.items():
-                if n.startswith(prefix) and "bf16" not in n and "e4m3" not in n:
-                    return int(v)
-            return None
+            # bytes per dispatch, averaged over the dispatches of every instance of the kernel (kinds of stores,
+            # stage counts): the same set of launches that bench.py times under this name
+            hits = [(cnt, (f + w) * 1024) for _, n, cnt, f, w in rows
+                    if n.startswith(prefix) and "bf16" not in n and "e4m3" not in n]
+            total = sum(c for c, _ in hits)
+            return int(sum(c * b for c, b in hits) / total) if total else None
         rec = {"workload": args.workload, "batch": args.batch, "sources_sha16": sources_sha16(),
                "source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py, KiB per dispatch x 1024, copy-kernel "
                          "factors %.3f / %.3f (python -m lc0_amd.profile_summary traffic)"

@@ -61,7 +61,10 @@ class Fp8BlasNetwork(BlasNetwork):
     """BlasNetwork whose body encoder layers run the fp8 configuration.
 
     scales: float array [layers][4] (x, attention output, x1, FFN hidden), value = code x scale.
-    gemms: which layers use e4m3 operands, subset of {"qkv", "dense", "ffn1", "ffn2", "smolgen"}.
+    gemms: which layers use e4m3 operands, subset of {"qkv", "dense", "ffn1", "ffn2", "smolgen", "smolgen_chain"}
+        ("smolgen": compression, both dense layers and the shared generator layer; "smolgen_chain": the first three,
+        with the generator on the half-precision output of the last row norm, as the backend computes it when the
+        generator runs inside its attention kernel).
     smolgen_scales: [layers][3], needed when "smolgen" is listed.
     perturb: None, "swap_x_x1" (the Q/K/V and FFN1 products are scaled back with each other's activation
       scale), "swap_x_att" (the same for Q/K/V and the attention-output layer) or "stale_layer" (every layer
@@ -95,7 +98,7 @@ class Fp8BlasNetwork(BlasNetwork):
                     q["ffn1"] = _QuantLinear(ffn.dense1_w, emb)
                 if "ffn2" in self.gemms:
                     q["ffn2"] = _QuantLinear(ffn.dense2_w, ffn.dense1_b.size)
-                if "smolgen" in self.gemms and mha.has_smolgen:
+                if ("smolgen" in self.gemms or "smolgen_chain" in self.gemms) and mha.has_smolgen:
                     sg = mha.smolgen
                     hc = sg.compress.size // emb
                     q["sg_compress"] = _QuantLinear(sg.compress, emb)
@@ -168,13 +171,14 @@ class Fp8BlasNetwork(BlasNetwork):
             xf = x
         self._note(li, 0, x)
         s_x = self._scale(li, 0) if qz else None
-        xq = quantize_activation(xf, self.scales[li][0]) if qz and ("qkv" in self.gemms or "smolgen" in self.gemms) else None
+        sg_q = "smolgen" in self.gemms or "smolgen_chain" in self.gemms
+        xq = quantize_activation(xf, self.scales[li][0]) if qz and ("qkv" in self.gemms or sg_q) else None
         qk_bias = None
         if mha.has_smolgen:
             sg = mha.smolgen
             hc = sg.compress.size // emb
             gen = sg.dense2_b.size
-            if qz and "smolgen" in self.gemms:
+            if qz and sg_q:
                 ss = self.smolgen_scales[li]
                 t = qw["sg_compress"](xq, s_x, None, nr.ACT_NONE)
                 tq = quantize_activation(t, ss[0]).reshape(bsz, 64 * hc)
@@ -184,8 +188,12 @@ class Fp8BlasNetwork(BlasNetwork):
                 tq = quantize_activation(t, ss[1])
                 t = self._h(qw["sg_dense2"](tq, ss[1], sg.dense2_b, smolgen_act))
                 t = layer_norm_skip(t, 1.0, None, sg.ln2_gammas, sg.ln2_betas, 1e-3)
-                tq = quantize_activation(t, ss[2]).reshape(bsz * heads, gen // heads)
-                qk_bias = self._h(qw["sg_global"](tq, ss[2], None, nr.ACT_NONE))
+                if "smolgen" in self.gemms:
+                    tq = quantize_activation(t, ss[2]).reshape(bsz * heads, gen // heads)
+                    qk_bias = self._h(qw["sg_global"](tq, ss[2], None, nr.ACT_NONE))
+                else:
+                    qk_bias = self._h(fc(self._h(t).reshape(bsz * heads, gen // heads), self.w.smolgen_w, None,
+                                         nr.ACT_NONE))
             else:
                 t = self._h(fc(x, sg.compress, None, nr.ACT_NONE))
                 self._note_sg(li, 0, t)

@@ -340,6 +340,45 @@ def test_gemm_f8_vs_exact_product(variant, m, n, k):
         K.set_gemm_variant(-1)
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("stores", ["cached", "stream", "write_through", "auto_keep"])
+def test_output_store_kinds_give_the_same_result(stores, variant):
+    """The 256-row tiles write a large output with ordinary, streaming or written-through stores, and the layer norm
+    reads and writes through: every kind must give the bits of the default (here: streaming by the size rule for
+    the GEMMs, ordinary loads and stores for the layer norm), which is held to the oracle on some rows. Variants:
+    the 256x256, 256x192 and 256x128 tiles."""
+    from lc0_amd import kernels as K
+    from oracle import fp8
+    kind = {"cached": K.STORES_CACHED, "stream": K.STORES_STREAM, "write_through": K.STORES_WRITE_THROUGH,
+            "auto_keep": K.STORES_AUTO_KEEP}[stores]
+    rng = np.random.default_rng(11)
+    m, n, k = 16384, 1024, 128                       # 32 MiB of half output from 16384 rows: the size rule's edge
+    a = _h(rng.standard_normal((m, k)) * 0.5)
+    w = _h(rng.standard_normal((n, k)) * 0.2)
+    b = rng.standard_normal(n).astype(f32)
+    a8 = fp8.e4m3_encode(rng.standard_normal((m, k)) * 2)
+    w8, wscale = fp8.quantize_rows(rng.standard_normal((n, k)) * 0.05)
+    x = _h(rng.standard_normal((4096, 1024)))
+    g, be = rng.standard_normal(1024).astype(f32), rng.standard_normal(1024).astype(f32)
+    K.set_gemm_variant(variant)
+    try:
+        want = K.gemm(a, w, b)
+        want8 = K.gemm_f8(a8, w8, f32(0.031) * wscale, b)
+        want_ln = K.layer_norm(x, x, g, be, 0.5, 1e-6)
+        K.set_out_stores(kind)
+        got = K.gemm(a, w, b)
+        got8 = K.gemm_f8(a8, w8, f32(0.031) * wscale, b)
+        got_ln = K.layer_norm(x, x, g, be, 0.5, 1e-6)
+    finally:
+        K.set_out_stores(K.STORES_AUTO)
+        K.set_gemm_variant(-1)
+    np.testing.assert_allclose(want.astype(f32)[-512:], onn.fc(a[-512:], w.reshape(-1), b, nr.ACT_NONE), rtol=2e-3,
+                               atol=2e-3)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got8, want8)
+    assert np.array_equal(got_ln, want_ln)
+
+
 def test_cold_cache_timing_hook_leaves_results_alone():
     """The profiling hook times launches one by one behind a cache-flushing copy: same output, a positive time."""
     from lc0_amd import kernels as K

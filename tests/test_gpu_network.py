@@ -239,6 +239,26 @@ def test_bt4_shape_batch_256(positions):
 
 
 @pytest.mark.timeout(600)
+def test_written_through_outputs_change_no_bits(positions):
+    """Where the big GEMMs and layer norms put their outputs (written through to the memory-side cache by default,
+    streamed past it with write_through=false) changes no value. 384 positions take the 256x128 tiles for some
+    GEMMs, whose written-through stores once lacked the wait states before their data registers are reused, and the
+    fp8 net writes e4m3 outputs the same way."""
+    rep = np.arange(384) % positions["masks"].shape[0]
+    masks, values = positions["masks"][rep], positions["values"][rep]
+    for name, opts, b in (("c2_bt4_15x1024", "", 256), ("c2_bt4_15x1024", "", 384),
+                          ("c2_bt4_15x1024", "precision=bf16", 384), ("c2_bt4_15x1024", "precision=fp8", 384)):
+        path = netgen.cached_config(name)
+        _, on = _run_gpu(path, masks[:b], values[:b], opts)
+        _, off = _run_gpu(path, masks[:b], values[:b], (opts + "," if opts else "") + "write_through=false")
+        for key in ("policy", "q", "d", "m"):
+            assert np.array_equal(on[key], off[key]), (name, opts, b, key)
+        # (rows 320.. repeat rows 0..: the same position gives the same output wherever it stands in the batch)
+        if b == 384:
+            np.testing.assert_allclose(on["policy"][320:], on["policy"][:64], rtol=0, atol=1e-5)
+
+
+@pytest.mark.timeout(600)
 def test_resnet_20x256_batch_512():
     """configs[3]: oracle comparison on 24 positions, then the full batch of 512
     through row-independence (same rows in a small and in the full batch)."""
@@ -393,13 +413,18 @@ def _legal_logit_rms(a, b, legal):
     return float(np.sqrt((err * err).mean()))
 
 
-def _emulation_of(path, net, gemms=None, **kw):
-    """oracle/fp8_net.py with the activation scales the backend is using (and, unless told, with the smolgen chain in
-    e4m3 exactly when the backend reports scales for it)."""
+FUSED_SMOLGEN_MIN_BATCH = 72   # default of the option fused_smolgen_min_batch
+
+
+def _emulation_of(path, net, gemms=None, batch=1, **kw):
+    """oracle/fp8_net.py with the activation scales the backend is using and, unless told, with the smolgen chain in
+    e4m3 exactly when the backend reports scales for it: all four of its layers, or, from the batch size on at which
+    the default fp8_gemms=auto runs the generator layer inside the attention kernel, the first three."""
     from oracle import fp8_net
     sc = net.Fp8Scales()
     if gemms is None:
-        gemms = ALL_FP8_GEMMS + (("smolgen",) if (sc[:, 4:] != 1.0).any() else ())
+        chain = "smolgen_chain" if batch >= FUSED_SMOLGEN_MIN_BATCH else "smolgen"
+        gemms = ALL_FP8_GEMMS + ((chain,) if (sc[:, 4:] != 1.0).any() else ())
     return fp8_net.Fp8BlasNetwork(nr.load(path), scales=sc[:, :4], smolgen_scales=sc[:, 4:], gemms=gemms, **kw)
 
 
@@ -433,7 +458,7 @@ def test_bt4_shape_fp8_batch_sweep(positions):
     s = _fp8_report(res, want, legal)
     assert s["kl_max"] <= 1e-4 and s["softmax_maxabs"] <= 1e-3
     assert s["q"] <= 1e-2 and s["d"] <= 1e-2 and s["mlh_rel"] <= 2e-2
-    emu = _emulation_of(path, net)
+    emu = _emulation_of(path, net, batch=len(masks))
     emu64 = emu.forward(masks, values)
     _check_fp8_against_emulation(res, emu64, want, legal, "64 positions")
     # A mis-wired activation scale is what such a comparison must notice: the emulation with the Q/K/V and FFN1
@@ -474,7 +499,7 @@ def test_bt4_shape_fp8_batch_sweep(positions):
         if n == 1024:
             rows = np.r_[0:8, 504:520, 1016:1024]
             want_rows = onn.BlasNetwork(nr.load(path)).forward(big_m[rows], big_v[rows])
-            emu_rows = emu.forward(big_m[rows], big_v[rows])
+            emu_rows = _emulation_of(path, net, batch=n).forward(big_m[rows], big_v[rows])
             _check_fp8_against_emulation({key: val[rows] for key, val in r.items()}, emu_rows, want_rows,
                                          [big_legal[i] for i in rows], "rows of three tiles at batch 1024")
     if s["top1"] < 0.99:
@@ -487,16 +512,20 @@ def test_bt4_shape_fp8_batch_sweep(positions):
                      % (s["top1"], s16["top1"], s["top1_decisive"]))
 
 
-@pytest.mark.parametrize("name,batch", [("tiny_attn_f8_sg", 40), ("c2_bt4_15x1024", 33)])
-def test_fp8_smolgen_chain_in_e4m3(name, batch, positions):
-    """fp8_gemms=...+smolgen (configs[4] lists the smolgen GEMMs among the e4m3 ones; the default where the chain's
-    widths allow it): compression, both dense layers and the shared generator run on e4m3 operands. Against the emulation of the same arithmetic and, by noise
-    level, against the fp32 oracle; the profile must show the chain's fp8 kernels."""
+@pytest.mark.parametrize("name,batch,explicit", [("tiny_attn_f8_sg", 40, True), ("c2_bt4_15x1024", 33, True),
+                                                 ("c2_bt4_15x1024", 80, True), ("c2_bt4_15x1024", 80, False)])
+def test_fp8_smolgen_chain_in_e4m3(name, batch, explicit, positions):
+    """fp8_gemms=...+smolgen (configs[4] lists the smolgen GEMMs among the e4m3 ones): compression, both dense layers
+    and the shared generator run on e4m3 operands, at every batch size. The default, fp8_gemms=auto, does the same
+    where the chain's widths allow it, except that from 72 positions on the generator layer runs inside the attention
+    kernel on half-precision operands (faster than an e4m3 GEMM of its own). Against the emulation of the same
+    arithmetic and, by noise level, against the fp32 oracle; the profile must show the kernels."""
     path = netgen.cached_config(name)
     masks, values, legal = positions["masks"][:batch], positions["values"][:batch], positions["legal"][:batch]
     want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
-    gemms = ALL_FP8_GEMMS + ("smolgen",)
-    net, res = _run_gpu(path, masks, values, "precision=fp8,fp8_gemms=" + "+".join(gemms))
+    gemms = ALL_FP8_GEMMS + ("smolgen" if explicit else "smolgen_chain",)
+    net, res = _run_gpu(path, masks, values,
+                        "precision=fp8" + (",fp8_gemms=" + "+".join(gemms) if explicit else ""))
     s = _fp8_report(res, want, legal)
     assert s["logit_rms"] <= 0.1 * s["logit_std"] and s["kl_max"] <= 1e-3 and s["top1_decisive"] >= 0.99
     sc = net.Fp8Scales()
@@ -509,8 +538,9 @@ def test_fp8_smolgen_chain_in_e4m3(name, batch, positions):
     comp.ComputeBlocking()
     names = [k.name for k in net.TakeProfile()]
     net.SetProfiling(False)
-    for layer in ("compress", "dense1", "dense2", "global"):
+    for layer in ("compress", "dense1", "dense2") + (("global",) if explicit else ()):
         assert any(n.startswith("gemm_smolgen_%s|gemm_f8" % layer) for n in names), (layer, names)
+    assert ("smolgen_attention" in names) == (not explicit), names
 
 
 def test_fp8_activation_scales_match_the_calibration_rule(positions):

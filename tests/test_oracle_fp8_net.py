@@ -84,3 +84,25 @@ def test_quantisation_noise_and_miswired_scales(positions):
         ref = fp8_net.Fp8BlasNetwork(net, scales=s2, smolgen_scales=sg_scales).forward(m, v)["policy"]
         bad = fp8_net.Fp8BlasNetwork(net, scales=s2, smolgen_scales=sg_scales, perturb=fault).forward(m, v)["policy"]
         assert rms(bad - ref) > 1.5 * noise, fault
+
+
+def test_generator_on_half_operands_is_the_chain_minus_one_quantisation(positions):
+    """gemms "smolgen_chain" (the generator layer on the half-precision output of the last row norm, the other three
+    smolgen layers on e4m3 operands) against "smolgen" (all four) and against no smolgen layer in e4m3: it differs from
+    both, by less than e4m3 noise, and it is the closer of the two to the fp32 oracle's attention bias path when only
+    the generator's quantisation is at stake (same scales, same everything else)."""
+    net = nr.load(netgen.cached_config("tiny_attn_f8_sg"))
+    m, v = positions["masks"], positions["values"]
+    big = ("qkv", "dense", "ffn1", "ffn2")
+    scales, sg_scales = fp8_net.Fp8BlasNetwork(net, gemms=big + ("smolgen",)).calibrate(m, v)
+    run = lambda gemms: fp8_net.Fp8BlasNetwork(net, scales=scales, smolgen_scales=sg_scales, gemms=gemms).forward(m, v)["policy"]
+    want = onn.BlasNetwork(net).forward(m, v)["policy"]
+    all4, chain3, none = run(big + ("smolgen",)), run(big + ("smolgen_chain",)), run(big)
+    rms = lambda a: float(np.sqrt(np.mean(a * a)))
+    noise = rms(all4 - want)
+    assert 0 < rms(chain3 - all4) < noise
+    assert 0 < rms(chain3 - none) < noise
+    # with nothing else quantised, taking the generator out of e4m3 can only bring the result closer to fp32
+    only4 = fp8_net.Fp8BlasNetwork(net, scales=scales, smolgen_scales=sg_scales, gemms=("smolgen",)).forward(m, v)["policy"]
+    only3 = fp8_net.Fp8BlasNetwork(net, scales=scales, smolgen_scales=sg_scales, gemms=("smolgen_chain",)).forward(m, v)["policy"]
+    assert rms(only3 - want) < rms(only4 - want)
