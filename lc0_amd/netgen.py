@@ -319,6 +319,9 @@ CONFIGS = {
     # smolgen inside the policy head's encoder layer as well (it shares the body's generator layer)
     "tiny_attn_polenc_sg": lambda: attention_body(64, 2, 2, 96, seed=2023, smolgen=(8, 32, 32), perturb_ln=True, std=0.1,
                                                   pol_encoder=(1, 2, 96, (8, 32, 32))),
+    # 24 heads of depth 32 at a width that is not a power of two (the shape family of the T78 / T82 nets), a few layers
+    "mid_attn_4x768": lambda: attention_body(768, 4, 24, 1024, seed=2024, smolgen=(32, 256, 256), perturb_ln=True,
+                                             std=0.03),
     "tiny_attn_nosmolgen": lambda: attention_body(64, 2, 2, 128, seed=2002, perturb_ln=True, std=0.1),
     # ---- what real files contain beyond FLOAT32 layers of the current format ----
     # batch-norm statistics on every convolution block, incl. the bias-less and gamma-less old forms

@@ -239,6 +239,28 @@ def test_bt4_shape_batch_256(positions):
 
 
 @pytest.mark.timeout(600)
+def test_24_heads_of_width_768_at_batch_256(positions):
+    """A body with 24 heads (the fused smolgen attention kernel's instance with missing head columns, whose head
+    pairs run one after the other) and GEMM widths that are multiples of 256 but not powers of two, at a batch large
+    enough for the 256-row tiles, the second stream and the written-through outputs: rows of the first, a middle and the
+    last tile against the oracle, and the same bits with the outputs streamed."""
+    path = netgen.cached_config("mid_attn_4x768")
+    masks, values = positions["masks"][:256], positions["values"][:256]
+    net, full = _run_gpu(path, masks, values)
+    rows = np.r_[0:8, 120:136, 248:256]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks[rows], values[rows])
+    _compare({k: v[rows] for k, v in full.items()}, want, [positions["legal"][i] for i in rows])
+    _, off = _run_gpu(path, masks, values, "write_through=false")
+    for key in ("policy", "q", "d", "m"):
+        assert np.array_equal(full[key], off[key]), key
+    # an odd batch: the last workgroup of the attention kernel has one sample only
+    comp = net.NewComputation()
+    comp.AddInputs(masks[:255], values[:255])
+    comp.ComputeBlocking()
+    np.testing.assert_allclose(comp.results()["policy"], full["policy"][:255], rtol=0, atol=5e-3)
+
+
+@pytest.mark.timeout(600)
 def test_written_through_outputs_change_no_bits(positions):
     """Where the big GEMMs and layer norms put their outputs (written through to the memory-side cache by default,
     streamed past it with write_through=false) changes no value. 384 positions take the 256x128 tiles for some
