@@ -1128,6 +1128,9 @@ GemmVariant PickGemmVariantHalf(const GemmArgs& a) {
   // A single 32-column panel (the smolgen compression): one workgroup per 64 rows, K split over its waves
   // (16384x32x1024: 9.5 us against 12.3 for the 64x64 tiles, but with twice the threads on every CU).
   if (a.latency_first && a.split_k == 1 && a.N <= 32 && a.K >= 512) return kRowPanel;
+  // Many products that each fit a 64x64 tile (the policy head's Q.K^T per position) would leave three quarters of
+  // every 128x128 tile empty (256 x 64x64x1024: 14.5 against 21.4 us).
+  if (a.M <= 64 && a.N <= 64) return kTile64;
   const long long big_tiles = tiles128;
   return big_tiles >= 192 ? kTile128 : kTile64;
 }

@@ -37,8 +37,10 @@ __global__ __launch_bounds__(256) void expand_planes_attn_kernel(const uint64_t*
   __syncthreads();
   T* o = out + (long long)b * 64 * ld;
   const int chunks = ld / V;
-  for (int i = threadIdx.x; i < 64 * chunks; i += 256) {
-    const int sq = i / chunks, c0 = (i - sq * chunks) * V;
+  // (a workgroup per 16 squares of a position: one per position left most CUs idle at up to a few hundred positions)
+  const int sq_begin = blockIdx.y * 16;
+  for (int i = threadIdx.x; i < 16 * chunks; i += 256) {
+    const int sq = sq_begin + i / chunks, c0 = (i % chunks) * V;
     T v[V];
 #pragma unroll
     for (int e = 0; e < V; e++) {
@@ -104,10 +106,10 @@ void LaunchExpandPlanesAttn(const uint64_t* masks, const float* values, const T*
                             int batch, hipStream_t stream) {
   if (batch <= 0) return;
   if (ld % 8 == 0) {
-    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 8>), dim3(batch), dim3(256), 0, stream, masks, values, pos_enc, 64,
+    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 8>), dim3(batch, 4), dim3(256), 0, stream, masks, values, pos_enc, 64,
                        0LL, out, ld);
   } else {
-    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 1>), dim3(batch), dim3(256), 0, stream, masks, values, pos_enc, 64,
+    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 1>), dim3(batch, 4), dim3(256), 0, stream, masks, values, pos_enc, 64,
                        0LL, out, ld);
   }
 }
@@ -117,10 +119,10 @@ void LaunchExpandPlanesDense(const uint64_t* masks, const float* values, const T
                              int batch, hipStream_t stream) {
   if (batch <= 0) return;
   if (ld % 8 == 0) {
-    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 8>), dim3(batch), dim3(256), 0, stream, masks, values, extra,
+    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 8>), dim3(batch, 4), dim3(256), 0, stream, masks, values, extra,
                        n_extra, 64LL * n_extra, out, ld);
   } else {
-    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 1>), dim3(batch), dim3(256), 0, stream, masks, values, extra,
+    hipLaunchKernelGGL((expand_planes_attn_kernel<T, 1>), dim3(batch, 4), dim3(256), 0, stream, masks, values, extra,
                        n_extra, 64LL * n_extra, out, ld);
   }
 }
