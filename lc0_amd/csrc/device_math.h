@@ -26,7 +26,13 @@ static __device__ __forceinline__ float Activate(float v, int act) {
     case 2: return v > 0.0f ? v : 0.0f;
     case 4: return tanhf(v);
     case 5: return ActSigmoid(v);
-    case 6: return v > 0.0f ? 1.05070098f * v : 1.05070098f * 1.67326324f * (__expf(v) - 1.0f);
+    case 6: {
+      // Both sides computed for every lane and one select: with the exponential on one side only of a conditional
+      // expression this became a branch per element (16384x1536x1024 product: 77 -> 73 us; 59 without activation).
+      const bool pos = v > 0.0f;
+      const float neg = 1.05070098f * 1.67326324f * (__expf(pos ? 0.0f : v) - 1.0f);
+      return pos ? 1.05070098f * v : neg;
+    }
     case 7: return v * ActSigmoid(v);
     case 8: return v > 0.0f ? v * v : 0.0f;
     default: return v;
