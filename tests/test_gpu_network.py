@@ -93,6 +93,45 @@ def test_attention_nets_match_oracle(name, batch, positions):
     np.testing.assert_allclose(comp.GetDVal(0) + 0 * comp.GetMVal(0), res["d"][3], atol=2e-3)
 
 
+def _random_attention_shape(seed):
+    """A seeded draw from the family of attention-body nets the backend takes: every layer width a multiple of 8,
+    head depth anything from 8 to 128 (the tuned attention kernels take 32, 64 and 128), embedding width equal to or
+    different from heads x depth, with and without smolgen, the dense position encoding, input gating and the
+    multi-head file format."""
+    rng = np.random.default_rng(seed)
+    depth = int(rng.choice([8, 16, 24, 32, 40, 64, 128]))
+    heads = int(rng.choice([1, 2, 3, 4, 6]))
+    d_model = heads * depth
+    emb = d_model if rng.random() < 0.5 else 8 * int(rng.integers(4, 33))
+    smolgen = None if rng.random() < 0.3 else (int(rng.choice([8, 16, 32])), 8 * int(rng.integers(2, 17)),
+                                                 heads * 8 * int(rng.integers(1, 5)))
+    pe_dense = None if rng.random() < 0.5 else (int(rng.choice([8, 16])), 8 * int(rng.integers(4, 17)))
+    return dict(emb=emb, layers=int(rng.integers(1, 4)), heads=heads, dff=8 * int(rng.integers(4, 49)), seed=5000 + seed,
+                smolgen=smolgen, std=0.08, perturb_ln=True, pe_dense=pe_dense,
+                gating=bool(rng.random() < 0.3) and pe_dense is not None,
+                multihead=bool(rng.random() < 0.3) and pe_dense is not None, d_model=d_model,
+                policy_d=8 * int(rng.integers(2, 17)), value_channels=int(rng.choice([8, 16, 32])),
+                value_fc=8 * int(rng.integers(2, 17)), mlh_channels=int(rng.choice([8, 16])),
+                mlh_fc=8 * int(rng.integers(1, 9)))
+
+
+@pytest.mark.parametrize("seed", list(range(100, 116)))
+def test_random_attention_body_shapes_match_oracle(seed, positions, tmp_path):
+    """Sixteen seeded random architectures and batch sizes (1 to 80): the shapes nobody tuned for go through the
+    same comparison as the named configurations. (Eighty such draws were run once with no difference beyond two
+    near-tie best moves in one net.)"""
+    from lc0_amd import netproto
+    kw = _random_attention_shape(seed)
+    batch = int(np.random.default_rng(seed + 99).integers(1, 81))
+    print("shape:", {k: v for k, v in kw.items() if k not in ("seed", "std", "perturb_ln")}, "batch", batch)
+    path = str(tmp_path / "net.pb.gz")
+    netproto.write_pb_gz(path, netgen.attention_body(**kw))
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    _, res = _run_gpu(path, masks, values)
+    _compare(res, want, positions["legal"][:batch])
+
+
 @pytest.mark.parametrize("name,batch,options", [("tiny_attn", 37, ""), ("c2_bt4_15x1024", 33, ""),
                                                 ("tiny_attn_f8", 21, "precision=fp8,")])
 def test_smolgen_generator_inside_attention_and_as_a_gemm_of_its_own(name, batch, options, positions):
