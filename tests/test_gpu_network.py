@@ -35,7 +35,7 @@ def _run_gpu(path, masks, values, options=""):
     return net, res
 
 
-def _compare(res, want, legal, tol=TOL, logit_frac=None):
+def _compare(res, want, legal, tol=TOL, logit_frac=None, tie_flips=1):
     pol_g, pol_o = res["policy"], want["policy"]
     sm_g, sm_o = onn.softmax_rows(pol_g), onn.softmax_rows(pol_o)
     stats = dict(policy_softmax=np.abs(sm_g - sm_o).max(),
@@ -69,7 +69,7 @@ def _compare(res, want, legal, tol=TOL, logit_frac=None):
     # Best legal move: the same as the oracle's on at least 99 % of the positions, and where it differs the two
     # moves are a tie within the logit bound (the only flip that arithmetic within that bound can cause).
     assert all(gap <= 2 * logit_tol for gap in flips), flips
-    assert stats["top1_agreement"] >= 0.99 or len(flips) <= 1, stats["top1_agreement"]
+    assert stats["top1_agreement"] >= 0.99 or len(flips) <= tie_flips, stats["top1_agreement"]
     return stats
 
 
@@ -130,6 +130,49 @@ def test_random_attention_body_shapes_match_oracle(seed, positions, tmp_path):
     want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
     _, res = _run_gpu(path, masks, values)
     _compare(res, want, positions["legal"][:batch])
+
+
+def _random_tower_shape(seed):
+    """A seeded draw from the residual towers the backend takes: filters and head widths multiples of 8, with or
+    without squeeze-and-excitation, classical, convolutional or attention policy head, with or without moves left."""
+    rng = np.random.default_rng(seed)
+    kind = int(rng.integers(0, 3))   # 0 classical policy, 1 convolutional policy, 2 attention policy
+    kw = dict(filters=8 * int(rng.integers(2, 25)), blocks=int(rng.integers(1, 5)),
+              se_channels=int(rng.choice([0, 8, 16, 32])), seed=6000 + seed,
+              policy_channels=int(rng.choice([8, 16, 32, 80])), value_channels=int(rng.choice([8, 16, 32])),
+              value_fc=8 * int(rng.integers(2, 17)), moves_left=bool(rng.random() < 0.5), conv_policy=kind == 1,
+              attn_policy=(8 * int(rng.integers(2, 13)), 8 * int(rng.integers(2, 13)), int(rng.integers(0, 3)),
+                           int(rng.choice([1, 2, 4])), 8 * int(rng.integers(2, 17))) if kind == 2 else None)
+    if kw["attn_policy"] is not None:   # encoder layers keep the embedding width; heads must divide it
+        e, d, layers, h, f = kw["attn_policy"]
+        kw["attn_policy"] = (e, e if layers else d, layers, h if e % h == 0 else 1, f)
+    return kw
+
+
+@pytest.mark.parametrize("seed", list(range(0, 18)))
+def test_random_residual_tower_shapes_match_oracle(seed, positions, tmp_path):
+    """Eighteen seeded random towers and batch sizes, every third one in fp32 (bound 1e-3), the others in fp16.
+    (Sixty such draws were run once: the classical and convolutional policy heads stayed inside the bounds of the
+    named configurations; with the attention policy head on an fp16 tower the raw logits differ by up to a tenth of
+    their spread - fp16 F(4x4) winograd activations under 1/fan_in weights, 2e-5 in fp32 on the same nets - while
+    the softmaxed policy stays within 1.5e-3, so those get a wider logit bound.)"""
+    from lc0_amd import netproto
+    kw = _random_tower_shape(seed)
+    batch = int(np.random.default_rng(seed + 99).integers(1, 81))
+    fp32 = seed % 3 == 0
+    print("shape:", {k: v for k, v in kw.items() if k != "seed"}, "batch", batch, "fp32" if fp32 else "fp16")
+    path = str(tmp_path / "net.pb.gz")
+    netproto.write_pb_gz(path, netgen.se_resnet(**kw))
+    masks, values = positions["masks"][:batch], positions["values"][:batch]
+    want = onn.BlasNetwork(nr.load(path)).forward(masks, values)
+    _, res = _run_gpu(path, masks, values, "precision=fp32" if fp32 else "")
+    if fp32:
+        _compare(res, want, positions["legal"][:batch], tol=1e-3)
+    else:
+        # (random 1/fan_in weights give near-uniform policies with exact near-ties: up to three such flips pass, each
+        #  still held to a gap of twice the logit bound)
+        _compare(res, want, positions["legal"][:batch], logit_frac=0.12 if kw["attn_policy"] is not None else None,
+                 tie_flips=3)
 
 
 @pytest.mark.parametrize("name,batch,options", [("tiny_attn", 37, ""), ("c2_bt4_15x1024", 33, ""),
