@@ -9,6 +9,7 @@
 #include "kernel_common.h"
 
 #include <algorithm>
+#include <cmath>
 #include <stdexcept>
 #include <type_traits>
 #include <utility>
@@ -1071,6 +1072,34 @@ GemmVariant PickGemmVariantHalf(const GemmArgs& a) {
     // output element and round (ns per element at K = 1024): 0.60 for 256x256, 0.61 for 256x192;
     // the two small shapes run two workgroups per CU, 0.68 (256x128) and 0.75 (128x128) per element
     // while sharing a CU, 0.84 and 0.95 when a single round leaves every workgroup alone on its CU.
+    // One product of at least 4096 rows with K and N of at least 512 (the encoder layers of the attention bodies
+    // from 64 positions up): a cost model in microseconds fitted to launches of all five shapes on 92 problems
+    // (M 4096 to 65536, N 512 to 3072, K 512 to 2048; the variant it picks is 0.6 % behind the fastest measured one
+    // on average and 9 % at worst, against 3 % and 24 % for the per-element model below, which was set when the
+    // large tiles were slower than they are now). A round of the one-workgroup-per-CU shapes costs a fixed part and
+    // a part per k-tile of 64; a last round that fills only a fraction f of the CUs costs 0.55 + 0.45 f of a full
+    // one (its workgroups find L2 and the memory system less contended); the shapes that share a CU are priced by
+    // tile count.
+    if (a.batch == 1 && a.M >= 4096 && a.K >= 512 && a.N >= 512) {
+      const double kt = a.K / 64.0;
+      auto tiles = [&](int bm, int bn) { return (double)((a.M + bm - 1) / bm) * (double)((a.N + bn - 1) / bn); };
+      auto rounds_of = [](double x) {
+        const double whole = std::floor(x + 1e-9), frac = x - whole;
+        return whole + (frac > 1e-9 ? 0.55 + 0.45 * frac : 0.0);
+      };
+      const double t256 = 1.6 + rounds_of(tiles(256, 256) / 256.0) * (6.93 + 1.814 * kt);
+      const double t192 = 1.6 + rounds_of(tiles(256, 192) / 256.0) * (5.37 + 1.444 * kt);
+      const double t128 = 1.08 * (1.6 + rounds_of(tiles(256, 128) / 256.0) * (2.53 + 1.215 * kt));
+      const double ts = 2.62 + std::max(0.5, tiles(128, 128) / 512.0) * (3.62 + 1.140 * kt);
+      const double t64 = 1.19 + std::max(0.34, tiles(128, 64) / 768.0) * (2.75 + 1.119 * kt);
+      GemmVariant best = kDma256x256;
+      double cost = t256;
+      if (t192 < cost && a.skip == nullptr) { best = kDma256x192; cost = t192; }
+      if (t128 < cost) { best = kDma256x128; cost = t128; }
+      if (ts < cost) { best = kDma128x128; cost = ts; }
+      if (t64 < cost) { best = kDma128x64; cost = t64; }
+      return best;
+    }
     auto rounds = [&](int bm, int bn) {
       const long long tiles = (long long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * a.batch;
       return (double)((tiles + 255) / 256);
