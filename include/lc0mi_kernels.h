@@ -21,6 +21,10 @@ extern "C" {
 int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* W, int ldw, long long strideW,
                  const float* bias, int M, int N, int K, int batch, float scale, int act, int out_f32, void* C,
                  int ldc, long long strideC, int time_iters, double* ms);
+/* Name of the tile shape lc0mi_k_gemm runs a half-precision product of this shape on ("gemm_dma_256x256x64", ...):
+ * the launcher's host-side choice, which needs no device. No counterpart in the reference, whose products go to a
+ * BLAS library (src/neural/backends/blas/fully_connected_layer.cc:90-101). */
+const char* lc0mi_k_gemm_variant_name(int M, int N, int K, int batch, int latency_first);
 /* Split-K form: K is cut into split_k slices whose float partial sums are added in
  * slice order (bias added once, no activation). C is float [M][N]. */
 int lc0mi_k_gemm_splitk(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,

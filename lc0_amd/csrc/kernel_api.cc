@@ -162,6 +162,14 @@ int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* 
   });
 }
 
+const char* lc0mi_k_gemm_variant_name(int M, int N, int K, int batch, int latency_first) {
+  lc0mi::GemmArgs g;
+  g.M = M; g.N = N; g.K = K; g.batch = batch < 1 ? 1 : batch;
+  g.lda = K; g.ldw = K; g.ldc = N;
+  g.latency_first = latency_first != 0;
+  return lc0mi::GemmVariantName(g);
+}
+
 int lc0mi_k_gemm_norm_producer(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,
                                int K, float scale, const uint16_t* skip, const float* skip_stats, int skip_parts,
                                const float* skip_gamma, const float* skip_beta, float eps, uint16_t* U,

@@ -18,6 +18,8 @@ def _lib():
         vp, ci, ll, cf, cd = C.c_void_p, C.c_int, C.c_longlong, C.c_float, C.POINTER(C.c_double)
         lib.lc0mi_k_gemm.argtypes = [vp, ci, ll, vp, ci, ll, vp, ci, ci, ci, ci, cf, ci, ci, vp, ci, ll, ci, cd]
         lib.lc0mi_k_gemm_splitk.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, ci, cf, vp, ci]
+        lib.lc0mi_k_gemm_variant_name.argtypes = [ci, ci, ci, ci, ci]
+        lib.lc0mi_k_gemm_variant_name.restype = C.c_char_p
         lib.lc0mi_k_gemm_norm_producer.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, vp, vp, ci, vp, vp, cf, vp, vp, ci,
                                                    C.POINTER(C.c_int), ci, cd]
         lib.lc0mi_k_gemm_norm_consumer.argtypes = [vp, ci, vp, ci, vp, vp, ci, ci, ci, vp, ci, cf, ci, ci, vp, ci, ci, cd]
@@ -109,6 +111,11 @@ def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
                                int(out_f32), _ptr(out), n, m * n, time_iters, C.byref(ms)))
     out = _ret16(out if batched else out[0])
     return (out, ms.value) if time_iters else out
+
+
+def gemm_variant_name(m, n, k, batch=1, latency_first=False):
+    """Tile shape the launcher picks for a half-precision product of this shape (host-side logic, no GPU needed)."""
+    return _lib().lc0mi_k_gemm_variant_name(m, n, k, batch, int(latency_first)).decode()
 
 
 STORES_AUTO, STORES_AUTO_KEEP, STORES_CACHED, STORES_STREAM, STORES_WRITE_THROUGH = range(5)
