@@ -548,6 +548,33 @@ def _check_fp8_against_emulation(res, emu_out, oracle_out, legal, what):
     return diff, noise, float(top_e), float(top_o)
 
 
+@pytest.mark.timeout(600)
+def test_bt4_shape_fp16_batch_sweep(positions):
+    """The BT4-shape net in fp16 at batch sizes between the tuned ones (other GEMM tile shapes, partial rounds, the
+    smolgen generator inside and outside the attention kernel, one and two streams): 24 rows spread over the batch
+    - from the first, a middle and the last 256-row tile - against the fp32 oracle at every size, with the bounds of
+    the named configurations."""
+    path = netgen.cached_config("c2_bt4_15x1024")
+    oracle = onn.BlasNetwork(nr.load(path))
+    from lc0_amd import Network
+    net = Network(path, "")
+    for n in (1, 7, 48, 71, 72, 96, 112, 160, 192, 320, 384, 640, 1024):
+        reps = -(-n // 320)
+        big_m = np.tile(positions["masks"], (reps, 1))[:n]
+        big_v = np.tile(positions["values"], (reps, 1))[:n]
+        big_legal = (positions["legal"] * reps)[:n]
+        comp = net.NewComputation()
+        comp.AddInputs(big_m, big_v)
+        comp.ComputeBlocking()
+        r = comp.results()
+        comp.close()
+        assert np.isfinite(r["policy"]).all()
+        rows = np.unique(np.r_[0:min(n, 8), max(0, n // 2 - 4):min(n, n // 2 + 4), max(0, n - 8):n])
+        want = oracle.forward(big_m[rows], big_v[rows])
+        print("batch", n, "rows", rows.tolist())
+        _compare({key: val[rows] for key, val in r.items()}, want, [big_legal[i] for i in rows])
+
+
 @pytest.mark.timeout(900)
 def test_bt4_shape_fp8_batch_sweep(positions):
     """configs[4]: the BT4-shape net with e4m3 GEMM operands. 64 positions against the fp32 oracle (KL, W/D/L, top-1)
