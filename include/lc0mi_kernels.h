@@ -25,6 +25,9 @@ int lc0mi_k_gemm(const uint16_t* A, int lda, long long strideA, const uint16_t* 
  * the launcher's host-side choice, which needs no device. No counterpart in the reference, whose products go to a
  * BLAS library (src/neural/backends/blas/fully_connected_layer.cc:90-101). */
 const char* lc0mi_k_gemm_variant_name(int M, int N, int K, int batch, int latency_first);
+/* Rows that lc0mi_k_gemm gives to a first launch of whole rounds of large tiles when it cuts a half-precision product
+ * of this shape along its rows (0: one launch). Host-side choice, no device needed; no counterpart in the reference. */
+int lc0mi_k_gemm_row_split(int M, int N, int K);
 /* Split-K form: K is cut into split_k slices whose float partial sums are added in
  * slice order (bias added once, no activation). C is float [M][N]. */
 int lc0mi_k_gemm_splitk(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,

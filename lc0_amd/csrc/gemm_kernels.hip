@@ -867,6 +867,11 @@ inline int OutputStores(int requested, long long m, long long n, long long batch
   if (!StreamOutput(m, n, batch, elem_bytes)) return 0;
   return requested == kStoresAutoKeep ? 2 : 1;
 }
+// The same as a value of GemmArgs::out_stores that no longer depends on the size (for the parts of a product).
+inline int ResolvedOutStores(const GemmArgs& a) {
+  const int s = OutputStores(a.out_stores, a.M, a.N, a.batch, 2);
+  return s == 1 ? kStoresStream : s == 2 ? kStoresWriteThrough : kStoresCached;
+}
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int NSTAGES = 2>
 void LaunchGemmDma(const GemmArgs& a, hipStream_t stream) {
@@ -1049,6 +1054,56 @@ int g_variant_override = -1;
 
 GemmVariant PickGemmVariantHalf(const GemmArgs& a);
 
+// Fitted cost model of the five direct-to-LDS tile shapes, in microseconds per launch (see PickGemmVariantHalf).
+struct FittedCosts {
+  double t256, t192, t128, ts, t64;
+  double Best() const { return std::min(std::min(std::min(t256, t192), std::min(t128, ts)), t64); }
+};
+inline bool InFittedDomain(const GemmArgs& a) { return a.batch == 1 && a.M >= 4096 && a.K >= 512 && a.N >= 512; }
+inline FittedCosts FitCosts(int M, int N, int K) {
+  const double kt = K / 64.0;
+  auto tiles = [&](int bm, int bn) { return (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn); };
+  auto rounds_of = [](double x) {
+    const double whole = std::floor(x + 1e-9), frac = x - whole;
+    return whole + (frac > 1e-9 ? 0.55 + 0.45 * frac : 0.0);
+  };
+  FittedCosts c;
+  c.t256 = 1.6 + rounds_of(tiles(256, 256) / 256.0) * (6.93 + 1.814 * kt);
+  c.t192 = 1.6 + rounds_of(tiles(256, 192) / 256.0) * (5.37 + 1.444 * kt);
+  c.t128 = 1.08 * (1.6 + rounds_of(tiles(256, 128) / 256.0) * (2.53 + 1.215 * kt));
+  c.ts = 2.62 + std::max(0.5, tiles(128, 128) / 512.0) * (3.62 + 1.140 * kt);
+  c.t64 = 1.19 + std::max(0.34, tiles(128, 64) / 768.0) * (2.75 + 1.119 * kt);
+  return c;
+}
+
+// A large product whose tiles do not fill whole rounds of the 256 CUs, cut along its rows: the rows that make whole
+// rounds of 256x256 (or 256x192) tiles go to one launch and the rest to a second launch on whatever shape suits it
+// (20480x1024x1536: 87 us on 320 tiles of 256x256, one and a quarter rounds, or 78 us on 128x128 tiles, against
+// 49 + 19 us for 16384 rows on one full round of large tiles and 4096 rows on small ones). Returns the rows of the
+// first launch (0: one launch) when the model above prices the pair at least 3 % below the best single shape.
+int PlanRowSplit(const GemmArgs& a, GemmVariant* first) {
+  if (g_variant_override >= 0 || !InFittedDomain(a) || a.out_f32 || a.split_k != 1 || a.K % 64 != 0 ||
+      a.skip != nullptr || a.row_stats != nullptr) {
+    return 0;
+  }
+  double best = FitCosts(a.M, a.N, a.K).Best() * 0.97;
+  int best_m1 = 0;
+  for (int v = 0; v < 2; v++) {
+    const int bn = v == 0 ? 256 : 192;
+    const int col_tiles = (a.N + bn - 1) / bn;
+    if (col_tiles > 256) continue;
+    const int rows_per_round = (256 / col_tiles) * 256;
+    // (the rest stays inside the range of sizes the model was fitted on: cut at 2048 rows, a 15x1024 pass at 96
+    //  positions lost 4 %)
+    for (int m1 = rows_per_round; m1 + 4096 <= a.M; m1 += rows_per_round) {
+      const FittedCosts top = FitCosts(m1, a.N, a.K);
+      const double c = (v == 0 ? top.t256 : top.t192) + FitCosts(a.M - m1, a.N, a.K).Best() + 1.0;
+      if (c < best) { best = c; best_m1 = m1; *first = v == 0 ? kDma256x256 : kDma256x192; }
+    }
+  }
+  return best_m1;
+}
+
 // bfloat16 operands run every variant except the row panels (kept out to bound the number of kernel instances):
 // such shapes take the register-staged 64x64 tiles.
 GemmVariant PickGemmVariant(const GemmArgs& a) {
@@ -1080,24 +1135,14 @@ GemmVariant PickGemmVariantHalf(const GemmArgs& a) {
     // a part per k-tile of 64; a last round that fills only a fraction f of the CUs costs 0.55 + 0.45 f of a full
     // one (its workgroups find L2 and the memory system less contended); the shapes that share a CU are priced by
     // tile count.
-    if (a.batch == 1 && a.M >= 4096 && a.K >= 512 && a.N >= 512) {
-      const double kt = a.K / 64.0;
-      auto tiles = [&](int bm, int bn) { return (double)((a.M + bm - 1) / bm) * (double)((a.N + bn - 1) / bn); };
-      auto rounds_of = [](double x) {
-        const double whole = std::floor(x + 1e-9), frac = x - whole;
-        return whole + (frac > 1e-9 ? 0.55 + 0.45 * frac : 0.0);
-      };
-      const double t256 = 1.6 + rounds_of(tiles(256, 256) / 256.0) * (6.93 + 1.814 * kt);
-      const double t192 = 1.6 + rounds_of(tiles(256, 192) / 256.0) * (5.37 + 1.444 * kt);
-      const double t128 = 1.08 * (1.6 + rounds_of(tiles(256, 128) / 256.0) * (2.53 + 1.215 * kt));
-      const double ts = 2.62 + std::max(0.5, tiles(128, 128) / 512.0) * (3.62 + 1.140 * kt);
-      const double t64 = 1.19 + std::max(0.34, tiles(128, 64) / 768.0) * (2.75 + 1.119 * kt);
+    if (InFittedDomain(a)) {
+      const FittedCosts c = FitCosts(a.M, a.N, a.K);
       GemmVariant best = kDma256x256;
-      double cost = t256;
-      if (t192 < cost && a.skip == nullptr) { best = kDma256x192; cost = t192; }
-      if (t128 < cost) { best = kDma256x128; cost = t128; }
-      if (ts < cost) { best = kDma128x128; cost = ts; }
-      if (t64 < cost) { best = kDma128x64; cost = t64; }
+      double cost = c.t256;
+      if (c.t192 < cost && a.skip == nullptr) { best = kDma256x192; cost = c.t192; }
+      if (c.t128 < cost) { best = kDma256x128; cost = c.t128; }
+      if (c.ts < cost) { best = kDma128x128; cost = c.ts; }
+      if (c.t64 < cost) { best = kDma128x64; cost = c.t64; }
       return best;
     }
     auto rounds = [&](int bm, int bn) {
@@ -1200,7 +1245,14 @@ int GemmStatsParts(const GemmArgs& a) {
   return bn == 0 ? 0 : (a.N + bn - 1) / bn;
 }
 
+int GemmRowSplit(const GemmArgs& a) {
+  GemmVariant first = kDma256x256;
+  return PlanRowSplit(a, &first);
+}
+
 const char* GemmVariantName(const GemmArgs& a) {
+  GemmVariant first = kDma256x256;
+  if (PlanRowSplit(a, &first) > 0) return first == kDma256x256 ? "gemm_dma_256x256x64+rest" : "gemm_dma_256x192x64+rest";
   switch (PickGemmVariant(a)) {
     case kDma256x256: return "gemm_dma_256x256x64";
     case kDma256x192: return "gemm_dma_256x192x64";
@@ -1215,11 +1267,8 @@ const char* GemmVariantName(const GemmArgs& a) {
   }
 }
 
-void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
-  if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
-  if ((a.skip != nullptr || a.row_stats != nullptr) && !GemmSupportsNormFolding(a)) {
-    throw std::runtime_error("LaunchGemm: no kernel variant with the folded layer-norm epilogue for this shape");
-  }
+namespace {
+void LaunchGemmOne(const GemmArgs& a, hipStream_t stream) {
   switch (PickGemmVariant(a)) {
     case kDma256x256: LaunchGemmDma<256, 256, 64, 2, 4>(a, stream); break;
     case kDma256x192: LaunchGemmDma<256, 192, 64, 4, 2>(a, stream); break;
@@ -1232,6 +1281,29 @@ void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
     case kTile128: LaunchGemmTile<128, 128, 64, 2, 2>(a, stream); break;
     default: LaunchGemmTile<64, 64, 64, 2, 2>(a, stream); break;
   }
+}
+}  // namespace
+
+void LaunchGemm(const GemmArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return;
+  if ((a.skip != nullptr || a.row_stats != nullptr) && !GemmSupportsNormFolding(a)) {
+    throw std::runtime_error("LaunchGemm: no kernel variant with the folded layer-norm epilogue for this shape");
+  }
+  GemmVariant first = kDma256x256;
+  const int m1 = PlanRowSplit(a, &first);
+  if (m1 > 0) {
+    GemmArgs top = a, rest = a;
+    top.out_stores = rest.out_stores = ResolvedOutStores(a);   // as for the whole product
+    top.M = m1;
+    rest.M = a.M - m1;
+    rest.A = a.A + static_cast<long long>(m1) * a.lda;
+    rest.C = static_cast<half_t*>(a.C) + static_cast<long long>(m1) * a.ldc;
+    if (first == kDma256x256) LaunchGemmDma<256, 256, 64, 2, 4>(top, stream);
+    else LaunchGemmDma<256, 192, 64, 4, 2>(top, stream);
+    LaunchGemmOne(rest, stream);   // (the rest is below one round of the large tiles: one launch)
+    return;
+  }
+  LaunchGemmOne(a, stream);
 }
 
 namespace {

@@ -170,6 +170,13 @@ const char* lc0mi_k_gemm_variant_name(int M, int N, int K, int batch, int latenc
   return lc0mi::GemmVariantName(g);
 }
 
+int lc0mi_k_gemm_row_split(int M, int N, int K) {
+  lc0mi::GemmArgs g;
+  g.M = M; g.N = N; g.K = K; g.batch = 1;
+  g.lda = K; g.ldw = K; g.ldc = N;
+  return lc0mi::GemmRowSplit(g);
+}
+
 int lc0mi_k_gemm_norm_producer(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,
                                int K, float scale, const uint16_t* skip, const float* skip_stats, int skip_parts,
                                const float* skip_gamma, const float* skip_beta, float eps, uint16_t* U,

@@ -84,8 +84,10 @@ void LaunchGemm(const GemmArgs& args, hipStream_t stream);
 // epilogue), and the number of partial sums per row a producer launch writes to stats_out.
 bool GemmSupportsNormFolding(const GemmArgs& args);
 int GemmStatsParts(const GemmArgs& args);
-// Name of the kernel variant LaunchGemm picks for these arguments (tile shape).
+// Name of the kernel variant LaunchGemm picks for these arguments (tile shape; "...+rest" when it cuts the product
+// along its rows into whole rounds of large tiles and a rest, GemmRowSplit() rows in the first launch).
 const char* GemmVariantName(const GemmArgs& args);
+int GemmRowSplit(const GemmArgs& args);
 
 // e4m3 (OCP fp8, "fn": max 448, no infinities) GEMM with fp32 accumulation:
 //   C[m][n] = act(col_scale[n] * sum_k A[m][k] * W[n][k] + bias[n])

@@ -20,6 +20,7 @@ def _lib():
         lib.lc0mi_k_gemm_splitk.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, ci, cf, vp, ci]
         lib.lc0mi_k_gemm_variant_name.argtypes = [ci, ci, ci, ci, ci]
         lib.lc0mi_k_gemm_variant_name.restype = C.c_char_p
+        lib.lc0mi_k_gemm_row_split.argtypes = [ci, ci, ci]
         lib.lc0mi_k_gemm_norm_producer.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, vp, vp, ci, vp, vp, cf, vp, vp, ci,
                                                    C.POINTER(C.c_int), ci, cd]
         lib.lc0mi_k_gemm_norm_consumer.argtypes = [vp, ci, vp, ci, vp, vp, ci, ci, ci, vp, ci, cf, ci, ci, vp, ci, ci, cd]
@@ -116,6 +117,11 @@ def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
 def gemm_variant_name(m, n, k, batch=1, latency_first=False):
     """Tile shape the launcher picks for a half-precision product of this shape (host-side logic, no GPU needed)."""
     return _lib().lc0mi_k_gemm_variant_name(m, n, k, batch, int(latency_first)).decode()
+
+
+def gemm_row_split(m, n, k):
+    """Rows of the first launch when the launcher cuts a product of this shape along its rows (0: one launch)."""
+    return _lib().lc0mi_k_gemm_row_split(m, n, k)
 
 
 STORES_AUTO, STORES_AUTO_KEEP, STORES_CACHED, STORES_STREAM, STORES_WRITE_THROUGH = range(5)

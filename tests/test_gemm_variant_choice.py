@@ -17,15 +17,31 @@ def _table():
     return [(int(r[0]), int(r[1]), int(r[2]), [float(t) for t in r[3:8]]) for r in rows]
 
 
+def _time_of_choice(m, n, k, table):
+    """Measured time of what the launcher does for this problem; None for a product cut along its rows into parts
+    the table does not hold."""
+    name = K.gemm_variant_name(m, n, k)
+    if not name.endswith("+rest"):
+        return table[(m, n, k)][COLUMN[name]]
+    m1 = K.gemm_row_split(m, n, k)
+    assert 0 < m1 < m and m1 % 256 == 0, (m, n, k, m1)
+    if (m1, n, k) not in table or (m - m1, n, k) not in table:
+        return None
+    return table[(m1, n, k)][COLUMN[name[:-5]]] + _time_of_choice(m - m1, n, k, table)
+
+
 def test_chosen_tile_shape_is_close_to_the_fastest_measured_one():
-    regrets = []
-    for m, n, k, times in _table():
-        name = K.gemm_variant_name(m, n, k)
-        assert name in COLUMN, (m, n, k, name)
-        regrets.append(times[COLUMN[name]] / min(times) - 1.0)
+    table = {(m, n, k): times for m, n, k, times in _table()}
+    regrets, cut = [], 0
+    for (m, n, k), times in table.items():
+        t = _time_of_choice(m, n, k, table)
+        cut += K.gemm_row_split(m, n, k) > 0
+        if t is not None:
+            regrets.append(t / min(times) - 1.0)   # (below zero where two launches beat every single shape)
+    print("%d of %d problems are cut along their rows" % (cut, len(table)))
     regrets = np.array(regrets)
     print("mean %.4f max %.4f over %d problems" % (regrets.mean(), regrets.max(), len(regrets)))
-    assert len(regrets) >= 90
+    assert len(regrets) >= 85
     assert regrets.mean() <= 0.012
     assert regrets.max() <= 0.10
 
@@ -36,6 +52,17 @@ def test_choices_for_the_encoder_layers_at_batch_256():
     assert K.gemm_variant_name(16384, 1024, 1024) == "gemm_dma_256x256x64"   # 256 tiles
     assert K.gemm_variant_name(16384, 1536, 1024) == "gemm_dma_256x192x64"   # 512 tiles
     assert K.gemm_variant_name(16384, 1024, 1536) == "gemm_dma_256x256x64"
+
+
+def test_products_that_leave_a_partial_round_are_cut_along_their_rows():
+    """Whole rounds of large tiles first, the rest on whatever suits it; products that fill their rounds stay whole."""
+    assert K.gemm_row_split(20480, 1024, 1536) == 16384
+    assert K.gemm_variant_name(20480, 1024, 1536) == "gemm_dma_256x256x64+rest"
+    assert K.gemm_row_split(24576, 1024, 1024) == 16384
+    for m, n, k in ((16384, 3072, 1024), (16384, 1024, 1024), (16384, 1536, 1024), (32768, 1024, 1536), (4096, 1024, 1024),
+                    (65536, 3072, 1024)):
+        assert K.gemm_row_split(m, n, k) == 0, (m, n, k)
+    assert K.gemm_row_split(20480, 64, 1024) == 0 and K.gemm_row_split(1 << 20, 1024, 256) == 0   # outside the model
 
 
 def test_small_and_batched_products_keep_their_kernels():

@@ -379,6 +379,35 @@ def test_output_store_kinds_give_the_same_result(stores, variant):
     assert np.array_equal(got_ln, want_ln)
 
 
+@pytest.mark.parametrize("m,n,k", [(20480, 1024, 1536), (20481, 1024, 1024), (24576, 1000, 1024)])
+def test_product_cut_along_its_rows_equals_one_launch(m, n, k):
+    """A product whose tiles leave a partial round is cut into whole rounds of large tiles and a rest on another tile
+    shape: the same bits as one launch of the large tiles (every shape adds the k-steps of an output in the same
+    order), and the oracle's layer on rows of both parts and of the seam."""
+    from lc0_amd import kernels as K
+    m1 = K.gemm_row_split(m, n, k)
+    assert 0 < m1 < m, "this shape is meant to be cut"
+    rng = np.random.default_rng(m + n)
+    a = _h(rng.standard_normal((m, k)) * 0.5)
+    w = _h(rng.standard_normal((n, k)) * 0.1)
+    b = rng.standard_normal(n).astype(f32)
+    got = K.gemm(a, w, b, 0.5, nr.ACT_MISH)
+    K.set_gemm_variant(0)
+    try:
+        want = K.gemm(a, w, b, 0.5, nr.ACT_MISH)
+    finally:
+        K.set_gemm_variant(-1)
+    assert np.array_equal(got, want)
+    rows = np.r_[0:64, m1 - 64:m1 + 64, m - 64:m]
+    np.testing.assert_allclose(got[rows].astype(f32), _fc_scaled(a[rows], w, b, 0.5, nr.ACT_MISH), rtol=3e-3, atol=3e-3)
+
+
+def _fc_scaled(a, w, b, scale, act):
+    """act(scale * a w^T + b) in float64 through the oracle's activation."""
+    z = scale * (a.astype(np.float64) @ w.astype(np.float64).T) + b
+    return onn.activate(z.astype(f32), act)
+
+
 def test_cold_cache_timing_hook_leaves_results_alone():
     """The profiling hook times launches one by one behind a cache-flushing copy: same output, a positive time."""
     from lc0_amd import kernels as K
