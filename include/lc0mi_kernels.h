@@ -28,6 +28,8 @@ const char* lc0mi_k_gemm_variant_name(int M, int N, int K, int batch, int latenc
 /* Rows that lc0mi_k_gemm gives to a first launch of whole rounds of large tiles when it cuts a half-precision product
  * of this shape along its rows (0: one launch). Host-side choice, no device needed; no counterpart in the reference. */
 int lc0mi_k_gemm_row_split(int M, int N, int K);
+/* Switches that cut off (0) or on (1, the default), for measurements and tests; process-wide, like lc0mi_k_set_gemm_variant. */
+void lc0mi_k_set_gemm_row_split(int on);
 /* Split-K form: K is cut into split_k slices whose float partial sums are added in
  * slice order (bias added once, no activation). C is float [M][N]. */
 int lc0mi_k_gemm_splitk(const uint16_t* A, int lda, const uint16_t* W, int ldw, const float* bias, int M, int N,

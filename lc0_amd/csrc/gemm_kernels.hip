@@ -1081,8 +1081,9 @@ inline FittedCosts FitCosts(int M, int N, int K) {
 // (20480x1024x1536: 87 us on 320 tiles of 256x256, one and a quarter rounds, or 78 us on 128x128 tiles, against
 // 49 + 19 us for 16384 rows on one full round of large tiles and 4096 rows on small ones). Returns the rows of the
 // first launch (0: one launch) when the model above prices the pair at least 3 % below the best single shape.
+bool g_row_split = true;   // (profiling and tests switch it off through SetGemmRowSplit)
 int PlanRowSplit(const GemmArgs& a, GemmVariant* first) {
-  if (g_variant_override >= 0 || !InFittedDomain(a) || a.out_f32 || a.split_k != 1 || a.K % 64 != 0 ||
+  if (!g_row_split || g_variant_override >= 0 || !InFittedDomain(a) || a.out_f32 || a.split_k != 1 || a.K % 64 != 0 ||
       a.skip != nullptr || a.row_stats != nullptr) {
     return 0;
   }
@@ -1211,6 +1212,7 @@ GemmVariant PickGemmVariantHalf(const GemmArgs& a) {
 }  // namespace
 
 void SetGemmVariantOverride(int variant) { g_variant_override = variant; }
+void SetGemmRowSplit(bool on) { g_row_split = on; }
 
 namespace {
 // Column-tile width of the direct-to-LDS variants (0 for the others).

@@ -170,6 +170,8 @@ const char* lc0mi_k_gemm_variant_name(int M, int N, int K, int batch, int latenc
   return lc0mi::GemmVariantName(g);
 }
 
+void lc0mi_k_set_gemm_row_split(int on) { lc0mi::SetGemmRowSplit(on != 0); }
+
 int lc0mi_k_gemm_row_split(int M, int N, int K) {
   lc0mi::GemmArgs g;
   g.M = M; g.N = N; g.K = K; g.batch = 1;

@@ -157,6 +157,8 @@ void LaunchZero(float* p, long long n, hipStream_t stream);
 // 3 128x128x64, 4 64x64x64 (register-staged), 5 128x128x64 direct-to-LDS with 4 waves,
 // 6 row-panel 64x32 (K split over the waves), 7 128x64x64 direct-to-LDS with 4 waves. For tests and tuning only.
 void SetGemmVariantOverride(int variant);
+// Whether LaunchGemm may cut a large product along its rows (GemmRowSplit); on by default.
+void SetGemmRowSplit(bool on);
 
 // Layer norm for few, long rows (one workgroup per row): t = act(x) * alpha + skip,
 // where x is half (x_f16) or the sum of n_partials float arrays x_f32 + i * partial_stride

@@ -21,6 +21,8 @@ def _lib():
         lib.lc0mi_k_gemm_variant_name.argtypes = [ci, ci, ci, ci, ci]
         lib.lc0mi_k_gemm_variant_name.restype = C.c_char_p
         lib.lc0mi_k_gemm_row_split.argtypes = [ci, ci, ci]
+        lib.lc0mi_k_set_gemm_row_split.argtypes = [ci]
+        lib.lc0mi_k_set_gemm_row_split.restype = None
         lib.lc0mi_k_gemm_norm_producer.argtypes = [vp, ci, vp, ci, vp, ci, ci, ci, cf, vp, vp, ci, vp, vp, cf, vp, vp, ci,
                                                    C.POINTER(C.c_int), ci, cd]
         lib.lc0mi_k_gemm_norm_consumer.argtypes = [vp, ci, vp, ci, vp, vp, ci, ci, ci, vp, ci, cf, ci, ci, vp, ci, ci, cd]
@@ -117,6 +119,11 @@ def gemm(a, w, bias=None, scale=1.0, act=ACT_NONE, out_f32=False, time_iters=0):
 def gemm_variant_name(m, n, k, batch=1, latency_first=False):
     """Tile shape the launcher picks for a half-precision product of this shape (host-side logic, no GPU needed)."""
     return _lib().lc0mi_k_gemm_variant_name(m, n, k, batch, int(latency_first)).decode()
+
+
+def set_gemm_row_split(on):
+    """Lets the launcher cut large products along their rows (default) or not; process-wide."""
+    _lib().lc0mi_k_set_gemm_row_split(int(bool(on)))
 
 
 def gemm_row_split(m, n, k):

@@ -382,8 +382,10 @@ def test_output_store_kinds_give_the_same_result(stores, variant):
 @pytest.mark.parametrize("m,n,k", [(20480, 1024, 1536), (20481, 1024, 1024), (24576, 1000, 1024)])
 def test_product_cut_along_its_rows_equals_one_launch(m, n, k):
     """A product whose tiles leave a partial round is cut into whole rounds of large tiles and a rest on another tile
-    shape: the same bits as one launch of the large tiles (every shape adds the k-steps of an output in the same
-    order), and the oracle's layer on rows of both parts and of the seam."""
+    shape. The first part carries the bits of one launch of the large tiles; in the rest the float sums of the two
+    shapes differ in the last bit now and then, so that a few outputs per million that sit on a half-precision tie
+    fall the other way: at most one half-precision step, in at most 2e-5 of the outputs. Rows of both parts and of
+    the seam against the oracle's layer."""
     from lc0_amd import kernels as K
     m1 = K.gemm_row_split(m, n, k)
     assert 0 < m1 < m, "this shape is meant to be cut"
@@ -397,7 +399,11 @@ def test_product_cut_along_its_rows_equals_one_launch(m, n, k):
         want = K.gemm(a, w, b, 0.5, nr.ACT_MISH)
     finally:
         K.set_gemm_variant(-1)
-    assert np.array_equal(got, want)
+    assert np.array_equal(got[:m1], want[:m1])
+    differ = got[m1:] != want[m1:]
+    assert differ.mean() <= 2e-5, differ.sum()
+    steps = np.abs(got[m1:].view(np.int16).astype(np.int32) - want[m1:].view(np.int16).astype(np.int32))
+    assert steps.max() <= 1   # neighbouring half values (same sign: a tie near zero does not occur with this bias)
     rows = np.r_[0:64, m1 - 64:m1 + 64, m - 64:m]
     np.testing.assert_allclose(got[rows].astype(f32), _fc_scaled(a[rows], w, b, 0.5, nr.ACT_MISH), rtol=3e-3, atol=3e-3)
 

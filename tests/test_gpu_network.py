@@ -357,9 +357,21 @@ def test_written_through_outputs_change_no_bits(positions):
         _, off = _run_gpu(path, masks[:b], values[:b], (opts + "," if opts else "") + "write_through=false")
         for key in ("policy", "q", "d", "m"):
             assert np.array_equal(on[key], off[key]), (name, opts, b, key)
-        # (rows 320.. repeat rows 0..: the same position gives the same output wherever it stands in the batch)
+        # (rows 320.. repeat rows 0..: the same position gives the same output wherever it stands in the batch, as long
+        #  as all rows go through the same kernels. At this size the launcher cuts some products along their rows and
+        #  runs the two parts on different tile shapes, whose float sums differ in the last bit now and then - a
+        #  handful of half-precision ties per product fall the other way - so the cut is switched off for this check
+        #  and the repeated rows are held to the parity tolerance with it.)
         if b == 384:
-            np.testing.assert_allclose(on["policy"][320:], on["policy"][:64], rtol=0, atol=1e-5)
+            from lc0_amd import kernels as K
+            np.testing.assert_allclose(on["policy"][320:], on["policy"][:64], rtol=0, atol=TOL)
+            K.set_gemm_row_split(False)
+            try:
+                _, whole = _run_gpu(path, masks[:b], values[:b], opts)
+            finally:
+                K.set_gemm_row_split(True)
+            np.testing.assert_allclose(whole["policy"][320:], whole["policy"][:64], rtol=0, atol=1e-5)
+            np.testing.assert_allclose(whole["policy"], on["policy"], rtol=0, atol=TOL)
 
 
 @pytest.mark.timeout(600)
