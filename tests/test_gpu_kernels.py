@@ -382,9 +382,10 @@ def test_output_store_kinds_give_the_same_result(stores, variant):
 @pytest.mark.parametrize("m,n,k", [(20480, 1024, 1536), (20481, 1024, 1024), (24576, 1000, 1024)])
 def test_product_cut_along_its_rows_equals_one_launch(m, n, k):
     """A product whose tiles leave a partial round is cut into whole rounds of large tiles and a rest on another tile
-    shape. The first part carries the bits of one launch of the large tiles; in the rest the float sums of the two
-    shapes differ in the last bit now and then, so that a few outputs per million that sit on a half-precision tie
-    fall the other way: at most one half-precision step, in at most 2e-5 of the outputs. Rows of both parts and of
+    shape. The first part carries the bits of one launch of the large tiles; in the rest a few outputs per million
+    that sit on a half-precision tie fall the other way (the compiler rounds scale * acc + bias once, straight to
+    half, in some places of one kernel instance and twice, through float, in another): at most one half-precision
+    step, in at most 2e-5 of the outputs. Rows of both parts and of
     the seam against the oracle's layer."""
     from lc0_amd import kernels as K
     m1 = K.gemm_row_split(m, n, k)

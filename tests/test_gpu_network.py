@@ -359,8 +359,8 @@ def test_written_through_outputs_change_no_bits(positions):
             assert np.array_equal(on[key], off[key]), (name, opts, b, key)
         # (rows 320.. repeat rows 0..: the same position gives the same output wherever it stands in the batch, as long
         #  as all rows go through the same kernels. At this size the launcher cuts some products along their rows and
-        #  runs the two parts on different tile shapes, whose float sums differ in the last bit now and then - a
-        #  handful of half-precision ties per product fall the other way - so the cut is switched off for this check
+        #  runs the two parts on different tile shapes, between which a handful of half-precision ties per product
+        #  fall the other way (one rounding against two in the epilogue) - so the cut is switched off for this check
         #  and the repeated rows are held to the parity tolerance with it.)
         if b == 384:
             from lc0_amd import kernels as K
